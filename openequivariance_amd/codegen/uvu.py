@@ -1,0 +1,911 @@
+"""Generator of gfx950 HIP source for channel-wise ("uvu") tensor products.
+
+One generator serves three operator families that share the per-row arithmetic:
+
+* ``tp``          - batch tensor product (forward; backward -> dX, dY, dW)
+* ``conv_atomic`` - fused gather/product/scatter over unsorted edges, scatter by atomics
+* ``conv_det``    - deterministic fused convolution over receiver-sorted edges: one
+                    wavefront owns a node (and a 64-channel chunk) and walks its edge list,
+                    so sums are formed in a fixed order without atomics
+
+Mapping to the hardware (the arithmetic follows the reference's kernels,
+openequivariance/templates/loop_unroll_tp.cuh:20-97 forward and :107-252 backward, but the
+schedule is new):
+
+* a workgroup is ONE 64-lane wavefront; ``__syncthreads`` therefore costs a wait, not a barrier;
+* lane <-> multiplicity channel ``u``.  Multiplicities above 64 are walked in chunks of 64;
+  multiplicities of at most 32 pack ``R = 64 / P`` rows (edges) into one wavefront,
+  ``P`` = the multiplicity rounded up to a power of two;
+* global memory is always touched in contiguous runs: rows of X / dZ are copied to LDS with
+  consecutive lanes reading consecutive words and are then read back transposed
+  (lane ``u`` reads words ``u*(2l+1)+m``; the stride is odd, hence conflict free); Z / dX take the
+  opposite route.  Blocks with l = 0 need no transposition and go straight to registers;
+* the Clebsch-Gordan coefficients, multiplied by the path normalisation, are emitted as exact
+  hexadecimal literals in fully unrolled fused multiply-adds; zero coefficients emit nothing;
+* Y (<= 16 words per row) is loaded once per row; with one row per wavefront its address is
+  wave-uniform, which lets the compiler keep it in scalar registers.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Tuple
+
+import numpy as np
+
+from ..problem import TPProblem
+from ..wigner import wigner_3j
+from .common import WAVE, Emitter, jinja_env, literal, next_pow2
+
+MAX_UNROLLED_V = 8
+
+
+@dataclass
+class Block:
+    idx: int
+    mul: int
+    l: int
+    off: int
+
+    @property
+    def D(self) -> int:
+        return 2 * self.l + 1
+
+    @property
+    def dim(self) -> int:
+        return self.mul * self.D
+
+
+@dataclass
+class Path:
+    t: int
+    a: Block
+    b: Block
+    o: Block
+    coeff: float
+    woff: int
+    pairs: Dict[Tuple[int, int], List[Tuple[int, float]]] = field(default_factory=dict)
+
+    @property
+    def mu(self) -> int:
+        return self.a.mul
+
+    @property
+    def mv(self) -> int:
+        return self.b.mul
+
+    @property
+    def nnz(self) -> int:
+        return sum(len(v) for v in self.pairs.values())
+
+    def ordered_pairs(self):
+        """(i, j) pairs sorted by j then i (the reference sorts its nonzeros by (j, i, k):
+        openequivariance/implementations/ComputationSchedule.py:52-66)."""
+        return sorted(self.pairs.items(), key=lambda kv: (kv[0][1], kv[0][0]))
+
+
+def _blocks(irreps) -> List[Block]:
+    out, off = [], 0
+    for i, mi in enumerate(irreps):
+        out.append(Block(i, mi.mul, mi.ir.l, off))
+        off += mi.dim
+    return out
+
+
+class UVUGenerator:
+    """Builds the source text and the launch plan for one uvu problem."""
+
+    def __init__(self, problem: TPProblem, kind: str = "tp", dw_partials: int = 1024):
+        if kind not in ("tp", "conv_atomic", "conv_det"):
+            raise ValueError(kind)
+        self.problem, self.kind = problem, kind
+        self.T = {np.float32: "float", np.float64: "double"}[problem.irrep_dtype]
+        self.itemsize = 4 if self.T == "float" else 8
+        self.shared = bool(problem.shared_weights)
+        self.in1 = _blocks(problem.irreps_in1)
+        self.in2 = _blocks(problem.irreps_in2)
+        self.out = _blocks(problem.irreps_out)
+        self.D1, self.D2, self.D3 = problem.irreps_in1.dim, problem.irreps_in2.dim, problem.irreps_out.dim
+        self.WN = problem.weight_numel
+
+        self.paths: List[Path] = []
+        woff = 0
+        for t, ins in enumerate(problem.instructions):
+            if ins.connection_mode != "uvu":
+                raise ValueError("UVUGenerator handles uvu instructions only")
+            if not ins.has_weight:
+                raise NotImplementedError("instructions without weights are not supported")
+            a, b, o = self.in1[ins.i_in1], self.in2[ins.i_in2], self.out[ins.i_out]
+            if a.mul != o.mul:
+                raise ValueError(f"uvu instruction {t}: mul(in1)={a.mul} must equal mul(out)={o.mul}")
+            if b.mul > MAX_UNROLLED_V:
+                raise NotImplementedError(f"uvu with mul(in2) = {b.mul} > {MAX_UNROLLED_V} is not supported yet")
+            c = wigner_3j(a.l, b.l, o.l) * ins.path_weight
+            p = Path(t, a, b, o, ins.path_weight, woff)
+            for i, j, k in np.argwhere(np.abs(c) > 1e-14):
+                p.pairs.setdefault((int(i), int(j)), []).append((int(k), float(c[i, j, k])))
+            self.paths.append(p)
+            woff += a.mul * b.mul
+        if not self.paths:
+            raise ValueError("Tensor product problem has no valid instructions!")
+        if kind != "tp":
+            if self.shared:
+                raise NotImplementedError("fused convolution requires per-edge weights (shared_weights=False)")
+            for b in self.in2:
+                if b.mul != 1:
+                    raise AssertionError("fused convolution requires multiplicity 1 for every irrep of in2")
+
+        self.used_in1 = sorted({p.a.idx for p in self.paths})
+        self.used_out = sorted({p.o.idx for p in self.paths})
+        self.used_y = sorted({p.b.off + v * p.b.D + j for p in self.paths for v in range(p.mv) for (_, j) in p.pairs})
+
+        max_mul = max(self.in1[i].mul for i in self.used_in1)
+        if max_mul <= 32:
+            self.P = next_pow2(max_mul)
+            self.R = WAVE // self.P
+            self.NCH = 1
+        else:
+            self.P, self.R = WAVE, 1
+            self.NCH = (max_mul + WAVE - 1) // WAVE
+        self.LOGP = self.P.bit_length() - 1
+        # the deterministic convolution spreads chunks over blockIdx.y and stages one chunk of X
+        self.chunk_in_grid = (kind == "conv_det")
+        self.x_chunk_layout = self.chunk_in_grid and self.NCH > 1
+        self.unroll_chunks = (self.NCH <= 2 or self.shared) and not self.chunk_in_grid
+        self.dw_partials = dw_partials if self.shared else 0
+
+        # ---- LDS map (in elements of T) --------------------------------------
+        self.xl: Dict[int, int] = {}
+        if self.x_chunk_layout:
+            pos = 0
+            for i in self.used_in1:
+                self.xl[i] = pos
+                pos += WAVE * self.in1[i].D
+            self.x_lds = pos
+        else:
+            self.x_lds = self.R * self.D1
+        stage = [WAVE * self.out[i].D for i in self.used_out if self.out[i].D > 1]
+        stage += [WAVE * b.D for b in self.in1 if b.D > 1]
+        self.ZB = self.x_lds
+        self.stage_lds = max(stage) if stage else 0
+        self.lds_elems = max(1, self.x_lds + self.stage_lds)
+
+    # ------------------------------------------------------------------ helpers
+    def lit(self, v: float) -> str:
+        return literal(v, self.T)
+
+    def widx(self, p: Path, u: str, v: int) -> str:
+        """oeq-order position of weight (u, v) of path ``p`` (see weight_order.py)."""
+        mu, mv = p.mu, p.mv
+        if mv == 1:
+            return f"{p.woff} + {u}"
+        if mu <= 32 and mv <= 32:
+            return f"{p.woff + v * mu} + {u}"
+        ulw = "32" if mu % 32 == 0 else f"min(32, {mu} - (({u}) >> 5) * 32)"
+        vc, vl = divmod(v, 32)
+        return f"{p.woff} + (({u}) >> 5) * {32 * mv} + {ulw} * {32 * vc + vl} + (({u}) & 31)"
+
+    def full(self, blk: Block) -> bool:
+        """True when every lane of every chunk maps to a valid channel of ``blk``."""
+        return blk.mul == self.P * self.NCH
+
+    def act(self, blk: Block) -> str:
+        return "rv" if self.full(blk) else f"(rv && u < {blk.mul})"
+
+    def paths_into(self, o_idx: int) -> List[Path]:
+        return [p for p in self.paths if p.o.idx == o_idx]
+
+    def chunk_count(self, blk: Block) -> str:
+        """Number of valid channels of ``blk`` in chunk ``c`` (C expression)."""
+        if self.full(blk):
+            return f"{self.P}"
+        if self.NCH == 1:
+            return f"{blk.mul}"
+        return f"max(0, min({self.P}, {blk.mul} - c * {self.P}))"
+
+    # ---------------------------------------------------------------- prologue
+    def emit_lane(self, E: Emitter) -> None:
+        E("const int lane = threadIdx.x;")
+        E(f"const int sub = lane >> {self.LOGP};")
+        E(f"const int ul = lane & {self.P - 1};")
+        E(f"__shared__ T lds[{self.lds_elems}];")
+
+    def emit_y_load(self, E: Emitter, ptr: str, valid: str) -> None:
+        for f in self.used_y:
+            E(f"const T y{f} = {valid} ? {ptr}[{f}] : (T)0;")
+
+    # ------------------------------------------------------------- X staging
+    def emit_x_stage(self, E: Emitter) -> None:
+        """Copy the X rows (or the X chunk) of this tile into LDS.
+
+        Row sources: ``tp`` -> rows row0 .. row0+R-1 (contiguous in memory);
+        convolution -> row ``xsrc`` of each sub-row (int, -1 when the sub-row is idle;
+        ``xsrc_u`` is its wave-uniform copy when R == 1)."""
+        D1, R = self.D1, self.R
+        if self.x_chunk_layout:
+            E("if (xsrc_u >= 0) {")
+            for i in self.used_in1:
+                a = self.in1[i]
+                E(f"    {{ const T* __restrict__ src = X + (u64)xsrc_u * {D1} + {a.off} + c * {self.P * a.D};")
+                E(f"      const int len = {self.chunk_count(a)} * {a.D};")
+                E(f"      #pragma unroll")
+                E(f"      for (int it = 0; it < {a.D}; ++it) {{ const int q = lane + it * 64; if (q < len) lds[{self.xl[i]} + q] = src[q]; }} }}")
+            E("}")
+            return
+        total = R * D1
+        iters = (total + WAVE - 1) // WAVE
+        if self.kind == "tp":
+            E("{")
+            E(f"    const u64 left = n - row0;")
+            E(f"    const int avail = (int)(left < {R} ? left : {R}) * {D1};")
+            E(f"    const T* __restrict__ src = X + row0 * {D1};")
+            E(f"    #pragma unroll")
+            E(f"    for (int it = 0; it < {iters}; ++it) {{ const int q = lane + it * 64; if (q < avail) lds[q] = src[q]; }}")
+            E("}")
+        elif R == 1:
+            E("if (xsrc_u >= 0) {")
+            E(f"    const T* __restrict__ src = X + (u64)xsrc_u * {D1};")
+            E(f"    #pragma unroll")
+            E(f"    for (int it = 0; it < {iters}; ++it) {{ const int q = lane + it * 64; if (q < {D1}) lds[q] = src[q]; }}")
+            E("}")
+        else:
+            E(f"#pragma unroll")
+            E(f"for (int it = 0; it < {iters}; ++it) {{")
+            E(f"    const int q = lane + it * 64;")
+            E(f"    const int r = q / {D1};")
+            E(f"    const int s = oeq_shfl_i32(xsrc, (r < {R} ? r : 0) << {self.LOGP});")
+            E(f"    if (q < {total} && s >= 0) lds[q] = X[(u64)s * {D1} + (q - r * {D1})];")
+            E("}")
+
+    def emit_x_regs(self, E: Emitter) -> None:
+        for i in self.used_in1:
+            a = self.in1[i]
+            for m in range(a.D):
+                if self.x_chunk_layout:
+                    addr = f"{self.xl[i]} + ul * {a.D} + {m}"
+                else:
+                    addr = f"sub * {self.D1} + {a.off} + u * {a.D} + {m}"
+                E(f"const T x{i}_{m} = {self.act(a)} ? lds[{addr}] : (T)0;")
+
+    def emit_weights(self, E: Emitter, p: Path, wptr: str) -> None:
+        for v in range(p.mv):
+            E(f"const T w{p.t}_{v} = {self.act(p.a)} ? {wptr}[{self.widx(p, 'u', v)}] : (T)0;")
+
+    # --------------------------------------------------------- forward arithmetic
+    def emit_forward_block(self, E: Emitter, o: Block, wptr: str, zname: str = "z", declare: bool = True) -> None:
+        """z_k (+)= sum over paths into ``o``: w * sum_ij c_ijk x_i y_j."""
+        if declare:
+            for k in range(o.D):
+                E(f"T {zname}{k} = (T)0;")
+        for p in self.paths_into(o.idx):
+            E(f"{{ // path {p.t}: l = {p.a.l} x {p.b.l} -> {p.o.l}, coefficient {p.coeff:.9g}")
+            self.emit_weights(E, p, wptr)
+            for v in range(p.mv):
+                body, seen = [], []
+                for (i, j), ks in p.ordered_pairs():
+                    yv = f"y{p.b.off + v * p.b.D + j}"
+                    body.append(f"{{ const T t = x{p.a.idx}_{i} * {yv};")
+                    for k, val in ks:
+                        if k in seen:
+                            body.append(f"  p{k} = oeq_fma({self.lit(val)}, t, p{k});")
+                        else:
+                            body.append(f"  p{k} = {self.lit(val)} * t;")
+                            seen.append(k)
+                    body.append("}")
+                E("{ T " + ", ".join(f"p{k}" for k in sorted(seen)) + ";")
+                E.extend("  " + b for b in body)
+                for k in sorted(seen):
+                    E(f"  {zname}{k} = oeq_fma(w{p.t}_{v}, p{k}, {zname}{k});")
+                E("}")
+            E("}")
+
+    # -------------------------------------------------------- backward arithmetic
+    def emit_backward_block(self, E: Emitter, o: Block, wptr: str, dw_sink) -> None:
+        """Given g_k = dZ[o][u, k] (registers g0..), update dx{a}_{i}, dy{f} and hand every
+        dW value to ``dw_sink(E, path, v, expr)``.  Formulas: loop_unroll_tp.cuh:167-174 of the
+        reference, regrouped per (i, j) pair: s = sum_k c_ijk g_k."""
+        for p in self.paths_into(o.idx):
+            E(f"{{ // path {p.t}: l = {p.a.l} x {p.b.l} -> {p.o.l}")
+            self.emit_weights(E, p, wptr)
+            for v in range(p.mv):
+                ya = lambda j: f"y{p.b.off + v * p.b.D + j}"
+                E(f"{{ T dw = (T)0;")
+                js = sorted({j for (_, j) in p.pairs})
+                is_ = sorted({i for (i, _) in p.pairs})
+                for j in js:
+                    E(f"  const T wy{j} = w{p.t}_{v} * {ya(j)};")
+                for i in is_:
+                    E(f"  const T wx{i} = w{p.t}_{v} * x{p.a.idx}_{i};")
+                for (i, j), ks in p.ordered_pairs():
+                    E("  {")
+                    for n_, (k, val) in enumerate(ks):
+                        if n_ == 0:
+                            E(f"    T s = {self.lit(val)} * g{k};")
+                        else:
+                            E(f"    s = oeq_fma({self.lit(val)}, g{k}, s);")
+                    E(f"    dw = oeq_fma(s, x{p.a.idx}_{i} * {ya(j)}, dw);")
+                    E(f"    dx{p.a.idx}_{i} = oeq_fma(s, wy{j}, dx{p.a.idx}_{i});")
+                    E(f"    dy{p.b.off + v * p.b.D + j} = oeq_fma(s, wx{i}, dy{p.b.off + v * p.b.D + j});")
+                    E("  }")
+                dw_sink(E, p, v, "dw")
+                E("}")
+            E("}")
+
+    # --------------------------------------------------------------- LDS slots
+    def emit_slot_write(self, E: Emitter, blk: Block, name: str, act: str) -> None:
+        """registers name0.. -> lds[ZB + lane*D + k]."""
+        E("oeq_sync();")
+        E(f"if ({act}) {{ " + " ".join(f"lds[{self.ZB} + lane * {blk.D} + {k}] = {name}{k};" for k in range(blk.D)) + " }")
+        E("oeq_sync();")
+
+    def emit_slot_read(self, E: Emitter, blk: Block, name: str, act: str) -> None:
+        for k in range(blk.D):
+            E(f"const T {name}{k} = {act} ? lds[{self.ZB} + lane * {blk.D} + {k}] : (T)0;")
+
+    def emit_slot_to_global(self, E: Emitter, blk: Block, ptr: str, rowdim: int, row_of, op: str = "store",
+                            zero: bool = False) -> None:
+        """Copy the slot of block ``blk`` (chunk c) from LDS to rows of ``ptr`` (row length
+        ``rowdim``).  ``row_of(r)`` -> (row expression, validity expression) for sub-row r;
+        op is "store" or "atomic".  With ``zero`` the slot is not read: zeros are stored."""
+        D, P, R = blk.D, self.P, self.R
+        val = lambda e: "(T)0" if zero else e
+
+        def put(dst: str, v: str) -> str:
+            return f"oeq_atomic_add(&{dst}, {v});" if op == "atomic" else f"{dst} = {v};"
+        if R == 1:
+            row, ok = row_of("0")
+            cnt = self.chunk_count(blk)
+            E(f"if ({ok}) {{")
+            E(f"    T* __restrict__ dst = {ptr} + (u64){row} * {rowdim} + {blk.off} + c * {P * D};")
+            E(f"    const int len = {cnt} * {D};")
+            E(f"    #pragma unroll")
+            E(f"    for (int it = 0; it < {D}; ++it) {{ const int q = lane + it * 64; if (q < len) {{ {put('dst[q]', val(f'lds[{self.ZB} + q]'))} }} }}")
+            E("}")
+        else:
+            L = blk.mul * D                      # NCH == 1 here
+            total = R * L
+            iters = (total + WAVE - 1) // WAVE
+            row, ok = row_of("rr")
+            E(f"#pragma unroll")
+            E(f"for (int it = 0; it < {iters}; ++it) {{")
+            E(f"    const int q = lane + it * 64;")
+            E(f"    const int r = q / {L};")
+            E(f"    const int rr = r < {R} ? r : 0;")
+            E(f"    const int qq = q - r * {L};")
+            E(f"    const i64 grow = (i64){row};")
+            E(f"    const bool ok = {ok};")
+            E(f"    if (q < {total} && ok) {{ {put(f'{ptr}[(u64)grow * {rowdim} + {blk.off} + qq]', val(f'lds[{self.ZB} + rr * {P * D} + qq]'))} }}")
+            E("}")
+
+    def emit_global_to_slot(self, E: Emitter, blk: Block, ptr: str, rowdim: int, row_of) -> None:
+        """Inverse of emit_slot_to_global (plain loads)."""
+        D, P, R = blk.D, self.P, self.R
+        E("oeq_sync();")
+        if R == 1:
+            row, ok = row_of("0")
+            cnt = self.chunk_count(blk)
+            E(f"if ({ok}) {{")
+            E(f"    const T* __restrict__ src = {ptr} + (u64){row} * {rowdim} + {blk.off} + c * {P * D};")
+            E(f"    const int len = {cnt} * {D};")
+            E(f"    #pragma unroll")
+            E(f"    for (int it = 0; it < {D}; ++it) {{ const int q = lane + it * 64; if (q < len) lds[{self.ZB} + q] = src[q]; }}")
+            E("}")
+        else:
+            L = blk.mul * D
+            total = R * L
+            iters = (total + WAVE - 1) // WAVE
+            row, ok = row_of("rr")
+            E(f"#pragma unroll")
+            E(f"for (int it = 0; it < {iters}; ++it) {{")
+            E(f"    const int q = lane + it * 64;")
+            E(f"    const int r = q / {L};")
+            E(f"    const int rr = r < {R} ? r : 0;")
+            E(f"    const int qq = q - r * {L};")
+            E(f"    const i64 grow = (i64){row};")
+            E(f"    const bool ok = {ok};")
+            E(f"    if (q < {total} && ok) lds[{self.ZB} + rr * {P * D} + qq] = {ptr}[(u64)grow * {rowdim} + {blk.off} + qq];")
+            E("}")
+        E("oeq_sync();")
+
+    # block output: registers -> global, choosing the direct path for l = 0
+    def emit_block_out(self, E: Emitter, blk: Block, name: str, ptr: str, rowdim: int, own_row: Tuple[str, str],
+                       row_of, op: str = "store") -> None:
+        act = self.act(blk)
+        if blk.D == 1:
+            row, ok = own_row
+            dst = f"{ptr}[(u64){row} * {rowdim} + {blk.off} + u]"
+            stmt = f"oeq_atomic_add(&{dst}, {name}0);" if op == "atomic" else f"{dst} = {name}0;"
+            E(f"if ({act} && {ok}) {{ {stmt} }}")
+        else:
+            self.emit_slot_write(E, blk, name, act)
+            self.emit_slot_to_global(E, blk, ptr, rowdim, row_of, op)
+
+    def emit_block_in(self, E: Emitter, blk: Block, name: str, ptr: str, rowdim: int, own_row: Tuple[str, str],
+                      row_of) -> None:
+        act = self.act(blk)
+        if blk.D == 1:
+            row, ok = own_row
+            E(f"const T {name}0 = ({act} && {ok}) ? {ptr}[(u64){row} * {rowdim} + {blk.off} + u] : (T)0;")
+        else:
+            self.emit_global_to_slot(E, blk, ptr, rowdim, row_of)
+            self.emit_slot_read(E, blk, name, act)
+
+    def emit_block_zero(self, E: Emitter, blk: Block, ptr: str, rowdim: int, own_row, row_of) -> None:
+        """Store zeros over chunk c of a block nothing contributes to."""
+        if blk.D == 1:
+            row, ok = own_row
+            E(f"if ({self.act(blk)} && {ok}) {ptr}[(u64){row} * {rowdim} + {blk.off} + u] = (T)0;")
+        else:
+            self.emit_slot_to_global(E, blk, ptr, rowdim, row_of, zero=True)
+
+    # ------------------------------------------------------------- dY reduction
+    def emit_dy_reduce(self, E: Emitter) -> None:
+        """Butterfly sum of dy* over the P lanes of each sub-row (fixed order -> deterministic)."""
+        m = self.P // 2
+        while m >= 1:
+            for f in self.used_y:
+                E(f"dy{f} += oeq_shfl_xor(dy{f}, {m});")
+            m //= 2
+
+    # ------------------------------------------------------------ chunk loops
+    def chunk_loop(self, E: Emitter, body) -> None:
+        """Run ``body(E)`` once per chunk with ``c`` and ``u`` defined."""
+        if self.chunk_in_grid:
+            E("{")
+            E.level += 1
+            E("const int c = blockIdx.y;")
+            E(f"const int u = c * {self.P} + ul;")
+            body(E)
+            E.level -= 1
+            E("}")
+        elif self.NCH == 1:
+            E("{")
+            E.level += 1
+            E("const int c = 0;")
+            E("const int u = ul;")
+            body(E)
+            E.level -= 1
+            E("}")
+        else:
+            E("#pragma unroll" if self.unroll_chunks else "#pragma unroll 1")
+            E(f"for (int c = 0; c < {self.NCH}; ++c) {{")
+            E.level += 1
+            E(f"const int u = c * {self.P} + ul;")
+            body(E)
+            E.level -= 1
+            E("}")
+
+    # =================================================================== batch TP
+    def tp_forward_body(self) -> str:
+        E = Emitter()
+        self.emit_lane(E)
+        R = self.R
+        ntiles = f"(n + {R - 1}) / {R}"
+        E(f"for (u64 tile = blockIdx.x; tile < {ntiles}; tile += gridDim.x) {{")
+        E.level += 1
+        E(f"const u64 row0 = tile * {R};")
+        E("const u64 row = row0 + sub;")
+        E("const bool rv = row < n;")
+        E(f"const T* __restrict__ Yr = Y + row * {self.D2};")
+        E("const T* __restrict__ Wr = W" + ("" if self.shared else f" + row * {self.WN}") + ";")
+        self.emit_y_load(E, "Yr", "rv")
+        E("oeq_sync();")
+        self.emit_x_stage(E)
+        E("oeq_sync();")
+        own = ("row", "rv")
+        row_of = lambda r: (f"(row0 + {r})", f"(row0 + {r} < n)")
+
+        def body(E):
+            self.emit_x_regs(E)
+            for o in self.out:
+                E("{")
+                E.level += 1
+                if o.idx in self.used_out:
+                    self.emit_forward_block(E, o, "Wr")
+                    self.emit_block_out(E, o, "z", "Z", self.D3, own, row_of)
+                elif o.dim > 0:
+                    if o.D > 1:
+                        E("oeq_sync();")
+                    self.emit_block_zero(E, o, "Z", self.D3, own, row_of)
+                E.level -= 1
+                E("}")
+        self.chunk_loop(E, body)
+        E.level -= 1
+        E("}")
+        return E.text()
+
+    def tp_backward_body(self) -> str:
+        E = Emitter()
+        self.emit_lane(E)
+        R = self.R
+        ntiles = f"(n + {R - 1}) / {R}"
+        if self.shared:
+            # per-workgroup dW partial sums live in registers across the tile loop
+            for p in self.paths:
+                for c in range(self.NCH):
+                    for v in range(p.mv):
+                        E(f"T dws{p.t}_{c}_{v} = (T)0;")
+        E(f"for (u64 tile = blockIdx.x; tile < {ntiles}; tile += gridDim.x) {{")
+        E.level += 1
+        E(f"const u64 row0 = tile * {R};")
+        E("const u64 row = row0 + sub;")
+        E("const bool rv = row < n;")
+        E(f"const T* __restrict__ Yr = Y + row * {self.D2};")
+        E("const T* __restrict__ Wr = W" + ("" if self.shared else f" + row * {self.WN}") + ";")
+        if not self.shared:
+            E(f"T* __restrict__ Wgr = Wg + row * {self.WN};")
+        self.emit_y_load(E, "Yr", "rv")
+        for f in self.used_y:
+            E(f"T dy{f} = (T)0;")
+        E("oeq_sync();")
+        self.emit_x_stage(E)
+        E("oeq_sync();")
+        own = ("row", "rv")
+        row_of = lambda r: (f"(row0 + {r})", f"(row0 + {r} < n)")
+
+        def body(E, cconst=None):
+            self.emit_x_regs(E)
+            for i in self.used_in1:
+                for m in range(self.in1[i].D):
+                    E(f"T dx{i}_{m} = (T)0;")
+            for oi in self.used_out:
+                o = self.out[oi]
+                E("{")
+                E.level += 1
+                self.emit_block_in(E, o, "g", "G", self.D3, own, row_of)
+
+                def sink(E, p, v, expr):
+                    if self.shared:
+                        if self.NCH == 1:
+                            E(f"  dws{p.t}_0_{v} += {expr};")
+                        else:
+                            for c in range(self.NCH):
+                                E(f"  if (c == {c}) dws{p.t}_{c}_{v} += {expr};")
+                    else:
+                        E(f"  if ({self.act(p.a)}) Wgr[{self.widx(p, 'u', v)}] = {expr};")
+                self.emit_backward_block(E, o, "Wr", sink)
+                E.level -= 1
+                E("}")
+            for a in self.in1:
+                if a.dim == 0:
+                    continue
+                E("{")
+                E.level += 1
+                if a.idx in self.used_in1:
+                    self.emit_block_out(E, a, f"dx{a.idx}_", "Xg", self.D1, own, row_of)
+                else:
+                    if a.D > 1:
+                        E("oeq_sync();")
+                    self.emit_block_zero(E, a, "Xg", self.D1, own, row_of)
+                E.level -= 1
+                E("}")
+        self.chunk_loop(E, body)
+        # dY: reduce over the lanes of the row, lane 0 of each sub-row stores
+        self.emit_dy_reduce(E)
+        E("if (rv && ul == 0) {")
+        E(f"    T* __restrict__ Ygr = Yg + row * {self.D2};")
+        for f in range(self.D2):
+            E(f"    Ygr[{f}] = " + (f"dy{f};" if f in self.used_y else "(T)0;"))
+        E("}")
+        E.level -= 1
+        E("}")
+        if self.shared:
+            E(f"T* __restrict__ part = (T*)ws + (u64)blockIdx.x * {self.WN};")
+            for p in self.paths:
+                for c in range(self.NCH):
+                    for v in range(p.mv):
+                        E(f"{{ const int u = {c * self.P} + ul;")
+                        # rows of the same wavefront (R > 1) hold separate partial sums: fold them
+                        m = 32
+                        while m >= self.P:
+                            E(f"  dws{p.t}_{c}_{v} += oeq_shfl_xor(dws{p.t}_{c}_{v}, {m});")
+                            m //= 2
+                        E(f"  if (sub == 0 && u < {p.mu}) part[{self.widx(p, 'u', v)}] = dws{p.t}_{c}_{v}; }}")
+        return E.text()
+
+    # =========================================================== atomic convolution
+    def _edge_prologue(self, E: Emitter, need_recv_rows: bool = True) -> None:
+        """Edge-parallel kernels: sub-row r handles edge e0 + r."""
+        R = self.R
+        E(f"const u64 e0 = (u64)blockIdx.x * {R};")
+        E("const u64 e = e0 + sub;")
+        E("i64 snd = -1, rcv = -1;")
+        E("if (e < nnz) { snd = cols[e]; rcv = rows[e]; }")
+        E("const bool rv = (snd >= 0 && snd < (i64)node_count && rcv >= 0 && rcv < (i64)node_count);")
+        E("const int xsrc = rv ? (int)snd : -1;")
+        E("const int zdst = rv ? (int)rcv : -1;")
+        if R == 1:
+            E("const int xsrc_u = __builtin_amdgcn_readfirstlane(xsrc);")
+            E("const int zdst_u = __builtin_amdgcn_readfirstlane(zdst);")
+        E(f"const T* __restrict__ Yr = Y + e * {self.D2};")
+        E(f"const T* __restrict__ Wr = W + e * {self.WN};")
+
+    def _shfl_row(self, var: str):
+        if self.R == 1:
+            return lambda r: (f"{var}_u", f"({var}_u >= 0)")
+        return lambda r: (f"oeq_shfl_i32({var}, ({r}) << {self.LOGP})", f"(oeq_shfl_i32({var}, ({r}) << {self.LOGP}) >= 0)")
+
+    def conv_atomic_forward_body(self) -> str:
+        E = Emitter()
+        self.emit_lane(E)
+        self._edge_prologue(E)
+        self.emit_y_load(E, "Yr", "rv")
+        self.emit_x_stage(E)
+        E("oeq_sync();")
+        own = ("zdst", "rv")
+        row_of = self._shfl_row("zdst")
+
+        def body(E):
+            self.emit_x_regs(E)
+            for oi in self.used_out:
+                o = self.out[oi]
+                E("{")
+                E.level += 1
+                self.emit_forward_block(E, o, "Wr")
+                self.emit_block_out(E, o, "z", "Z", self.D3, own, row_of, op="atomic")
+                E.level -= 1
+                E("}")
+        self.chunk_loop(E, body)
+        return E.text()
+
+    def conv_atomic_backward_body(self) -> str:
+        E = Emitter()
+        self.emit_lane(E)
+        self._edge_prologue(E)
+        E(f"T* __restrict__ Wgr = Wg + e * {self.WN};")
+        self.emit_y_load(E, "Yr", "rv")
+        for f in self.used_y:
+            E(f"T dy{f} = (T)0;")
+        self.emit_x_stage(E)
+        E("oeq_sync();")
+        own_z = ("zdst", "rv")
+        own_x = ("xsrc", "rv")
+        zrow_of = self._shfl_row("zdst")
+        xrow_of = self._shfl_row("xsrc")
+
+        def body(E):
+            self.emit_x_regs(E)
+            for i in self.used_in1:
+                for m in range(self.in1[i].D):
+                    E(f"T dx{i}_{m} = (T)0;")
+            for oi in self.used_out:
+                o = self.out[oi]
+                E("{")
+                E.level += 1
+                self.emit_block_in(E, o, "g", "G", self.D3, own_z, zrow_of)
+
+                def sink(E, p, v, expr):
+                    E(f"  if ({self.act(p.a)}) Wgr[{self.widx(p, 'u', v)}] = {expr};")
+                self.emit_backward_block(E, o, "Wr", sink)
+                E.level -= 1
+                E("}")
+            for i in self.used_in1:
+                a = self.in1[i]
+                E("{")
+                E.level += 1
+                self.emit_block_out(E, a, f"dx{a.idx}_", "Xg", self.D1, own_x, xrow_of, op="atomic")
+                E.level -= 1
+                E("}")
+        self.chunk_loop(E, body)
+        self.emit_dy_reduce(E)
+        E("if (e < nnz && ul == 0) {")
+        E(f"    T* __restrict__ Ygr = Yg + e * {self.D2};")
+        for f in range(self.D2):
+            E(f"    Ygr[{f}] = " + (f"dy{f};" if f in self.used_y else "(T)0;"))
+        E("}")
+        # weights of idle lanes / invalid edges: dW rows must still be defined
+        E("if (e < nnz && !rv) {")
+        E(f"    for (int q = ul; q < {self.WN}; q += {self.P}) Wgr[q] = (T)0;")
+        E("}")
+        return E.text()
+
+    # ==================================================== deterministic convolution
+    def _node_prologue(self, E: Emitter, ptr_name: str) -> None:
+        """Node-parallel kernels: sub-row r owns node node0 + r and the edge positions
+        [ptr[node], ptr[node+1]) of the sorted edge list."""
+        R = self.R
+        E(f"const u64 node0 = (u64)blockIdx.x * {R};")
+        E("const u64 node = node0 + sub;")
+        E("const bool nv = node < node_count;")
+        E(f"const i64* __restrict__ ptr = (const i64*)ws + {ptr_name};")
+        E("i64 beg = 0, end = 0;")
+        E("if (nv && nnz > 0) { beg = ptr[node]; end = ptr[node + 1]; }")
+        E("if (beg < 0) beg = 0;")
+        E("if (end > (i64)nnz) end = (i64)nnz;")
+        E("if (end < beg) end = beg;")
+        E("int len = (int)(end - beg);")
+        E("int maxlen = len;")
+        m = 32
+        while m >= self.P:
+            E(f"maxlen = max(maxlen, oeq_shfl_xor_i32(maxlen, {m}));")
+            m //= 2
+        if R == 1:
+            E("maxlen = __builtin_amdgcn_readfirstlane(maxlen);")
+
+    def conv_det_forward_body(self) -> str:
+        """Z[node] = sum over the node's incoming edges, in edge order."""
+        E = Emitter()
+        self.emit_lane(E)
+        self._node_prologue(E, "0")
+        own_z = ("node", "nv")
+        zrow_of = lambda r: (f"(node0 + {r})", f"(node0 + {r} < node_count)")
+
+        def body(E):
+            for oi in self.used_out:
+                for k in range(self.out[oi].D):
+                    E(f"T z{oi}_{k} = (T)0;")
+            E("for (int it = 0; it < maxlen; ++it) {")
+            E.level += 1
+            E("const bool ev = it < len;")
+            E("const u64 e = (u64)(beg + it);")
+            E("i64 snd = -1;")
+            E("if (ev) snd = cols[e];")
+            E("const bool rv = ev && snd >= 0 && snd < (i64)node_count;")
+            E("const int xsrc = rv ? (int)snd : -1;")
+            if self.R == 1:
+                E("const int xsrc_u = __builtin_amdgcn_readfirstlane(xsrc);")
+            E(f"const T* __restrict__ Yr = Y + e * {self.D2};")
+            E(f"const T* __restrict__ Wr = W + e * {self.WN};")
+            self.emit_y_load(E, "Yr", "rv")
+            E("oeq_sync();")
+            self.emit_x_stage(E)
+            E("oeq_sync();")
+            self.emit_x_regs(E)
+            for oi in self.used_out:
+                self.emit_forward_block(E, self.out[oi], "Wr", zname=f"z{oi}_", declare=False)
+            E.level -= 1
+            E("}")
+            E("const bool rv = nv;")
+            for o in self.out:
+                if o.dim == 0:
+                    continue
+                E("{")
+                E.level += 1
+                if o.idx in self.used_out:
+                    self.emit_block_out(E, o, f"z{o.idx}_", "Z", self.D3, own_z, zrow_of)
+                else:
+                    if o.D > 1:
+                        E("oeq_sync();")
+                    self.emit_block_zero(E, o, "Z", self.D3, own_z, zrow_of)
+                E.level -= 1
+                E("}")
+        self.chunk_loop(E, body)
+        return E.text()
+
+    def conv_det_backward_body(self) -> str:
+        """dX[node] = sum over the node's outgoing edges (walked in sender-sorted order through
+        the transpose permutation); dW[e] chunk and dY[e] (partial per chunk) written per edge."""
+        E = Emitter()
+        self.emit_lane(E)
+        self._node_prologue(E, "PTR_STRIDE")
+        own_x = ("node", "nv")
+        xrow_of = lambda r: (f"(node0 + {r})", f"(node0 + {r} < node_count)")
+
+        def body(E):
+            # this node's own X chunk is staged once
+            E("{")
+            E("    const bool rv = nv;")
+            E("    const int xsrc = nv ? (int)node : -1;")
+            if self.R == 1:
+                E("    const int xsrc_u = __builtin_amdgcn_readfirstlane(xsrc);")
+            E.level += 1
+            self.emit_x_stage(E)
+            E.level -= 1
+            E("}")
+            E("oeq_sync();")
+            E("bool rv = nv;")
+            self.emit_x_regs(E)
+            for i in self.used_in1:
+                for m in range(self.in1[i].D):
+                    E(f"T dx{i}_{m} = (T)0;")
+            E("for (int it = 0; it < maxlen; ++it) {")
+            E.level += 1
+            E("const bool ev = it < len;")
+            E("i64 e = -1, rcv = -1;")
+            E("if (ev) { e = tperm[beg + it]; }")
+            E("if (e >= 0 && e < (i64)nnz) rcv = rows[e];")
+            E("rv = ev && rcv >= 0 && rcv < (i64)node_count;")
+            E("const int zdst = rv ? (int)rcv : -1;")
+            if self.R == 1:
+                E("const int zdst_u = __builtin_amdgcn_readfirstlane(zdst);")
+            E("const u64 eu = rv ? (u64)e : 0;")
+            E(f"const T* __restrict__ Yr = Y + eu * {self.D2};")
+            E(f"const T* __restrict__ Wr = W + eu * {self.WN};")
+            E(f"T* __restrict__ Wgr = Wg + eu * {self.WN};")
+            self.emit_y_load(E, "Yr", "rv")
+            for f in self.used_y:
+                E(f"T dy{f} = (T)0;")
+            own_z = ("zdst", "rv")
+            zrow_of = self._shfl_row("zdst")
+            for oi in self.used_out:
+                o = self.out[oi]
+                E("{")
+                E.level += 1
+                self.emit_block_in(E, o, "g", "G", self.D3, own_z, zrow_of)
+
+                def sink(E, p, v, expr):
+                    E(f"  if ({self.act(p.a)}) Wgr[{self.widx(p, 'u', v)}] = {expr};")
+                self.emit_backward_block(E, o, "Wr", sink)
+                E.level -= 1
+                E("}")
+            self.emit_dy_reduce(E)
+            E("if (rv && ul == 0) {")
+            if self.NCH > 1:
+                E(f"    T* __restrict__ Ygr = (T*)((char*)ws + DYPART_OFF) + ((u64)c * nnz + eu) * {self.D2};")
+            else:
+                E(f"    T* __restrict__ Ygr = Yg + eu * {self.D2};")
+            for f in range(self.D2):
+                E(f"    Ygr[{f}] = " + (f"dy{f};" if f in self.used_y else "(T)0;"))
+            E("}")
+            E.level -= 1
+            E("}")
+            E("rv = nv;")
+            for a in self.in1:
+                if a.dim == 0:
+                    continue
+                E("{")
+                E.level += 1
+                if a.idx in self.used_in1:
+                    self.emit_block_out(E, a, f"dx{a.idx}_", "Xg", self.D1, own_x, xrow_of)
+                else:
+                    if a.D > 1:
+                        E("oeq_sync();")
+                    self.emit_block_zero(E, a, "Xg", self.D1, own_x, xrow_of)
+                E.level -= 1
+                E("}")
+        self.chunk_loop(E, body)
+        return E.text()
+
+    # ---------------------------------------------------------------- rendering
+    def render(self, prelude: str = None) -> str:
+        env = jinja_env()
+        if prelude is None:
+            prelude = env.get_template("prelude.hip.jinja").render(T=self.T)
+        tmpl = env.get_template({"tp": "tp_uvu.hip.jinja", "conv_atomic": "conv_atomic.hip.jinja",
+                                 "conv_det": "conv_det.hip.jinja"}[self.kind])
+        return tmpl.render(g=self, prelude=prelude)
+
+    def describe(self) -> str:
+        return (f"uvu[{self.kind}] T={self.T} P={self.P} R={self.R} chunks={self.NCH} paths={len(self.paths)} "
+                f"nnz={sum(p.nnz for p in self.paths)} d1={self.D1} d2={self.D2} d3={self.D3} wn={self.WN} "
+                f"lds={self.lds_elems * self.itemsize}B")
+
+    # -------------------------------------------------------------- launch plan
+    @property
+    def dy_rows_per_block(self) -> int:
+        return max(1, 256 // max(1, self.D2))
+
+    def plan(self):
+        """(forward steps, backward steps, workspace sizing) as plain dictionaries; the
+        frontends turn them into ``runtime.Step`` records.  ``workspace`` is a function
+        ``(nnz, node_count) -> bytes`` (0 when no workspace is needed)."""
+        ROW, NODE, FIXED = 1, 2, 0
+        w = 64
+        if self.kind == "tp":
+            fwd = [dict(kernel="forward", num_threads=w, grid_kind=ROW, work_per_block=self.R)]
+            if self.shared:
+                bwd = [dict(kernel="backward", num_threads=w, grid_kind=FIXED, num_blocks=self.dw_partials),
+                       dict(kernel="backward_reduce", num_threads=256, grid_kind=FIXED,
+                            num_blocks=(self.WN + 255) // 256)]
+                ws = lambda nnz=0, nodes=0: self.dw_partials * self.WN * self.itemsize
+            else:
+                bwd = [dict(kernel="backward", num_threads=w, grid_kind=ROW, work_per_block=self.R)]
+                ws = lambda nnz=0, nodes=0: 0
+            return fwd, bwd, ws
+        if self.kind == "conv_atomic":
+            fwd = [dict(kernel="forward", num_threads=w, grid_kind=ROW, work_per_block=self.R)]
+            bwd = [dict(kernel="backward", num_threads=w, grid_kind=ROW, work_per_block=self.R)]
+            return fwd, bwd, (lambda nnz=0, nodes=0: 0)
+        fwd = [dict(kernel="prep_forward", num_threads=256, grid_kind=ROW, work_per_block=256),
+               dict(kernel="forward", num_threads=w, grid_kind=NODE, work_per_block=self.R, grid_y=self.NCH)]
+        bwd = [dict(kernel="prep_backward", num_threads=256, grid_kind=ROW, work_per_block=256),
+               dict(kernel="backward", num_threads=w, grid_kind=NODE, work_per_block=self.R, grid_y=self.NCH)]
+        if self.NCH > 1:
+            bwd.append(dict(kernel="backward_dy_reduce", num_threads=256, grid_kind=ROW,
+                            work_per_block=self.dy_rows_per_block))
+
+        def ws(nnz=0, nodes=0):
+            b = 2 * (nodes + 1) * 8
+            if self.NCH > 1:
+                b += self.NCH * nnz * self.D2 * self.itemsize
+            return b
+        return fwd, bwd, ws

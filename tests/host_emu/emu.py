@@ -1,0 +1,257 @@
+"""CPU emulation of the generated kernels (test infrastructure).
+
+The kernel generator's output is ordinary C++ apart from a small prelude of
+device helpers.  Here the same generated source is compiled for the host with a
+prelude that maps one wavefront to 64 threads (LDS -> a static array, waits ->
+a pthread barrier, lane shuffles -> an exchange buffer) and is linked with
+AddressSanitizer, then run as a separate executable on files.  This checks
+indexing, bounds and arithmetic of the generated code in the build container,
+where there is no GPU; the numbers that count are still the ones the GPU tests
+produce.
+"""
+from __future__ import annotations
+
+import hashlib
+import os
+import pathlib
+import subprocess
+import tempfile
+from typing import Dict, List, Sequence
+
+import numpy as np
+
+CACHE = pathlib.Path(tempfile.gettempdir()) / "oeq_host_emu"
+
+EMU_PRELUDE = r"""
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <functional>
+#include <mutex>
+#include <string>
+#include <thread>
+#include <vector>
+#include <pthread.h>
+using std::min; using std::max;
+typedef @T@ T;
+typedef long long i64;
+typedef unsigned long long u64;
+struct emu_dim3 { unsigned x, y, z; };
+static thread_local emu_dim3 threadIdx, blockIdx;
+static emu_dim3 gridDim, blockDim;
+#define __global__
+#define __device__
+#define __forceinline__ inline
+#define __launch_bounds__(x)
+#define __shared__ static
+static pthread_barrier_t g_bar;
+static T g_xT[1024];
+static int g_xi[1024];
+static std::mutex g_atomic_mutex;
+static inline void oeq_sync() { pthread_barrier_wait(&g_bar); }
+static inline T oeq_fma(T a, T b, T c) { return std::fma(a, b, c); }
+static inline void oeq_atomic_add(T* p, T v) { std::lock_guard<std::mutex> g(g_atomic_mutex); *p += v; }
+static inline T oeq_shfl_xor(T v, int mask) { g_xT[threadIdx.x] = v; oeq_sync(); T r = g_xT[threadIdx.x ^ mask]; oeq_sync(); return r; }
+static inline int oeq_shfl_i32(int v, int src) { g_xi[threadIdx.x] = v; oeq_sync(); int r = g_xi[src & 63]; oeq_sync(); return r; }
+static inline int oeq_shfl_xor_i32(int v, int mask) { g_xi[threadIdx.x] = v; oeq_sync(); int r = g_xi[threadIdx.x ^ mask]; oeq_sync(); return r; }
+#define __builtin_amdgcn_readfirstlane(x) oeq_shfl_i32((x), 0)
+
+static void emu_run(unsigned gx, unsigned gy, unsigned block, const std::function<void()>& kernel) {
+    gridDim = {gx, gy, 1}; blockDim = {block, 1, 1};
+    pthread_barrier_init(&g_bar, nullptr, block);
+    for (unsigned by = 0; by < gy; ++by)
+        for (unsigned bx = 0; bx < gx; ++bx) {
+            std::vector<std::thread> th;
+            for (unsigned t = 0; t < block; ++t)
+                th.emplace_back([&, t] { threadIdx = {t, 0, 0}; blockIdx = {bx, by, 0}; kernel(); });
+            for (auto& x : th) x.join();
+        }
+    pthread_barrier_destroy(&g_bar);
+}
+static std::vector<char> emu_read(const std::string& path, size_t expect) {
+    FILE* f = fopen(path.c_str(), "rb");
+    if (!f) { fprintf(stderr, "cannot open %s\n", path.c_str()); exit(3); }
+    std::vector<char> buf(expect);                 // exact size: ASan sees any overrun
+    size_t got = expect ? fread(buf.data(), 1, expect, f) : 0;
+    fclose(f);
+    if (got != expect) { fprintf(stderr, "short read %s\n", path.c_str()); exit(3); }
+    return buf;
+}
+static void emu_write(const std::string& path, const std::vector<char>& buf) {
+    FILE* f = fopen(path.c_str(), "wb");
+    if (buf.size()) fwrite(buf.data(), 1, buf.size(), f);
+    fclose(f);
+}
+"""
+
+# main() for the two operator families.  argv: dir; the directory holds job.txt:
+#   line 1: sizes; following lines: "<kernel> <threads> <grid_x> <grid_y>"
+TP_MAIN = r"""
+int main(int argc, char** argv) {
+    std::string d = argv[1];
+    FILE* job = fopen((d + "/job.txt").c_str(), "r");
+    unsigned long long n, d1, d2, d3, wrow, wsz, ws_bytes; int backward_pass;
+    if (fscanf(job, "%llu %llu %llu %llu %llu %llu %llu %d", &n, &d1, &d2, &d3, &wrow, &wsz, &ws_bytes, &backward_pass) != 8) return 3;
+    auto X = emu_read(d + "/X.bin", n * d1 * sizeof(T));
+    auto Y = emu_read(d + "/Y.bin", n * d2 * sizeof(T));
+    auto W = emu_read(d + "/W.bin", wsz * sizeof(T));
+    std::vector<char> Z(n * d3 * sizeof(T), (char)0x7f), ws(ws_bytes, (char)0x7f);
+    std::vector<char> G, Xg(n * d1 * sizeof(T), (char)0x7f), Yg(n * d2 * sizeof(T), (char)0x7f), Wg(wsz * sizeof(T), (char)0x7f);
+    if (backward_pass) G = emu_read(d + "/G.bin", n * d3 * sizeof(T));
+    char name[64]; unsigned threads, gx, gy;
+    while (fscanf(job, "%63s %u %u %u", name, &threads, &gx, &gy) == 4) {
+        std::string k = name;
+        if (k == "forward") emu_run(gx, gy, threads, [&] { forward(n, (const T*)X.data(), (const T*)Y.data(), (T*)Z.data(), (const T*)W.data(), ws.data()); });
+        else if (k == "backward") emu_run(gx, gy, threads, [&] { backward(n, (const T*)X.data(), (T*)Xg.data(), (const T*)Y.data(), (T*)Yg.data(), (const T*)W.data(), (T*)Wg.data(), (const T*)G.data(), ws.data()); });
+@EXTRA@
+        else { fprintf(stderr, "unknown kernel %s\n", name); return 3; }
+    }
+    fclose(job);
+    emu_write(d + "/Z.bin", Z); emu_write(d + "/Xg.bin", Xg); emu_write(d + "/Yg.bin", Yg); emu_write(d + "/Wg.bin", Wg);
+    return 0;
+}
+"""
+
+TP_EXTRA_SHARED = r"""
+        else if (k == "backward_reduce") emu_run(gx, gy, threads, [&] { backward_reduce(n, (const T*)X.data(), (T*)Xg.data(), (const T*)Y.data(), (T*)Yg.data(), (const T*)W.data(), (T*)Wg.data(), (const T*)G.data(), ws.data()); });
+"""
+
+CONV_MAIN = r"""
+int main(int argc, char** argv) {
+    std::string d = argv[1];
+    FILE* job = fopen((d + "/job.txt").c_str(), "r");
+    unsigned long long nnz, nodes, d1, d2, d3, wn, ws_bytes; int backward_pass, has_tperm;
+    if (fscanf(job, "%llu %llu %llu %llu %llu %llu %llu %d %d", &nnz, &nodes, &d1, &d2, &d3, &wn, &ws_bytes, &backward_pass, &has_tperm) != 9) return 3;
+    auto X = emu_read(d + "/X.bin", nodes * d1 * sizeof(T));
+    auto Y = emu_read(d + "/Y.bin", nnz * d2 * sizeof(T));
+    auto W = emu_read(d + "/W.bin", nnz * wn * sizeof(T));
+    auto rows = emu_read(d + "/rows.bin", nnz * 8);
+    auto cols = emu_read(d + "/cols.bin", nnz * 8);
+    std::vector<char> tperm;
+    if (has_tperm) tperm = emu_read(d + "/tperm.bin", nnz * 8);
+    // accumulation targets start at zero (caller contract of the atomic kernels); the
+    // deterministic kernels overwrite them, so fill those with junk instead
+    const char fill = has_tperm ? (char)0x7f : (char)0;
+    std::vector<char> Z(nodes * d3 * sizeof(T), fill), ws(ws_bytes, (char)0x7f);
+    std::vector<char> G, Xg(nodes * d1 * sizeof(T), fill), Yg(nnz * d2 * sizeof(T), (char)0x7f), Wg(nnz * wn * sizeof(T), (char)0x7f);
+    if (backward_pass) G = emu_read(d + "/G.bin", nodes * d3 * sizeof(T));
+    char name[64]; unsigned threads, gx, gy;
+#define FWD_CALL(fn) emu_run(gx, gy, threads, [&] { fn((const T*)X.data(), (const T*)Y.data(), (const T*)W.data(), (T*)Z.data(), (const i64*)rows.data(), (const i64*)cols.data(), nnz, nodes, ws.data(), (const i64*)tperm.data()); })
+#define BWD_CALL(fn) emu_run(gx, gy, threads, [&] { fn((const T*)X.data(), (T*)Xg.data(), (const T*)Y.data(), (T*)Yg.data(), (const T*)W.data(), (T*)Wg.data(), (const T*)G.data(), (const i64*)rows.data(), (const i64*)cols.data(), nnz, nodes, ws.data(), (const i64*)tperm.data()); })
+    while (fscanf(job, "%63s %u %u %u", name, &threads, &gx, &gy) == 4) {
+        std::string k = name;
+        if (k == "forward") FWD_CALL(forward);
+        else if (k == "backward") BWD_CALL(backward);
+@EXTRA@
+        else { fprintf(stderr, "unknown kernel %s\n", name); return 3; }
+    }
+    fclose(job);
+    emu_write(d + "/Z.bin", Z); emu_write(d + "/Xg.bin", Xg); emu_write(d + "/Yg.bin", Yg); emu_write(d + "/Wg.bin", Wg);
+    return 0;
+}
+"""
+
+CONV_EXTRA_DET = r"""
+        else if (k == "prep_forward") FWD_CALL(prep_forward);
+        else if (k == "prep_backward") BWD_CALL(prep_backward);
+"""
+CONV_EXTRA_DYRED = r"""
+        else if (k == "backward_dy_reduce") BWD_CALL(backward_dy_reduce);
+"""
+
+
+def emu_prelude(ctype: str) -> str:
+    return EMU_PRELUDE.replace("@T@", ctype)
+
+
+def build(source: str, main: str) -> pathlib.Path:
+    """Compile generated source (rendered with ``emu_prelude``) + ``main`` with ASan."""
+    text = source + "\n" + main
+    key = hashlib.sha256(text.encode()).hexdigest()[:24]
+    CACHE.mkdir(parents=True, exist_ok=True)
+    exe = CACHE / f"emu_{key}"
+    if exe.exists():
+        return exe
+    src = CACHE / f"emu_{key}.cpp"
+    src.write_text(text)
+    cmd = ["g++", "-std=c++17", "-O1", "-g", "-fsanitize=address", "-static-libasan", "-fno-omit-frame-pointer",
+           "-Wno-unknown-pragmas", "-ffp-contract=off", str(src), "-o", str(exe) + ".tmp", "-lpthread"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("host build of generated kernel failed:\n" + res.stderr[-6000:])
+    os.replace(str(exe) + ".tmp", exe)
+    return exe
+
+
+def grid_of(step: Dict, rows: int, nodes: int) -> int:
+    """Same rule as the C library's launch()."""
+    kind = step.get("grid_kind", 1)
+    if kind == 0:
+        return step["num_blocks"]
+    work = rows if kind == 1 else nodes
+    wpb = step["work_per_block"]
+    g = (work + wpb - 1) // wpb
+    if step.get("num_blocks", 0):
+        g = min(g, step["num_blocks"])
+    return g
+
+
+def _run(exe: pathlib.Path, workdir: str) -> None:
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0:verify_asan_link_order=0")
+    res = subprocess.run([str(exe), workdir], capture_output=True, text=True, env=env, timeout=600)
+    if res.returncode != 0:
+        raise RuntimeError(f"emulated kernel failed (exit {res.returncode}):\n{res.stderr[-6000:]}")
+
+
+def run_tp(gen, steps: Sequence[Dict], X, Y, W, G=None, ws_bytes: int = 0):
+    """Run TP steps; returns dict of outputs (Z or dX, dY, dW)."""
+    dt = np.float32 if gen.T == "float" else np.float64
+    main = TP_MAIN.replace("@EXTRA@", TP_EXTRA_SHARED if gen.shared else "")
+    exe = build(gen.render(prelude=emu_prelude(gen.T)), main)
+    n = X.shape[0]
+    with tempfile.TemporaryDirectory() as d:
+        for name, arr in (("X", X), ("Y", Y), ("W", W)) + ((("G", G),) if G is not None else ()):
+            np.ascontiguousarray(arr, dtype=dt).tofile(os.path.join(d, name + ".bin"))
+        with open(os.path.join(d, "job.txt"), "w") as f:
+            f.write(f"{n} {gen.D1} {gen.D2} {gen.D3} {W.shape[-1]} {W.size} {ws_bytes} {int(G is not None)}\n")
+            for s in steps:
+                f.write(f"{s['kernel']} {s['num_threads']} {grid_of(s, n, 0)} {s.get('grid_y', 1)}\n")
+        _run(exe, d)
+        out = {}
+        out["Z"] = np.fromfile(os.path.join(d, "Z.bin"), dtype=dt).reshape(n, gen.D3)
+        out["Xg"] = np.fromfile(os.path.join(d, "Xg.bin"), dtype=dt).reshape(n, gen.D1)
+        out["Yg"] = np.fromfile(os.path.join(d, "Yg.bin"), dtype=dt).reshape(n, gen.D2)
+        out["Wg"] = np.fromfile(os.path.join(d, "Wg.bin"), dtype=dt).reshape(W.shape)
+    return out
+
+
+def run_conv(gen, steps: Sequence[Dict], X, Y, W, rows, cols, G=None, tperm=None, ws_bytes: int = 0):
+    dt = np.float32 if gen.T == "float" else np.float64
+    extra = ""
+    if gen.kind == "conv_det":
+        extra += CONV_EXTRA_DET
+        if gen.NCH > 1:
+            extra += CONV_EXTRA_DYRED
+    exe = build(gen.render(prelude=emu_prelude(gen.T)), CONV_MAIN.replace("@EXTRA@", extra))
+    nodes, nnz = X.shape[0], rows.shape[0]
+    with tempfile.TemporaryDirectory() as d:
+        for name, arr in (("X", X), ("Y", Y), ("W", W)) + ((("G", G),) if G is not None else ()):
+            np.ascontiguousarray(arr, dtype=dt).tofile(os.path.join(d, name + ".bin"))
+        np.ascontiguousarray(rows, dtype=np.int64).tofile(os.path.join(d, "rows.bin"))
+        np.ascontiguousarray(cols, dtype=np.int64).tofile(os.path.join(d, "cols.bin"))
+        if tperm is not None:
+            np.ascontiguousarray(tperm, dtype=np.int64).tofile(os.path.join(d, "tperm.bin"))
+        with open(os.path.join(d, "job.txt"), "w") as f:
+            f.write(f"{nnz} {nodes} {gen.D1} {gen.D2} {gen.D3} {gen.WN} {ws_bytes} {int(G is not None)} {int(tperm is not None)}\n")
+            for s in steps:
+                f.write(f"{s['kernel']} {s['num_threads']} {grid_of(s, nnz, nodes)} {s.get('grid_y', 1)}\n")
+        _run(exe, d)
+        out = {}
+        out["Z"] = np.fromfile(os.path.join(d, "Z.bin"), dtype=dt).reshape(nodes, gen.D3)
+        out["Xg"] = np.fromfile(os.path.join(d, "Xg.bin"), dtype=dt).reshape(nodes, gen.D1)
+        out["Yg"] = np.fromfile(os.path.join(d, "Yg.bin"), dtype=dt).reshape(nnz, gen.D2)
+        out["Wg"] = np.fromfile(os.path.join(d, "Wg.bin"), dtype=dt).reshape(nnz, gen.WN)
+    return out
