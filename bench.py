@@ -1,0 +1,182 @@
+"""Headline benchmark: MACE-style uvu tensor product, forward + backward, on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload mace_uvu|nequip_conv_atomic|...]
+
+A step is one forward and one backward pass of the hot path over one batch of synthetic,
+seeded inputs that already live in HBM.  Prints ONE JSON line.  Besides the whole-job
+throughput (edges/s) it reports, for the dominant kernel, the achieved algorithmic bandwidth
+measured with HIP events around every launch of the timed region, and a CPU baseline (the
+e3nn-equivalent torch implementation on the host cores, on a bounded sample).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import pathlib
+import sys
+import time
+
+ROOT = pathlib.Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+MFMA_FP32_PEAK_TFLOPS = 157.3
+MFMA_FP64_PEAK_TFLOPS = 78.6
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="mace_uvu")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-sample", type=int, default=0, help="edges in the CPU sample (0 = automatic)")
+    return ap.parse_args()
+
+
+class Events:
+    """HIP event pairs on torch's current stream (the stream every kernel is launched on)."""
+
+    def __init__(self):
+        import torch
+        self.torch = torch
+        self.pairs = {}
+
+    def wrap(self, name, fn):
+        a = self.torch.cuda.Event(enable_timing=True)
+        b = self.torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        self.pairs.setdefault(name, []).append((a, b))
+
+    def mean_ms(self, name):
+        v = [a.elapsed_time(b) for a, b in self.pairs.get(name, [])]
+        return sum(v) / len(v) if v else float("nan")
+
+
+def load_traffic(key):
+    """Measured HBM bytes per launch from committed counter summaries (None when absent)."""
+    p = ROOT / "profiles" / "traffic.json"
+    if p.exists():
+        try:
+            return json.loads(p.read_text()).get(key)
+        except Exception:
+            return None
+    return None
+
+
+def cpu_baseline(wl, case, sample):
+    """e3nn-equivalent torch implementation on the host cores, forward+backward, fp32, on a
+    bounded sample of the same seeded inputs (the op is independent per row/edge, so the rate of
+    the sample is the rate of the workload).  This is the only place where the oracle package is
+    used by the benchmark: as the thing timed beside the GPU, never as the product."""
+    from oracle import spec, torch_cpu
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+    h = case.host
+    if wl.mode == "uvw":
+        oprob = spec.fully_connected(*wl.irreps, shared_weights=True)
+    elif wl.name == "readme_uvu":
+        oprob = spec.Problem(*wl.irreps, [(0, 0, 0, "uvu", True)], shared_weights=False)
+    else:
+        oprob = spec.channelwise(*wl.irreps)
+    if wl.kind == "tp":
+        n = sample or min(wl.units, {"mace_uvu": 1000, "readme_uvu": 1000}.get(wl.name, 2000))
+        W = h["W"] if h["W"].ndim == 1 else h["W"][:n]
+        args_ = (h["X"][:n], h["Y"][:n], W, h["G"][:n])
+        sec = torch_cpu.time_forward_backward(oprob, *args_, threads=cores, repeats=1)
+        reps = max(1, min(20, int(10.0 / max(sec, 1e-3))))
+        sec = torch_cpu.time_forward_backward(oprob, *args_, threads=cores, repeats=reps)
+        what = f"first {n} rows of the same seeded batch, {reps} repeats"
+    else:
+        n = sample or min(wl.units, 5000)
+        rows, cols = h["rows"][:n], h["cols"][:n]
+        args_ = (h["X"], h["Y"][:n], h["W"][:n], h["G"])
+        sec = torch_cpu.time_forward_backward(oprob, *args_, threads=cores, repeats=1, rows=rows, cols=cols)
+        reps = max(1, min(20, int(10.0 / max(sec, 1e-3))))
+        sec = torch_cpu.time_forward_backward(oprob, *args_, threads=cores, repeats=reps, rows=rows, cols=cols)
+        what = f"first {n} edges of the same seeded graph (all nodes), {reps} repeats"
+    return {"value": round(n / sec, 1), "unit": wl.unit, "cores": cores, "kind": "port",
+            "sample": what + "; torch CPU einsum + autograd, fp32 (e3nn itself is not installable offline)"}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (the path shards over rows/edges "
+              "without communication, see DESIGN.md)", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    import openequivariance_amd as oeq
+    from openequivariance_amd import workloads
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    dev = torch.device("cuda:0")
+    wl = workloads.get(args.workload)
+    case = wl.build(dev)                      # operator + device tensors + raw-call closures
+    ev = Events()
+
+    def step(timed):
+        if timed:
+            ev.wrap("forward", case.forward)
+            ev.wrap("backward", case.backward)
+        else:
+            case.forward()
+            case.backward()
+
+    for _ in range(args.warmup):
+        step(False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(True)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    value = wl.units / (ms_per_step * 1e-3)
+
+    fwd_ms, bwd_ms = ev.mean_ms("forward"), ev.mean_ms("backward")
+    dom = "backward" if bwd_ms >= fwd_ms else "forward"
+    dom_ms = max(fwd_ms, bwd_ms)
+    if wl.bound == "hbm":
+        alg = wl.alg_bytes[dom]
+        achieved = alg / (dom_ms * 1e-3) / 1e9
+        peak, unit = HBM_PEAK_GBS, "GB/s"
+    else:
+        alg = wl.alg_flops[dom]
+        achieved = alg / (dom_ms * 1e-3) / 1e12
+        peak, unit = (MFMA_FP32_PEAK_TFLOPS if wl.dtype == "f32" else MFMA_FP64_PEAK_TFLOPS), "TFLOP/s"
+    roofline = {"bound": wl.bound, "kernel": f"{wl.name}:{dom}", "achieved": round(achieved, 2), "peak": peak,
+                "unit": unit, "frac": round(achieved / peak, 4), "traffic": load_traffic(f"{wl.name}:{dom}"),
+                "algorithmic_per_launch": alg, "avg_launch_ms": round(dom_ms, 5),
+                "forward_ms": round(fwd_ms, 5), "backward_ms": round(bwd_ms, 5)}
+    if wl.bound == "hbm":
+        tot = wl.alg_bytes["forward"] + wl.alg_bytes["backward"]
+        roofline["fwd_bwd_frac"] = round(tot / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / peak, 4)
+        roofline["forward_frac"] = round(wl.alg_bytes["forward"] / (fwd_ms * 1e-3) / 1e9 / peak, 4)
+        roofline["backward_frac"] = round(wl.alg_bytes["backward"] / (bwd_ms * 1e-3) / 1e9 / peak, 4)
+    else:
+        tot = wl.alg_flops["forward"] + wl.alg_flops["backward"]
+        roofline["fwd_bwd_frac"] = round(tot / ((fwd_ms + bwd_ms) * 1e-3) / 1e12 / peak, 4)
+
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline(wl, case, args.cpu_sample)
+
+    out = {"metric": "fwd+bwd edges/s and % HBM roofline, MACE-style uvu TP and fused conv",
+           "value": round(value, 1), "unit": wl.unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak",
+           "vs_baseline": None, "dtype": wl.dtype, "data": "synthetic",
+           "config": {"workload": wl.description, **wl.config},
+           "roofline": roofline, "cpu_baseline": cpu,
+           "device": torch.cuda.get_device_name(0)}
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,326 @@
+"""``TensorProductConv``: fused gather - tensor product - scatter over graph edges.
+
+Host-side mirror of the reference's ``oeq.TensorProductConv`` / ``LoopUnrollConv``
+(reference: openequivariance/implementations/convolution/LoopUnrollConv.py:7-90,
+ConvolutionBase.py:72-100 and :560-709): same constructor
+``(problem, torch_op=False, deterministic=False)``, same ``forward`` signatures
+(five arguments, plus ``transpose_perm`` when deterministic), first and second
+derivatives through torch custom ops, raw-pointer entry points.
+
+``rows`` are receivers (where Z rows are accumulated), ``cols`` are senders
+(where X rows are gathered), both int64.  The deterministic variant requires
+the edge list sorted by receiver and ``transpose_perm[j]`` = position in that
+list of the j-th edge in (sender, receiver) order; it makes no symmetry
+assumption about the graph.
+"""
+from __future__ import annotations
+
+import typing
+
+import numpy as np
+import torch
+
+from . import runtime as rt
+from .codegen.uvu import UVUGenerator
+from .problem import TPProblem
+from .tensor_product import _make_steps, validate_problem
+from .weight_order import WeightReorder
+from .wigner import wigner_3j
+
+
+def flops_data_per_tp(config: TPProblem, direction: str):
+    """(flops, bytes, nnz) per edge by the reference's model
+    (reference: convolution/ConvolutionBase.py:11-43)."""
+    s = np.dtype(config.irrep_dtype).itemsize
+    L1, L2, L3 = config.irreps_in1, config.irreps_in2, config.irreps_out
+    if direction == "forward":
+        ops_per_nz, words = 3, L1.dim + L2.dim + L3.dim + config.weight_numel
+    elif direction == "backward":
+        ops_per_nz, words = 9, 2 * L1.dim + 2 * L2.dim + L3.dim + 2 * config.weight_numel
+    else:
+        raise ValueError(direction)
+    ops = nnz = 0
+    for ins in config.instructions:
+        c = wigner_3j(L1[ins.i_in1].ir.l, L2[ins.i_in2].ir.l, L3[ins.i_out].ir.l)
+        k = int(np.count_nonzero(np.abs(c) > 1e-14))
+        nnz += k
+        ops += ops_per_nz * k * L1[ins.i_in1].mul * L2[ins.i_in2].mul
+        if ins.connection_mode == "uvu":
+            ops += L3[ins.i_out].mul * L3[ins.i_out].ir.dim
+        else:
+            ops += L1[ins.i_in1].mul * L2[ins.i_in2].mul * L3[ins.i_out].ir.dim * L3[ins.i_out].mul
+    return ops, words * s, nnz
+
+
+class CoordGraph:
+    """Receiver-sorted COO graph with its transpose permutation
+    (reference: convolution/ConvolutionBase.py:45-70, vectorised)."""
+
+    def __init__(self, coords, rows, cols, name="graph"):
+        rows, cols = np.asarray(rows), np.asarray(cols)
+        assert len(rows) == len(cols)
+        self.nnz = len(rows)
+        self.node_count = coords.shape[0] if hasattr(coords, "shape") else int(coords)
+        self.coords, self.name = coords, name
+        order = np.lexsort((cols, rows))
+        self.rows, self.cols = rows[order], cols[order]
+        self.order = order
+        self.transpose_perm = np.lexsort((np.arange(self.nnz), self.rows, self.cols)).astype(self.rows.dtype)
+
+
+class TensorProductConv:
+    """Drop-in for ``oeq.TensorProductConv``."""
+    next_conv_id = 0
+
+    def __init__(self, config: TPProblem, torch_op: bool = False, deterministic: bool = False,
+                 idx_dtype=np.int64):
+        assert isinstance(config, TPProblem)
+        self.config = config
+        self.L1, self.L2, self.L3 = config.irreps_in1, config.irreps_in2, config.irreps_out
+        self.torch_op, self.deterministic = torch_op, deterministic
+        if np.dtype(idx_dtype) != np.dtype(np.int64):
+            raise NotImplementedError("index tensors must be int64")
+        self.idx_dtype = np.int64
+        self.conv_id = TensorProductConv.next_conv_id
+        TensorProductConv.next_conv_id += 1
+
+        mode = validate_problem(config)
+        for (mul, ir) in self.L2:
+            assert mul == 1, "TensorProductConv requires multiplicity 1 for every irrep of the second operand"
+        if mode != "uvu":
+            raise NotImplementedError("TensorProductConv supports uvu problems")
+
+        self.generator = UVUGenerator(config, "conv_det" if deterministic else "conv_atomic")
+        self.jit_kernel = self.generator.render()
+        code = rt.compile_source(self.jit_kernel)
+        fwd, bwd, self._ws_bytes = self.generator.plan()
+        self.internal = rt.ConvImpl(code, _make_steps(fwd), _make_steps(bwd))
+        self.workspace_buffer = None
+        self.workspace_size = 0
+        self._reorder = WeightReorder(config)
+        self.reorder_weights_e3nn_to_oeq = self._reorder.e3nn_to_oeq
+        self.reorder_weights_oeq_to_e3nn = self._reorder.oeq_to_e3nn
+        if torch_op:
+            self._setup_torch_module()
+
+    @staticmethod
+    def name():
+        return "LoopUnrollConv"
+
+    # ------------------------------------------------------------------ helpers
+    def workspace_ptr(self, nnz: int, node_count: int) -> int:
+        """Device scratch for the deterministic variant, grown on demand and kept for the
+        lifetime of the object (reference: ConvolutionBase.py:93-100 allocates it once)."""
+        need = self._ws_bytes(nnz, node_count)
+        if need == 0:
+            return 0
+        if self.workspace_buffer is None or self.workspace_size < need:
+            self.workspace_size = int(need * 1.25) + 256
+            self.workspace_buffer = torch.empty(self.workspace_size, dtype=torch.uint8, device="cuda")
+        return self.workspace_buffer.data_ptr()
+
+    @staticmethod
+    def _stream() -> int:
+        return torch.cuda.current_stream().cuda_stream
+
+    def _check(self, x, y, w, rows, cols, tperm=None):
+        E, N = rows.shape[0], x.shape[0]
+        if N >= 2 ** 31:
+            raise ValueError("node count must be below 2^31")
+        if x.ndim != 2 or x.shape[1] != self.L1.dim:
+            raise ValueError(f"L1_in must have shape [nodes, {self.L1.dim}], got {tuple(x.shape)}")
+        if tuple(y.shape) != (E, self.L2.dim):
+            raise ValueError(f"L2_in must have shape [{E}, {self.L2.dim}], got {tuple(y.shape)}")
+        if tuple(w.shape) != (E, self.config.weight_numel):
+            raise ValueError(f"weights must have shape [{E}, {self.config.weight_numel}], got {tuple(w.shape)}")
+        for name, t in (("rows", rows), ("cols", cols)) + ((("transpose_perm", tperm),) if tperm is not None else ()):
+            if t.dtype != torch.int64 or tuple(t.shape) != (E,):
+                raise TypeError(f"{name} must be an int64 tensor of shape [{E}]")
+        tdt = {np.float32: torch.float32, np.float64: torch.float64}[self.config.irrep_dtype]
+        if x.dtype != tdt or y.dtype != tdt or w.dtype != tdt:
+            raise TypeError(f"tensors must be {tdt}")
+
+    # ---------------------------------------------------------- raw entry points
+    def exec_conv_rawptrs(self, L1_in, L2_in, weights, L3_out, rows, cols, nnz, node_count, workspace=0,
+                          transpose_perm=0, stream=None):
+        """reference: extension/convolution.hpp:121-147"""
+        self.internal.exec_conv_rawptrs(L1_in, L2_in, weights, L3_out, rows, cols, int(nnz), int(node_count),
+                                        workspace, transpose_perm, self._stream() if stream is None else stream)
+
+    def backward_rawptrs(self, L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_grad, rows, cols, nnz,
+                         node_count, workspace=0, transpose_perm=0, stream=None):
+        """reference: extension/convolution.hpp:149-173"""
+        self.internal.backward_rawptrs(L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_grad, rows, cols,
+                                       int(nnz), int(node_count), workspace, transpose_perm,
+                                       self._stream() if stream is None else stream)
+
+    # ------------------------------------------------------------------ torch ops
+    def _setup_torch_module(self) -> None:
+        """reference: ConvolutionBase.py:560-709."""
+        L3_dim = self.L3.dim
+        det = self.deterministic
+        cid = self.conv_id
+
+        def fwd_impl(L1_in, L2_in, weights, rows, cols, tperm):
+            x, y, w = L1_in.contiguous(), L2_in.contiguous(), weights.contiguous()
+            rows, cols = rows.contiguous(), cols.contiguous()
+            tperm = tperm.contiguous() if tperm is not None else None
+            self._check(x, y, w, rows, cols, tperm)
+            E, N = rows.shape[0], x.shape[0]
+            # the atomic kernels accumulate into Z; the deterministic ones write every row
+            out = (torch.empty if det else torch.zeros)((N, L3_dim), dtype=x.dtype, device=x.device)
+            self.exec_conv_rawptrs(x.data_ptr(), y.data_ptr(), w.data_ptr(), out.data_ptr(), rows.data_ptr(),
+                                   cols.data_ptr(), E, N, self.workspace_ptr(E, N),
+                                   tperm.data_ptr() if tperm is not None else 0)
+            return out
+
+        def bwd_impl(L1_in, L2_in, weights, L3_grad, rows, cols, tperm):
+            x, y, w, g = L1_in.contiguous(), L2_in.contiguous(), weights.contiguous(), L3_grad.contiguous()
+            rows, cols = rows.contiguous(), cols.contiguous()
+            tperm = tperm.contiguous() if tperm is not None else None
+            self._check(x, y, w, rows, cols, tperm)
+            E, N = rows.shape[0], x.shape[0]
+            xg = (torch.empty_like if det else torch.zeros_like)(x)
+            yg, wg = torch.empty_like(y), torch.empty_like(w)
+            self.backward_rawptrs(x.data_ptr(), xg.data_ptr(), y.data_ptr(), yg.data_ptr(), w.data_ptr(),
+                                  wg.data_ptr(), g.data_ptr(), rows.data_ptr(), cols.data_ptr(), E, N,
+                                  self.workspace_ptr(E, N), tperm.data_ptr() if tperm is not None else 0)
+            return [xg, yg, wg]
+
+        if not det:
+            @torch.library.custom_op(f"openequivariance_amd::conv_forward{cid}", mutates_args=(), device_types="cuda")
+            def forward(L1_in: torch.Tensor, L2_in: torch.Tensor, weights: torch.Tensor, rows: torch.Tensor,
+                        cols: torch.Tensor) -> torch.Tensor:
+                return fwd_impl(L1_in, L2_in, weights, rows, cols, None)
+
+            @forward.register_fake
+            def _(L1_in, L2_in, weights, rows, cols):
+                return L1_in.new_empty(L1_in.shape[0], L3_dim)
+
+            @torch.library.custom_op(f"openequivariance_amd::conv_backward{cid}", mutates_args=(), device_types="cuda")
+            def backward_helper(L1_in: torch.Tensor, L2_in: torch.Tensor, weights: torch.Tensor, L3_grad: torch.Tensor,
+                                rows: torch.Tensor, cols: torch.Tensor) -> typing.List[torch.Tensor]:
+                return bwd_impl(L1_in, L2_in, weights, L3_grad, rows, cols, None)
+
+            @backward_helper.register_fake
+            def _(L1_in, L2_in, weights, L3_grad, rows, cols):
+                return [L1_in.new_empty(*L1_in.shape), L2_in.new_empty(*L2_in.shape), weights.new_empty(*weights.shape)]
+
+            def setup_context(ctx, inputs, output):
+                ctx.L1_in, ctx.L2_in, ctx.weights, ctx.rows, ctx.cols = inputs
+
+            def backward(ctx, grad_output):
+                r = backward_helper(ctx.L1_in, ctx.L2_in, ctx.weights, grad_output, ctx.rows, ctx.cols)
+                return r[0], r[1], r[2], None, None
+
+            forward.register_autograd(backward, setup_context=setup_context)
+
+            def setup_context_double_backward(ctx, inputs, output):
+                ctx.L1_in, ctx.L2_in, ctx.weights, ctx.L3_grad, ctx.rows, ctx.cols = inputs
+
+            def double_backward(ctx, grad_output):
+                A, B, C, D = ctx.L1_in, ctx.L2_in, ctx.L3_grad, ctx.weights
+                E, F, G = grad_output[0], grad_output[1], grad_output[2]
+                r, c = ctx.rows, ctx.cols
+                op1 = backward_helper(E, F, D, C, r, c)
+                op2 = backward_helper(A, B, G, C, r, c)
+                op3 = forward(E, B, D, r, c)
+                op4 = backward_helper(E, B, D, C, r, c)
+                op5 = backward_helper(A, F, D, C, r, c)
+                op6 = forward(A, F, D, r, c)
+                op7 = forward(A, B, G, r, c)
+                return op1[0] + op2[0], op1[1] + op2[1], (op4[2] + op5[2]), (op3 + op6 + op7), None, None
+
+            backward_helper.register_autograd(double_backward, setup_context=setup_context_double_backward)
+        else:
+            @torch.library.custom_op(f"openequivariance_amd::conv_forward{cid}", mutates_args=(), device_types="cuda")
+            def forward(L1_in: torch.Tensor, L2_in: torch.Tensor, weights: torch.Tensor, rows: torch.Tensor,
+                        cols: torch.Tensor, transpose_perm: torch.Tensor) -> torch.Tensor:
+                return fwd_impl(L1_in, L2_in, weights, rows, cols, transpose_perm)
+
+            @forward.register_fake
+            def _(L1_in, L2_in, weights, rows, cols, transpose_perm):
+                return L1_in.new_empty(L1_in.shape[0], L3_dim)
+
+            @torch.library.custom_op(f"openequivariance_amd::conv_backward{cid}", mutates_args=(), device_types="cuda")
+            def backward_helper(L1_in: torch.Tensor, L2_in: torch.Tensor, weights: torch.Tensor, L3_grad: torch.Tensor,
+                                rows: torch.Tensor, cols: torch.Tensor,
+                                transpose_perm: torch.Tensor) -> typing.List[torch.Tensor]:
+                return bwd_impl(L1_in, L2_in, weights, L3_grad, rows, cols, transpose_perm)
+
+            @backward_helper.register_fake
+            def _(L1_in, L2_in, weights, L3_grad, rows, cols, transpose_perm):
+                return [L1_in.new_empty(*L1_in.shape), L2_in.new_empty(*L2_in.shape), weights.new_empty(*weights.shape)]
+
+            def setup_context(ctx, inputs, output):
+                ctx.L1_in, ctx.L2_in, ctx.weights, ctx.rows, ctx.cols, ctx.transpose_perm = inputs
+
+            def backward(ctx, grad_output):
+                r = backward_helper(ctx.L1_in, ctx.L2_in, ctx.weights, grad_output, ctx.rows, ctx.cols,
+                                    ctx.transpose_perm)
+                return r[0], r[1], r[2], None, None, None
+
+            forward.register_autograd(backward, setup_context=setup_context)
+
+            def setup_context_double_backward(ctx, inputs, output):
+                ctx.L1_in, ctx.L2_in, ctx.weights, ctx.L3_grad, ctx.rows, ctx.cols, ctx.transpose_perm = inputs
+
+            def double_backward(ctx, grad_output):
+                A, B, C, D = ctx.L1_in, ctx.L2_in, ctx.L3_grad, ctx.weights
+                E, F, G = grad_output[0], grad_output[1], grad_output[2]
+                r, c, t = ctx.rows, ctx.cols, ctx.transpose_perm
+                op1 = backward_helper(E, F, D, C, r, c, t)
+                op2 = backward_helper(A, B, G, C, r, c, t)
+                op3 = forward(E, B, D, r, c, t)
+                op4 = backward_helper(E, B, D, C, r, c, t)
+                op5 = backward_helper(A, F, D, C, r, c, t)
+                op6 = forward(A, F, D, r, c, t)
+                op7 = forward(A, B, G, r, c, t)
+                return (op1[0] + op2[0], op1[1] + op2[1], (op4[2] + op5[2]), (op3 + op6 + op7), None, None, None)
+
+            backward_helper.register_autograd(double_backward, setup_context=setup_context_double_backward)
+
+        self.forward = forward
+        self.backward_helper = backward_helper
+
+    def __call__(self, *args):
+        return self.forward(*args)
+
+    # ---------------------------------------------------- numpy entry points (tests)
+    def forward_cpu(self, L1_in, L2_in, weights, L3_out, graph) -> None:
+        """Host arrays; ``graph`` has rows / cols / node_count / nnz (and transpose_perm when
+        deterministic) (reference: ConvolutionBase.py:106-137)."""
+        assert graph.rows.dtype == self.idx_dtype
+        x, y, w = rt.DeviceBuffer(L1_in), rt.DeviceBuffer(L2_in), rt.DeviceBuffer(weights)
+        L3_out[...] = 0
+        z = rt.DeviceBuffer(L3_out)
+        r, c = rt.DeviceBuffer(graph.rows), rt.DeviceBuffer(graph.cols)
+        tp = rt.DeviceBuffer(graph.transpose_perm) if self.deterministic else None
+        nbytes = self._ws_bytes(graph.nnz, graph.node_count)
+        ws = rt.DeviceBuffer(nbytes) if nbytes else None
+        self.internal.exec_conv_rawptrs(x.data_ptr(), y.data_ptr(), w.data_ptr(), z.data_ptr(), r.data_ptr(),
+                                        c.data_ptr(), graph.nnz, graph.node_count, ws.data_ptr() if ws else 0,
+                                        tp.data_ptr() if tp else 0, 0)
+        rt.stream_synchronize(0)
+        L3_out[...] = z.copy_to_host()
+
+    def backward_cpu(self, L1_in, L1_grad, L2_in, L2_grad, L3_grad, weights, weights_grad, graph) -> None:
+        """reference: ConvolutionBase.py:139-170."""
+        assert graph.rows.dtype == self.idx_dtype
+        x, y, w, g = (rt.DeviceBuffer(a) for a in (L1_in, L2_in, weights, L3_grad))
+        L1_grad[...] = 0
+        xg, yg, wg = rt.DeviceBuffer(L1_grad), rt.DeviceBuffer(L2_grad), rt.DeviceBuffer(weights_grad)
+        r, c = rt.DeviceBuffer(graph.rows), rt.DeviceBuffer(graph.cols)
+        tp = rt.DeviceBuffer(graph.transpose_perm) if self.deterministic else None
+        nbytes = self._ws_bytes(graph.nnz, graph.node_count)
+        ws = rt.DeviceBuffer(nbytes) if nbytes else None
+        self.internal.backward_rawptrs(x.data_ptr(), xg.data_ptr(), y.data_ptr(), yg.data_ptr(), w.data_ptr(),
+                                       wg.data_ptr(), g.data_ptr(), r.data_ptr(), c.data_ptr(), graph.nnz,
+                                       graph.node_count, ws.data_ptr() if ws else 0, tp.data_ptr() if tp else 0, 0)
+        rt.stream_synchronize(0)
+        L1_grad[...] = xg.copy_to_host()
+        L2_grad[...] = yg.copy_to_host()
+        weights_grad[...] = wg.copy_to_host()
+
+
+LoopUnrollConv = TensorProductConv

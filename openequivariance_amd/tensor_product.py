@@ -1,0 +1,273 @@
+"""``TensorProduct``: the batch Clebsch-Gordan tensor product operator.
+
+Host-side mirror of the reference's ``oeq.TensorProduct`` / ``LoopUnrollTP``
+(reference: openequivariance/implementations/LoopUnrollTP.py:12-105,
+TensorProductBase.py:11-298): same constructor, same callable
+``tp(X, Y, W) -> Z``, same torch custom-op wiring with first and second
+derivatives, same raw-pointer and numpy entry points and the same weight
+reordering helpers.  Underneath, the kernels are generated for gfx950, compiled
+with hipRTC and launched through the C-ABI runtime on torch's current stream.
+"""
+from __future__ import annotations
+
+import typing
+
+import numpy as np
+import torch
+
+from . import runtime as rt
+from .codegen.uvu import UVUGenerator
+from .problem import TPProblem
+from .weight_order import WeightReorder, is_identity
+from .wigner import wigner_3j
+
+
+def _make_steps(descs):
+    return [rt.Step.make(d["kernel"], d["num_threads"], d.get("smem", 0), d.get("grid_kind", rt.GRID_PER_ROW),
+                         d.get("work_per_block", 1), d.get("num_blocks", 0), d.get("grid_y", 1)) for d in descs]
+
+
+def validate_problem(config: TPProblem) -> str:
+    """Checks shared by every operator (reference: LoopUnrollTP.py:23-30).  Returns the mode."""
+    if len(config.instructions) == 0:
+        raise ValueError("Tensor product problem has no valid intructions!")
+    mode = config.instructions[0].connection_mode
+    for inst in config.instructions:
+        assert inst.connection_mode == mode, "all instructions must share one connection mode"
+    assert mode in ("uvu", "uvw"), f"connection mode {mode!r} is not supported (uvu and uvw are)"
+    assert config.irrep_dtype == config.weight_dtype, "irrep_dtype and weight_dtype must be equal"
+    return mode
+
+
+class TensorProductBase:
+    next_tp_id = 0   # unique suffix of the torch op names (reference: TensorProductBase.py:12)
+
+    @staticmethod
+    def load_cg_tensor(l1, l2, l3):
+        return wigner_3j(l1, l2, l3)
+
+    def __init__(self, config: TPProblem, torch_op: bool = False):
+        assert isinstance(config, TPProblem)
+        assert isinstance(torch_op, bool)
+        self.config, self.torch_op = config, torch_op
+        self.L1, self.L2, self.L3 = config.irreps_in1, config.irreps_in2, config.irreps_out
+        self.irrep_dtype, self.weight_dtype = config.irrep_dtype, config.weight_dtype
+        self.tp_id = TensorProductBase.next_tp_id
+        TensorProductBase.next_tp_id += 1
+
+    def __call__(self, L1_in, L2_in, weights):
+        return self.forward(L1_in, L2_in, weights)
+
+
+class TensorProduct(TensorProductBase):
+    """Drop-in for ``oeq.TensorProduct(problem, torch_op=True)``."""
+
+    def __init__(self, problem: TPProblem, torch_op: bool = True):
+        super().__init__(problem, torch_op=torch_op)
+        config = self.config
+        mode = validate_problem(config)
+        self.is_uvw = (mode == "uvw")
+        if self.is_uvw:
+            from .codegen.uvw import UVWGenerator
+            self.generator = UVWGenerator(config)
+        else:
+            self.generator = UVUGenerator(config, "tp")
+        self.jit_kernel = self.generator.render()
+        code = rt.compile_source(self.jit_kernel)
+        fwd, bwd, ws = self.generator.plan()
+        self.workspace_bytes = ws()
+        self.internal = rt.TPImpl(code, _make_steps(fwd), _make_steps(bwd))
+        self._workspace = None
+
+        self._reorder = WeightReorder(config)
+        if is_identity(self._reorder.perm):
+            # same convention as the reference: the attribute is still callable
+            pass
+        self.reorder_weights_e3nn_to_oeq = self._reorder.e3nn_to_oeq
+        self.reorder_weights_oeq_to_e3nn = self._reorder.oeq_to_e3nn
+
+        if self.torch_op:
+            self._setup_torch_custom_op()
+
+    @staticmethod
+    def name():
+        return "LoopUnrollTP"
+
+    # ----------------------------------------------------------- raw entry points
+    def _workspace_ptr(self) -> int:
+        if self.workspace_bytes == 0:
+            return 0
+        if self._workspace is None:
+            self._workspace = torch.empty(self.workspace_bytes, dtype=torch.uint8, device="cuda")
+        return self._workspace.data_ptr()
+
+    @staticmethod
+    def _stream() -> int:
+        return torch.cuda.current_stream().cuda_stream
+
+    def forward_raw(self, batch, L1_in, L2_in, L3_out, weights, stream=None) -> None:
+        """Device pointers as integers (reference: TensorProductBase.py:41-49)."""
+        self.internal.exec_tensor_product(int(batch), L1_in, L2_in, L3_out, weights, self._workspace_ptr(),
+                                          self._stream() if stream is None else stream)
+
+    def backward_raw(self, batch_size, L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_grad,
+                     stream=None) -> None:
+        """reference: TensorProductBase.py:51-61."""
+        self.internal.backward(int(batch_size), L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_grad,
+                               self._workspace_ptr(), self._stream() if stream is None else stream)
+
+    # ------------------------------------------------- numpy entry points (tests)
+    def forward_cpu(self, L1_in, L2_in, L3_out, weights) -> None:
+        """Host arrays in, result written into ``L3_out``; ``weights`` in e3nn order
+        (reference: TensorProductBase.py:63-84)."""
+        w = np.zeros_like(weights)
+        self.reorder_weights_e3nn_to_oeq(weights, w, not self.config.shared_weights)
+        bufs = [rt.DeviceBuffer(a) for a in (L1_in, L2_in, L3_out, w)]
+        ws = rt.DeviceBuffer(self.workspace_bytes) if self.workspace_bytes else None
+        self.internal.exec_tensor_product(L1_in.shape[0], bufs[0].data_ptr(), bufs[1].data_ptr(), bufs[2].data_ptr(),
+                                          bufs[3].data_ptr(), ws.data_ptr() if ws else 0, 0)
+        rt.stream_synchronize(0)
+        L3_out[...] = bufs[2].copy_to_host()
+
+    def backward_cpu(self, L1_in, L1_grad, L2_in, L2_grad, L3_grad, weights, weights_grad) -> None:
+        """reference: TensorProductBase.py:86-112; weights and weights_grad in e3nn order."""
+        w = np.zeros_like(weights)
+        self.reorder_weights_e3nn_to_oeq(weights, w, not self.config.shared_weights)
+        x, y, g = rt.DeviceBuffer(L1_in), rt.DeviceBuffer(L2_in), rt.DeviceBuffer(L3_grad)
+        xg, yg = rt.DeviceBuffer(L1_grad), rt.DeviceBuffer(L2_grad)
+        wd, wg = rt.DeviceBuffer(w), rt.DeviceBuffer(weights_grad)
+        ws = rt.DeviceBuffer(self.workspace_bytes) if self.workspace_bytes else None
+        self.internal.backward(L1_in.shape[0], x.data_ptr(), xg.data_ptr(), y.data_ptr(), yg.data_ptr(),
+                               wd.data_ptr(), wg.data_ptr(), g.data_ptr(), ws.data_ptr() if ws else 0, 0)
+        rt.stream_synchronize(0)
+        L1_grad[...] = xg.copy_to_host()
+        L2_grad[...] = yg.copy_to_host()
+        wg_oeq = wg.copy_to_host().copy()
+        self.reorder_weights_oeq_to_e3nn(wg_oeq, weights_grad, not self.config.shared_weights)
+
+    # ------------------------------------------------------------------ torch op
+    def _setup_torch_custom_op(self) -> None:
+        """reference: TensorProductBase.py:234-298 (forward, backward, double backward)."""
+        L3_dim = self.L3.dim
+        shared = self.config.shared_weights
+
+        @torch.library.custom_op(f"openequivariance_amd::tp_forward{self.tp_id}", mutates_args=(), device_types="cuda")
+        def forward(L1_in: torch.Tensor, L2_in: torch.Tensor, weights: torch.Tensor) -> torch.Tensor:
+            x, y, w = L1_in.contiguous(), L2_in.contiguous(), weights.contiguous()
+            self._check_inputs(x, y, w)
+            out = torch.empty((x.shape[0], L3_dim), dtype=x.dtype, device=x.device)
+            self.forward_raw(x.shape[0], x.data_ptr(), y.data_ptr(), out.data_ptr(), w.data_ptr())
+            return out
+
+        @forward.register_fake
+        def _(L1_in, L2_in, weights):
+            return L1_in.new_empty(L1_in.shape[0], L3_dim)
+
+        self.forward = forward
+
+        @torch.library.custom_op(f"openequivariance_amd::tp_grad_helper{self.tp_id}", mutates_args=(), device_types="cuda")
+        def backward_helper(L1_in: torch.Tensor, L2_in: torch.Tensor, weights: torch.Tensor,
+                            L3_grad: torch.Tensor) -> typing.List[torch.Tensor]:
+            x, y, w, g = L1_in.contiguous(), L2_in.contiguous(), weights.contiguous(), L3_grad.contiguous()
+            self._check_inputs(x, y, w)
+            xg, yg, wg = torch.empty_like(x), torch.empty_like(y), torch.empty_like(w)
+            self.backward_raw(x.shape[0], x.data_ptr(), xg.data_ptr(), y.data_ptr(), yg.data_ptr(),
+                              w.data_ptr(), wg.data_ptr(), g.data_ptr())
+            return [xg, yg, wg]
+
+        @backward_helper.register_fake
+        def _(L1_in, L2_in, weights, L3_grad):
+            return [L1_in.new_empty(*L1_in.shape), L2_in.new_empty(*L2_in.shape), weights.new_empty(*weights.shape)]
+
+        self.backward_helper = backward_helper
+
+        def setup_context(ctx, inputs, output):
+            ctx.L1_in, ctx.L2_in, ctx.weights = inputs
+
+        def backward(ctx, grad_output):
+            r = backward_helper(ctx.L1_in, ctx.L2_in, ctx.weights, grad_output)
+            return r[0], r[1], r[2]
+
+        forward.register_autograd(backward, setup_context=setup_context)
+
+        def setup_context_double_backward(ctx, inputs, output):
+            ctx.L1_in, ctx.L2_in, ctx.weights, ctx.L3_grad = inputs
+
+        def double_backward(ctx, grad_output):
+            A, B, C, D = ctx.L1_in, ctx.L2_in, ctx.L3_grad, ctx.weights
+            E, F, G = grad_output[0], grad_output[1], grad_output[2]
+            op1 = backward_helper(E, F, D, C)
+            op2 = backward_helper(A, B, G, C)
+            op3 = forward(E, B, D)
+            op4 = backward_helper(E, B, D, C)
+            op5 = backward_helper(A, F, D, C)
+            op6 = forward(A, F, D)
+            op7 = forward(A, B, G)
+            return op1[0] + op2[0], op1[1] + op2[1], (op4[2] + op5[2]), (op3 + op6 + op7)
+
+        backward_helper.register_autograd(double_backward, setup_context=setup_context_double_backward)
+
+    def _check_inputs(self, x, y, w) -> None:
+        B = x.shape[0]
+        if x.ndim != 2 or x.shape[1] != self.L1.dim:
+            raise ValueError(f"L1_in must have shape [batch, {self.L1.dim}], got {tuple(x.shape)}")
+        if tuple(y.shape) != (B, self.L2.dim):
+            raise ValueError(f"L2_in must have shape [{B}, {self.L2.dim}], got {tuple(y.shape)}")
+        want = (self.config.weight_numel,) if self.config.shared_weights else (B, self.config.weight_numel)
+        if tuple(w.shape) != want:
+            raise ValueError(f"weights must have shape {want}, got {tuple(w.shape)}")
+        tdt = {np.float32: torch.float32, np.float64: torch.float64}[self.irrep_dtype]
+        if x.dtype != tdt or y.dtype != tdt or w.dtype != tdt:
+            raise TypeError(f"tensors must be {tdt}")
+
+    # ------------------------------------------------------ work / traffic models
+    def calculate_flops_forward(self, batch_size: int) -> dict:
+        """FLOP model of the reference (LoopUnrollTP.py:77-91)."""
+        tpp = self.config
+        if self.is_uvw:
+            dense = sum(2 * np.prod(ins.path_shape) * tpp.irreps_out[ins.i_out].ir.dim for ins in tpp.instructions)
+            return {"dense_contraction": int(dense) * batch_size, "total": int(dense) * batch_size}
+        cg = lin = 0
+        for ins in tpp.instructions:
+            l1, l2, l3 = tpp.irreps_in1[ins.i_in1].ir.l, tpp.irreps_in2[ins.i_in2].ir.l, tpp.irreps_out[ins.i_out].ir.l
+            nnz = int(np.count_nonzero(np.abs(wigner_3j(l1, l2, l3)) > 1e-14))
+            cg += nnz * ins.path_shape[0] * ins.path_shape[1]
+            lin += (2 * l3 + 1) * int(np.prod(ins.path_shape))
+        out = {"CG_decomposition": 3 * cg * batch_size, "linear_combination": lin * batch_size, "outer_products": 0}
+        out["total"] = sum(out.values())
+        return out
+
+    def calculate_flops_backward(self, batch_size: int) -> dict:
+        """reference: LoopUnrollTP.py:93-105."""
+        tpp = self.config
+        if self.is_uvw:
+            dense = sum(4 * np.prod(ins.path_shape) * tpp.irreps_out[ins.i_out].ir.dim for ins in tpp.instructions)
+            return {"dense_contraction": int(dense) * batch_size, "total": int(dense) * batch_size}
+        cg = 0
+        for ins in tpp.instructions:
+            l1, l2, l3 = tpp.irreps_in1[ins.i_in1].ir.l, tpp.irreps_in2[ins.i_in2].ir.l, tpp.irreps_out[ins.i_out].ir.l
+            nnz = int(np.count_nonzero(np.abs(wigner_3j(l1, l2, l3)) > 1e-14))
+            cg += nnz * ins.path_shape[0] * ins.path_shape[1]
+        return {"backward": 9 * cg * batch_size, "total": 9 * cg * batch_size}
+
+    def calculate_memory_streamed_forward(self, batch_size: int) -> dict:
+        """Minimum bytes moved (reference: benchmark/perf_metrics_utils.py:11-25)."""
+        s = np.dtype(self.irrep_dtype).itemsize
+        wn = self.config.weight_numel
+        w = wn if self.config.shared_weights else wn * batch_size
+        d = {"input": (self.L1.dim + self.L2.dim) * batch_size * s, "weights": w * s, "output": self.L3.dim * batch_size * s}
+        d["total"] = sum(d.values())
+        return d
+
+    def calculate_memory_streamed_backward(self, batch_size: int) -> dict:
+        """reference: benchmark/perf_metrics_utils.py:27-44."""
+        s = np.dtype(self.irrep_dtype).itemsize
+        wn = self.config.weight_numel
+        w = wn if self.config.shared_weights else wn * batch_size
+        d = {"input": (self.L1.dim + self.L2.dim + self.L3.dim) * batch_size * s + w * s,
+             "output": (self.L1.dim + self.L2.dim) * batch_size * s + w * s}
+        d["total"] = sum(d.values())
+        return d
+
+
+LoopUnrollTP = TensorProduct

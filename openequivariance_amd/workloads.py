@@ -1,0 +1,226 @@
+"""The benchmark workloads: problems, seeded synthetic inputs and algorithmic work.
+
+Each workload names the problem, generates its inputs on the host with
+``numpy.random.default_rng(seed)`` (seed 12345 + configuration index, the default seed of the
+reference's suites: openequivariance/benchmark/TestBenchmarkSuite.py:36), moves them to the
+GPU and exposes ``forward()`` / ``backward()`` closures that call the C-ABI entry points on
+preallocated outputs.  The byte model is the reference's own for the batch product
+(openequivariance/benchmark/perf_metrics_utils.py:11-44) and the compulsory traffic for the
+fused convolution (every tensor touched once).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Callable, Dict, Optional
+
+import numpy as np
+
+from .conv import TensorProductConv
+from .problem import ChannelwiseTPP, FullyConnectedTPProblem, TPProblem
+from .sh import random_unit_vectors, spherical_harmonics
+from .tensor_product import TensorProduct
+
+MACE = ("128x0e+128x1o+128x2e", "1x0e+1x1o+1x2e+1x3o", "128x0e+128x1o+128x2e+128x3o")
+NEQUIP = ("32x0e+32x1o+32x2e", "1x0e+1x1o+1x2e", "32x0e+32x1o+32x2e")
+LARGE = ("256x0e+256x1o+256x2e", "1x0e+1x1o+1x2e+1x3o", "256x0e+256x1o+256x2e")
+DENSE = ("64x0e+64x1o+64x2e", "1x0e+1x1o+1x2e", "64x0e+64x1o+64x2e")
+
+
+def _normal(rng, shape, dtype, scale=1.0, chunk=1 << 24):
+    """N(0, scale^2) samples drawn in chunks directly in the target precision."""
+    out = np.empty(shape, dtype=dtype)
+    flat = out.reshape(-1)
+    for s in range(0, flat.size, chunk):
+        e = min(flat.size, s + chunk)
+        flat[s:e] = rng.standard_normal(e - s, dtype=np.float32 if dtype == np.float32 else np.float64)
+    if scale != 1.0:
+        out *= dtype(scale)
+    return out
+
+
+@dataclass
+class Case:
+    op: object
+    tensors: Dict[str, object]
+    forward: Callable[[], None]
+    backward: Callable[[], None]
+    host: Dict[str, np.ndarray] = field(default_factory=dict)
+
+
+@dataclass
+class Workload:
+    name: str
+    description: str
+    kind: str                    # "tp" | "conv"
+    irreps: tuple
+    units: int                   # rows / edges per step
+    unit: str
+    bound: str                   # "hbm" | "mfma"
+    dtype: str
+    seed: int
+    config: dict
+    nodes: int = 0
+    deterministic: bool = False
+    sh_lmax: Optional[int] = None
+    mode: str = "uvu"
+    w_scale: float = 1.0
+    alg_bytes: Dict[str, int] = field(default_factory=dict)
+    alg_flops: Dict[str, int] = field(default_factory=dict)
+
+    # ------------------------------------------------------------------ problem
+    def problem(self) -> TPProblem:
+        dt = np.float32 if self.dtype == "f32" else np.float64
+        if self.mode == "uvw":
+            return FullyConnectedTPProblem(*self.irreps, shared_weights=True, internal_weights=False,
+                                           irrep_dtype=dt, weight_dtype=dt)
+        if self.irreps == ("1x2e", "1x3e", "1x2e"):
+            return TPProblem(*self.irreps, [(0, 0, 0, "uvu", True)], shared_weights=False, internal_weights=False)
+        return ChannelwiseTPP(*self.irreps, irrep_dtype=dt, weight_dtype=dt)
+
+    # ------------------------------------------------------------------- inputs
+    def graph(self, rng):
+        """rows (receivers), cols (senders)[, transpose_perm] for the convolution workloads."""
+        N, E = self.nodes, self.units
+        if self.name.startswith("large"):
+            deg = rng.poisson(40, N)
+            rows = np.repeat(np.arange(N, dtype=np.int64), deg)
+            cols = rng.integers(0, N, rows.size).astype(np.int64)
+        else:
+            rows = rng.integers(0, N, E).astype(np.int64)
+            cols = rng.integers(0, N, E).astype(np.int64)
+            clash = rows == cols
+            cols[clash] = (cols[clash] + 1 + rng.integers(0, N - 1, int(clash.sum()))) % N
+        tperm = None
+        if self.deterministic:
+            order = np.lexsort((cols, rows))
+            rows, cols = rows[order], cols[order]
+            tperm = np.lexsort((np.arange(rows.size), rows, cols)).astype(np.int64)
+        return rows, cols, tperm
+
+    def host_inputs(self, n_rows: Optional[int] = None):
+        """Seeded host arrays; ``n_rows`` truncates the batch for the CPU sample (TP only)."""
+        prob = self.problem()
+        dt = np.float32 if self.dtype == "f32" else np.float64
+        rng = np.random.default_rng(self.seed)
+        d1, d2, d3, wn = prob.irreps_in1.dim, prob.irreps_in2.dim, prob.irreps_out.dim, prob.weight_numel
+        h = {}
+        if self.kind == "tp":
+            n = self.units if n_rows is None else n_rows
+            h["X"] = _normal(rng, (n, d1), dt)
+            if self.sh_lmax is not None:
+                h["Y"] = spherical_harmonics(self.sh_lmax, random_unit_vectors(n, rng)).astype(dt)
+            else:
+                h["Y"] = rng.uniform(size=(n, d2)).astype(dt)
+            wshape = (wn,) if prob.shared_weights else (n, wn)
+            h["W"] = _normal(rng, wshape, dt, self.w_scale)
+            h["G"] = _normal(rng, (n, d3), dt)
+        else:
+            rows, cols, tperm = self.graph(rng)
+            E = rows.size
+            h["rows"], h["cols"] = rows, cols
+            if tperm is not None:
+                h["tperm"] = tperm
+            h["X"] = _normal(rng, (self.nodes, d1), dt)
+            h["Y"] = spherical_harmonics(self.sh_lmax, random_unit_vectors(E, rng)).astype(dt)
+            h["W"] = _normal(rng, (E, wn), dt)
+            h["G"] = _normal(rng, (self.nodes, d3), dt)
+        return prob, h
+
+    # -------------------------------------------------------------------- build
+    def build(self, device) -> Case:
+        import torch
+        prob, h = self.host_inputs()
+        t = {k: torch.from_numpy(v).to(device) for k, v in h.items()}
+        stream = torch.cuda.current_stream().cuda_stream
+        if self.kind == "tp":
+            op = TensorProduct(prob, torch_op=True)
+            n = h["X"].shape[0]
+            t["Z"] = torch.empty((n, prob.irreps_out.dim), dtype=t["X"].dtype, device=device)
+            t["Xg"], t["Yg"], t["Wg"] = (torch.empty_like(t[k]) for k in ("X", "Y", "W"))
+            p = {k: v.data_ptr() for k, v in t.items()}
+
+            def fwd():
+                op.forward_raw(n, p["X"], p["Y"], p["Z"], p["W"], stream)
+
+            def bwd():
+                op.backward_raw(n, p["X"], p["Xg"], p["Y"], p["Yg"], p["W"], p["Wg"], p["G"], stream)
+            self.units = n
+        else:
+            op = TensorProductConv(prob, torch_op=True, deterministic=self.deterministic)
+            E, N = h["rows"].size, self.nodes
+            self.units = E
+            self._fill_conv_bytes(prob, E, N)
+            t["Z"] = torch.zeros((N, prob.irreps_out.dim), dtype=t["X"].dtype, device=device)
+            t["Xg"] = torch.zeros_like(t["X"])
+            t["Yg"], t["Wg"] = torch.empty_like(t["Y"]), torch.empty_like(t["W"])
+            p = {k: v.data_ptr() for k, v in t.items()}
+            tp_ptr = p.get("tperm", 0)
+            ws = op.workspace_ptr(E, N)
+            det = self.deterministic
+
+            def fwd():
+                if not det:
+                    t["Z"].zero_()              # the atomic kernels accumulate: part of the operator's work
+                op.exec_conv_rawptrs(p["X"], p["Y"], p["W"], p["Z"], p["rows"], p["cols"], E, N, ws, tp_ptr, stream)
+
+            def bwd():
+                if not det:
+                    t["Xg"].zero_()
+                op.backward_rawptrs(p["X"], p["Xg"], p["Y"], p["Yg"], p["W"], p["Wg"], p["G"], p["rows"], p["cols"],
+                                    E, N, ws, tp_ptr, stream)
+        return Case(op, t, fwd, bwd, h)
+
+    def _fill_conv_bytes(self, prob, E, N):
+        s = 4 if self.dtype == "f32" else 8
+        d1, d2, d3, wn = prob.irreps_in1.dim, prob.irreps_in2.dim, prob.irreps_out.dim, prob.weight_numel
+        self.alg_bytes = {"forward": E * (d2 + wn) * s + N * (d1 + d3) * s + E * 16,
+                          "backward": 2 * E * (d2 + wn) * s + N * (2 * d1 + d3) * s + E * 24}
+        self.config["edges"] = int(E)
+
+
+def _tp_bytes(prob, n, s):
+    d1, d2, d3, wn = prob.irreps_in1.dim, prob.irreps_in2.dim, prob.irreps_out.dim, prob.weight_numel
+    w = wn if prob.shared_weights else wn * n
+    return {"forward": (n * (d1 + d2 + d3) + w) * s, "backward": (n * (2 * d1 + 2 * d2 + d3) + 2 * w) * s}
+
+
+def get(name: str) -> Workload:
+    if name == "mace_uvu":
+        w = Workload(name, "MACE-style per-edge uvu TP, 128x0e+128x1o+128x2e (x) SH(lmax 3) -> l3<=3, 17 paths, "
+                     "batch 50000, fp32, forward+backward", "tp", MACE, 50000, "edges/s", "hbm", "f32", 12346,
+                     {"batch": 50000, "paths": 17}, sh_lmax=3)
+        w.alg_bytes = _tp_bytes(w.problem(), w.units, 4)
+        return w
+    if name == "readme_uvu":
+        w = Workload(name, "single-path uvu TP 1x2e (x) 1x3e -> 1x2e, batch 1000, fp32", "tp",
+                     ("1x2e", "1x3e", "1x2e"), 1000, "rows/s", "hbm", "f32", 12345, {"batch": 1000, "paths": 1})
+        w.alg_bytes = _tp_bytes(w.problem(), w.units, 4)
+        return w
+    if name in ("nequip_conv_atomic", "nequip_conv_det"):
+        det = name.endswith("det")
+        return Workload(name, "NequIP-style fused uvu conv, 32x0e+32x1o+32x2e (x) SH(lmax 2), 11 paths, 5000 nodes, "
+                        "150000 edges, fp32, forward+backward, " + ("deterministic (receiver-sorted)" if det else "atomic (unsorted)"),
+                        "conv", NEQUIP, 150000, "edges/s", "hbm", "f32", 12347,
+                        {"nodes": 5000, "paths": 11, "deterministic": det}, nodes=5000, deterministic=det, sh_lmax=2)
+    if name in ("large_conv_det", "large_conv_atomic"):
+        det = name.endswith("det")
+        return Workload(name, "large fused uvu conv, 256x0e+256x1o+256x2e (x) SH(lmax 3) -> l3<=2, 13 paths, 20000 nodes, "
+                        "Poisson(40) in-degree (~800000 edges), fp32, forward+backward, "
+                        + ("deterministic" if det else "atomic"),
+                        "conv", LARGE, 800000, "edges/s", "hbm", "f32", 12349,
+                        {"nodes": 20000, "paths": 13, "deterministic": det}, nodes=20000, deterministic=det, sh_lmax=3)
+    if name in ("dense_uvw_f32", "dense_uvw_f64"):
+        dt = "f32" if name.endswith("f32") else "f64"
+        w = Workload(name, "dense uvw TP with shared weights, 64x0e+64x1o+64x2e (x) SH(lmax 2) -> 64x0e+64x1o+64x2e, "
+                     f"11 paths, batch 100000, {dt}, forward+backward", "tp", DENSE, 100000, "rows/s", "mfma", dt,
+                     12348, {"batch": 100000, "paths": 11}, sh_lmax=2, mode="uvw", w_scale=0.125)
+        prob = w.problem()
+        dense = sum(2 * int(np.prod(t.path_shape)) * prob.irreps_out[t.i_out].ir.dim for t in prob.instructions)
+        w.alg_flops = {"forward": dense * w.units, "backward": 2 * dense * w.units}
+        w.alg_bytes = _tp_bytes(prob, w.units, 4 if dt == "f32" else 8)
+        return w
+    raise KeyError(f"unknown workload {name!r}")
+
+
+ALL = ("readme_uvu", "mace_uvu", "nequip_conv_atomic", "nequip_conv_det", "dense_uvw_f32", "dense_uvw_f64",
+       "large_conv_det")

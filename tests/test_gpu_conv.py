@@ -1,0 +1,122 @@
+"""GPU parity of the fused convolution (atomic and deterministic) against the fp64 oracle."""
+import numpy as np
+import pytest
+
+import common
+from common import FP32_TOL, FP64_TOL, rel_err
+from oracle import tp as otp
+
+pytestmark = pytest.mark.gpu
+
+
+def _graph(nodes, nnz, seed, sort):
+    rows, cols = common.random_graph(nodes, nnz, seed)
+    tperm = None
+    if sort:
+        rows, cols, tperm, _ = otp.coord_graph(rows, cols)
+    return rows, cols, tperm
+
+
+def _run(prob, oprob, nodes, nnz, seed, deterministic, dtype=np.float32, sh_lmax=None, graph=None):
+    import torch
+    import openequivariance_amd as oeq
+    tol = FP32_TOL if dtype == np.float32 else FP64_TOL
+    rows, cols, tperm = graph if graph is not None else _graph(nodes, nnz, seed, deterministic)
+    nnz = len(rows)
+    X, Y, W, G = common.conv_inputs(prob, nodes, nnz, seed, dtype, sh_lmax)
+    conv = oeq.TensorProductConv(prob, torch_op=True, deterministic=deterministic)
+    dev = torch.device("cuda:0")
+    x, y, w = (torch.tensor(a, device=dev, requires_grad=True) for a in (X, Y, W))
+    idx = [torch.tensor(a, device=dev) for a in ((rows, cols, tperm) if deterministic else (rows, cols))]
+    z = conv.forward(x, y, w, *idx)
+    z.backward(torch.tensor(G, device=dev))
+    torch.cuda.synchronize()
+    Zr = otp.conv_forward(oprob, X, Y, W, rows, cols)
+    dXr, dYr, dWr = otp.conv_backward(oprob, X, Y, W, G, rows, cols)
+    errs = dict(Z=rel_err(z.detach().cpu().numpy(), Zr), dX=rel_err(x.grad.cpu().numpy(), dXr),
+                dY=rel_err(y.grad.cpu().numpy(), dYr), dW=rel_err(w.grad.cpu().numpy(), dWr))
+    print(f"nodes={nodes} nnz={nnz} det={deterministic} {errs}", flush=True)
+    for k, v in errs.items():
+        assert v <= tol, f"{k}: relative error {v:.3e} > {tol}"
+    return conv, (x, y, w, idx, z, torch.tensor(G, device=dev))
+
+
+@pytest.mark.parametrize("deterministic", [False, True])
+def test_nequip_conv(cuda, deterministic):
+    """BASELINE config 3 problem on a scaled-down random graph (no self loops)."""
+    prob, oprob = common.channelwise(common.NEQUIP)
+    _run(prob, oprob, 300, 9001, 31, deterministic, sh_lmax=2)
+
+
+@pytest.mark.parametrize("deterministic", [False, True])
+def test_large_conv(cuda, deterministic):
+    """BASELINE config 5 problem (mul 256 = four chunks) on a small graph."""
+    prob, oprob = common.channelwise(common.LARGE)
+    _run(prob, oprob, 40, 700, 32, deterministic, sh_lmax=3)
+
+
+@pytest.mark.parametrize("deterministic", [False, True])
+def test_readme_conv(cuda, deterministic):
+    prob, oprob = common.readme_problem()
+    _run(prob, oprob, 130, 1000, 33, deterministic)
+
+
+@pytest.mark.parametrize("deterministic", [False, True])
+def test_ragged_conv(cuda, deterministic):
+    irreps = ("5x0e+3x1o+70x2e", "1x0e+1x1o+1x2e", "5x0e+3x1o+70x2e+7x3o")
+    prob, oprob = common.channelwise(irreps)
+    _run(prob, oprob, 50, 333, 34, deterministic)
+
+
+def test_conv_fp64(cuda):
+    prob, oprob = common.channelwise(common.NEQUIP, dtype=np.float64)
+    _run(prob, oprob, 64, 900, 35, True, dtype=np.float64, sh_lmax=2)
+    _run(prob, oprob, 64, 900, 36, False, dtype=np.float64, sh_lmax=2)
+
+
+def test_isolated_nodes_and_asymmetric_graph(cuda):
+    """Nodes without incoming or outgoing edges get zero rows; the graph is not symmetric."""
+    prob, oprob = common.channelwise(common.NEQUIP)
+    nodes = 40
+    rng = np.random.default_rng(5)
+    rows = rng.integers(10, 20, 200).astype(np.int64)          # receivers only in [10, 20)
+    cols = rng.integers(25, 40, 200).astype(np.int64)          # senders only in [25, 40)
+    for det in (False, True):
+        r, c, t = rows, cols, None
+        if det:
+            r, c, t, _ = otp.coord_graph(rows, cols)
+        conv, (x, y, w, idx, z, g) = _run(prob, oprob, nodes, len(r), 37, det, graph=(r, c, t))
+        assert float(z.detach()[:10].abs().max()) == 0.0 and float(z.detach()[20:].abs().max()) == 0.0
+        assert float(x.grad[:25].abs().max()) == 0.0
+
+
+def test_no_edges(cuda):
+    import torch
+    import openequivariance_amd as oeq
+    prob, _ = common.channelwise(common.NEQUIP)
+    e = torch.zeros(0, dtype=torch.int64, device=cuda)
+    for det in (False, True):
+        conv = oeq.TensorProductConv(prob, torch_op=True, deterministic=det)
+        args = [torch.randn(7, 288, device=cuda), torch.zeros(0, 9, device=cuda), torch.zeros(0, 352, device=cuda), e, e]
+        if det:
+            args.append(e)
+        z = conv.forward(*args)
+        assert z.shape == (7, 1120) and float(z.abs().max()) == 0.0
+
+
+def test_deterministic_bit_reproducible(cuda):
+    """Five repeats of forward and backward give identical bits (reference protocol:
+    convolution/ConvolutionBase.py:229-247)."""
+    import torch
+    prob, oprob = common.channelwise(common.NEQUIP)
+    conv, (x, y, w, idx, z, g) = _run(prob, oprob, 500, 15000, 38, True, sh_lmax=2)
+    z0 = z.detach().clone()
+    grads0 = [t.grad.clone() for t in (x, y, w)]
+    for _ in range(5):
+        for t in (x, y, w):
+            t.grad = None
+        z1 = conv.forward(x, y, w, *idx)
+        z1.backward(g)
+        assert torch.equal(z1.detach(), z0)
+        for a, b in zip(grads0, (x.grad, y.grad, w.grad)):
+            assert torch.equal(a, b)
