@@ -22,6 +22,7 @@ import torch
 
 from . import runtime as rt
 from .codegen.uvu import UVUGenerator
+from .codegen.uvu_fast import UVUFastGenerator
 from .problem import TPProblem
 from .tensor_product import _make_steps, validate_problem
 from .weight_order import WeightReorder
@@ -97,6 +98,13 @@ class TensorProductConv:
         self.internal = rt.ConvImpl(code, _make_steps(fwd), _make_steps(bwd))
         self.workspace_buffer = None
         self.workspace_size = 0
+        self.internal_fast = None
+        kind = self.generator.kind
+        if UVUFastGenerator.eligible(config, kind):
+            self.generator_fast = UVUFastGenerator(config, kind)
+            ffwd, fbwd, _ = self.generator_fast.plan()
+            self.internal_fast = rt.ConvImpl(rt.compile_source(self.generator_fast.render()),
+                                             _make_steps(ffwd), _make_steps(fbwd))
         self._reorder = WeightReorder(config)
         self.reorder_weights_e3nn_to_oeq = self._reorder.e3nn_to_oeq
         self.reorder_weights_oeq_to_e3nn = self._reorder.oeq_to_e3nn
@@ -140,19 +148,26 @@ class TensorProductConv:
         if x.dtype != tdt or y.dtype != tdt or w.dtype != tdt:
             raise TypeError(f"tensors must be {tdt}")
 
+    def _pick(self, *ptrs):
+        if self.internal_fast is not None and all(int(p) % 16 == 0 for p in ptrs):
+            return self.internal_fast
+        return self.internal
+
     # ---------------------------------------------------------- raw entry points
     def exec_conv_rawptrs(self, L1_in, L2_in, weights, L3_out, rows, cols, nnz, node_count, workspace=0,
                           transpose_perm=0, stream=None):
         """reference: extension/convolution.hpp:121-147"""
-        self.internal.exec_conv_rawptrs(L1_in, L2_in, weights, L3_out, rows, cols, int(nnz), int(node_count),
-                                        workspace, transpose_perm, self._stream() if stream is None else stream)
+        impl = self._pick(L1_in, L2_in, weights, L3_out)
+        impl.exec_conv_rawptrs(L1_in, L2_in, weights, L3_out, rows, cols, int(nnz), int(node_count),
+                               workspace, transpose_perm, self._stream() if stream is None else stream)
 
     def backward_rawptrs(self, L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_grad, rows, cols, nnz,
                          node_count, workspace=0, transpose_perm=0, stream=None):
         """reference: extension/convolution.hpp:149-173"""
-        self.internal.backward_rawptrs(L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_grad, rows, cols,
-                                       int(nnz), int(node_count), workspace, transpose_perm,
-                                       self._stream() if stream is None else stream)
+        impl = self._pick(L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_grad)
+        impl.backward_rawptrs(L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_grad, rows, cols,
+                              int(nnz), int(node_count), workspace, transpose_perm,
+                              self._stream() if stream is None else stream)
 
     # ------------------------------------------------------------------ torch ops
     def _setup_torch_module(self) -> None:

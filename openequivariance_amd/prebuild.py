@@ -12,6 +12,7 @@ import numpy as np
 
 from . import runtime as rt
 from .codegen.uvu import UVUGenerator
+from .codegen.uvu_fast import UVUFastGenerator
 from .problem import ChannelwiseTPP, FullyConnectedTPProblem, TPProblem
 
 MACE = ("128x0e+128x1o+128x2e", "1x0e+1x1o+1x2e+1x3o", "128x0e+128x1o+128x2e+128x3o")
@@ -29,6 +30,9 @@ def benchmark_generators():
             ("nequip/conv_det", UVUGenerator(ChannelwiseTPP(*NEQUIP), "conv_det")),
             ("large/conv_atomic", UVUGenerator(ChannelwiseTPP(*LARGE), "conv_atomic")),
             ("large/conv_det", UVUGenerator(ChannelwiseTPP(*LARGE), "conv_det"))]
+    for name, g in list(gens):
+        if UVUFastGenerator.eligible(g.problem, g.kind):
+            gens.append((name + "/fast", UVUFastGenerator(g.problem, g.kind)))
     try:
         from .codegen.uvw import UVWGenerator
     except ImportError:

@@ -17,6 +17,7 @@ import torch
 
 from . import runtime as rt
 from .codegen.uvu import UVUGenerator
+from .codegen.uvu_fast import UVUFastGenerator
 from .problem import TPProblem
 from .weight_order import WeightReorder, is_identity
 from .wigner import wigner_3j
@@ -78,6 +79,14 @@ class TensorProduct(TensorProductBase):
         self.workspace_bytes = ws()
         self.internal = rt.TPImpl(code, _make_steps(fwd), _make_steps(bwd))
         self._workspace = None
+        # bandwidth-oriented schedule for 16-byte granular problems; used whenever the tensors
+        # handed in are 16-byte aligned, the generic kernels otherwise
+        self.internal_fast = None
+        if not self.is_uvw and UVUFastGenerator.eligible(config, "tp"):
+            self.generator_fast = UVUFastGenerator(config, "tp")
+            ffwd, fbwd, _ = self.generator_fast.plan()
+            self.internal_fast = rt.TPImpl(rt.compile_source(self.generator_fast.render()),
+                                           _make_steps(ffwd), _make_steps(fbwd))
 
         self._reorder = WeightReorder(config)
         if is_identity(self._reorder.perm):
@@ -105,16 +114,23 @@ class TensorProduct(TensorProductBase):
     def _stream() -> int:
         return torch.cuda.current_stream().cuda_stream
 
+    def _pick(self, *ptrs):
+        if self.internal_fast is not None and all(int(p) % 16 == 0 for p in ptrs):
+            return self.internal_fast
+        return self.internal
+
     def forward_raw(self, batch, L1_in, L2_in, L3_out, weights, stream=None) -> None:
         """Device pointers as integers (reference: TensorProductBase.py:41-49)."""
-        self.internal.exec_tensor_product(int(batch), L1_in, L2_in, L3_out, weights, self._workspace_ptr(),
-                                          self._stream() if stream is None else stream)
+        impl = self._pick(L1_in, L2_in, L3_out, weights)
+        impl.exec_tensor_product(int(batch), L1_in, L2_in, L3_out, weights, self._workspace_ptr(),
+                                 self._stream() if stream is None else stream)
 
     def backward_raw(self, batch_size, L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_grad,
                      stream=None) -> None:
         """reference: TensorProductBase.py:51-61."""
-        self.internal.backward(int(batch_size), L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_grad,
-                               self._workspace_ptr(), self._stream() if stream is None else stream)
+        impl = self._pick(L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_grad)
+        impl.backward(int(batch_size), L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_grad,
+                      self._workspace_ptr(), self._stream() if stream is None else stream)
 
     # ------------------------------------------------- numpy entry points (tests)
     def forward_cpu(self, L1_in, L2_in, L3_out, weights) -> None:
