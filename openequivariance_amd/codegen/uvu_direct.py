@@ -1,0 +1,367 @@
+"""Register-direct schedule for uvu kernels: no LDS, no transposition.
+
+In the ``mul x irrep`` layout element ``(u, m)`` sits at ``u * (2l+1) + m``, so with lane <-> channel
+``u`` every lane owns a CONTIGUOUS record of ``2l+1`` words in X, Z, dZ and dX.  A lane therefore
+reads and writes its records straight from/to global memory with per-lane vector accesses
+(dword x1 / x3 / x4+x1 / x4+x3, dword aligned); consecutive lanes touch consecutive records, so a
+wavefront still covers a contiguous span and every cache line it touches is fully used - the L1
+merges the partial touches of the two instructions of a record.  Compared with staging through
+LDS this removes all LDS traffic and all intra-wave synchronisation, frees the LDS limit on
+occupancy, and lets the compiler issue every load of a work item up front (there is no fence in
+the way), which is what keeps HBM busy.
+
+It needs nothing from the problem's sizes (any multiplicity, any alignment), so it serves as
+the general schedule for the batch product and the atomic convolution.
+
+Stores are the exception where measurement favours a detour through LDS: a record store covers
+only part of each cache line per instruction, and on MI355X streams of such partial-line writes
+(Z is 73 % of the forward traffic) run about 20 % slower than full-line writes, and strided
+atomics are several times slower than coalesced ones.  So the big outputs (Z; dX when it is
+scattered with atomics) are transposed through a 2 KB LDS slot and leave as full 16-byte-per-lane
+vector stores or as coalesced atomics; loads stay register-direct.
+"""
+from __future__ import annotations
+
+from ..problem import TPProblem
+from .common import WAVE, Emitter
+from .uvu import Block, Path, UVUGenerator
+
+
+class UVUDirectGenerator(UVUGenerator):
+
+    def __init__(self, problem: TPProblem, kind: str = "tp", waves_per_eu: int = 0, vector_stores: bool = True):
+        super().__init__(problem, kind)
+        if kind == "conv_det" or self.shared:
+            raise NotImplementedError("direct schedule: batch product with per-row weights and atomic convolution")
+        self.waves_per_eu = waves_per_eu
+        # False: outputs are written with dword-aligned record stores only (for callers whose
+        # output tensor is not 16-byte aligned)
+        self.vector_stores = vector_stores
+        self.VW = 16 // self.itemsize
+        stage = [WAVE * b.D for b in list(self.out) + list(self.in1) if b.D > 1 and b.dim]
+        self.lds_elems = max(stage) if stage else 0
+        self.ZB = 0
+        self.unroll_bwd_chunks = 1
+        # one row per wavefront: the row index is wave-uniform and an out-of-range wavefront exits
+        self.uniform_rows = (self.R == 1)
+        self._cur_c = None
+
+    def describe(self) -> str:
+        return super().describe().replace(f"lds={0}B", "lds=0B") + " direct"
+
+    # ------------------------------------------------------------------ pieces
+    def emit_lane_direct(self, E: Emitter, lds: bool = False) -> None:
+        E("const int lane = threadIdx.x;")
+        E(f"const int sub = lane >> {self.LOGP};")
+        E(f"const int ul = lane & {self.P - 1};")
+        if lds and self.lds_elems:
+            E(f"__shared__ __attribute__((aligned(16))) T lds[{self.lds_elems}];")
+
+    # ---- stores through an LDS slot ---------------------------------------------
+    def dense(self, blk: Block) -> int:
+        """Channels of ``blk`` held per sub-row in the (gap-free) LDS slot."""
+        return blk.mul if self.NCH == 1 else WAVE
+
+    def vector_ok(self, blk: Block, rowdim: int) -> bool:
+        """Rows of this block can be written as aligned 16-byte vectors."""
+        vw = self.VW
+        if not self.vector_stores or rowdim % vw or blk.off % vw:
+            return False
+        if self.NCH > 1:
+            return blk.mul % WAVE == 0
+        return (blk.mul * blk.D) % vw == 0
+
+    def emit_slot_out(self, E: Emitter, blk: Block, names, ptr: str, rowdim: int, row_of, op: str) -> None:
+        """registers -> LDS slot (transposed) -> global rows: 16-byte vectors per lane (op "store",
+        needs vector_ok and 16-byte aligned tensors) or coalesced scalar atomics (op "atomic")."""
+        dn, D, base = self.dense(blk), blk.D, self.ZB
+        E("oeq_sync();")
+        E(f"if ({self.act(blk)}) {{ " + " ".join(f"lds[{base} + (sub * {dn} + ul) * {D} + {k}] = {n};" for k, n in enumerate(names)) + " }")
+        E("oeq_sync();")
+        coff = f" + c * {WAVE * D}" if self.NCH > 1 else ""
+        cnt = dn * D                       # elements per sub-row in the slot
+        if op == "store":
+            per_row, unit, total_it = cnt // self.VW, self.VW, None
+        else:
+            per_row, unit = cnt, 1
+        total = self.R * per_row
+        # a partly filled last chunk holds fewer valid channels than the slot has room for
+        limit = f"{total}" if (self.NCH == 1 or self.full(blk)) else f"{self.chunk_count(blk)} * {D}"
+        for it in range((total + WAVE - 1) // WAVE):
+            E(f"{{ const int q = lane + {it * 64};")
+            if self.R == 1:
+                row, ok = row_of("0")
+                guard = f"q < {limit}" + ("" if ok == "true" else f" && {ok}")
+                tgt = f"{ptr} + (u64){row} * {rowdim} + {blk.off}{coff} + q * {unit}"
+            else:
+                E(f"  const int r = q / {per_row};")
+                E(f"  const int rr = r < {self.R} ? r : 0;")
+                row, ok = row_of("rr")
+                E(f"  const u64 grow = (u64){row};")
+                E(f"  const bool ok = {ok};")
+                guard = f"q < {total} && ok"
+                tgt = f"{ptr} + grow * {rowdim} + {blk.off} + (q - r * {per_row}) * {unit}"
+            if op == "store":
+                E(f"  if ({guard}) *(VT*)({tgt}) = *(const VT*)(lds + {base} + q * {unit}); }}")
+            else:
+                E(f"  if ({guard}) oeq_atomic_add({tgt}, lds[{base} + q]); }}")
+
+    def emit_block_store(self, E: Emitter, blk: Block, names, ptr: str, rowdim: int, own_row: str, row_of,
+                         op: str, via_lds: bool) -> None:
+        """One block of one chunk: registers -> memory, by the cheapest correct route."""
+        if blk.D == 1 or not via_lds or (op == "store" and not self.vector_ok(blk, rowdim)):
+            self.emit_record_store(E, names, f"{ptr} + (u64){own_row} * {rowdim} + {blk.off} + u * {blk.D}",
+                                   self.act(blk), op)
+        else:
+            self.emit_slot_out(E, blk, names, ptr, rowdim, row_of, op)
+
+    def uexpr(self, c) -> str:
+        return f"({c * self.P} + ul)" if isinstance(c, int) else f"(c * {self.P} + ul)"
+
+    def uclamp(self, blk: Block, c) -> str:
+        """Channel index of this lane in chunk c, clamped into the block."""
+        return self.uexpr(c) if self.full(blk) else f"min({self.uexpr(c)}, {blk.mul - 1})"
+
+    def act(self, blk: Block) -> str:
+        rv = "true" if self.uniform_rows else "rv"
+        if self.full(blk):
+            return rv
+        return f"(u < {blk.mul})" if self.uniform_rows else f"(rv && u < {blk.mul})"
+
+    def act_c(self, blk: Block, c) -> str:
+        rv = "true" if self.uniform_rows else "rv"
+        if self.full(blk):
+            return rv
+        return f"({self.uexpr(c)} < {blk.mul})" if self.uniform_rows else f"(rv && {self.uexpr(c)} < {blk.mul})"
+
+    def emit_record_load(self, E: Emitter, names, ptr: str, act: str, zero: bool = False) -> None:
+        """Unconditional loads (the caller passes an address that is valid for every lane: idle
+        lanes are clamped onto a valid row/channel).  Branch-free loads are what lets the compiler
+        merge them into x3/x4 accesses and hoist them.  With ``zero`` idle lanes get 0 instead of
+        the clamped lane's data (needed where the value feeds a cross-lane sum)."""
+        if zero and act != "true":
+            E("T " + ", ".join(names) + ";")
+            E(f"{{ const T* __restrict__ p_ = {ptr}; " + " ".join(f"{n} = p_[{k}];" for k, n in enumerate(names)) + " }")
+            E(f"if (!({act})) {{ " + " ".join(f"{n} = (T)0;" for n in names) + " }")
+        else:
+            E(f"const T* __restrict__ p_{names[0]} = {ptr};")
+            E("const T " + ", ".join(f"{n} = p_{names[0]}[{k}]" for k, n in enumerate(names)) + ";")
+
+    def emit_record_store(self, E: Emitter, names, ptr: str, act: str, op: str = "store") -> None:
+        if op == "atomic":
+            E(f"if ({act}) {{ T* __restrict__ p_ = {ptr}; " + " ".join(f"oeq_atomic_add(p_ + {k}, {n});" for k, n in enumerate(names)) + " }")
+        else:
+            E(f"if ({act}) {{ T* __restrict__ p_ = {ptr}; " + " ".join(f"p_[{k}] = {n};" for k, n in enumerate(names)) + " }")
+
+    def emit_y_load_direct(self, E: Emitter) -> None:
+        for f in self.used_y:
+            E(f"const T y{f} = Yr[{f}];")
+
+    def emit_weights(self, E: Emitter, p: Path, wptr: str) -> None:
+        for v in range(p.mv):
+            E(f"const T w{p.t}_{v} = W{self._cur_c}_{p.t}_{v};")
+
+    def emit_weight_preload(self, E: Emitter, c, wptr: str = "Wr") -> None:
+        tag = c if isinstance(c, int) else "c"
+        ue = self.uexpr(c)
+        for p in self.paths:
+            for v in range(p.mv):
+                E(f"const T W{tag}_{p.t}_{v} = {wptr}[{self.widx(p, self.uclamp(p.a, c), v)}];")
+
+    def emit_x_preload(self, E: Emitter, c, xrow: str) -> None:
+        tag = c if isinstance(c, int) else "c"
+        ue = self.uexpr(c)
+        for i in self.used_in1:
+            a = self.in1[i]
+            self.emit_record_load(E, [f"X{tag}_{i}_{m}" for m in range(a.D)],
+                                  f"X + (u64){xrow} * {self.D1} + {a.off} + {self.uclamp(a, c)} * {a.D}",
+                                  self.act_c(a, c))
+
+    def emit_x_alias(self, E: Emitter, tag) -> None:
+        for i in self.used_in1:
+            for m in range(self.in1[i].D):
+                E(f"const T x{i}_{m} = X{tag}_{i}_{m};")
+
+    def _rows(self, E: Emitter, backward: bool = False):
+        """Emit the row prologue; returns (x row, z row, per-row stream index)."""
+        if self.kind == "tp":
+            if self.uniform_rows:
+                E("const u64 row = blockIdx.x;")          # wave-uniform; the grid has exactly n workgroups
+                E("if (row >= n) return;")
+                E("const bool rv = true; (void)rv;")
+                rc = "row"
+            else:
+                E(f"const u64 row = (u64)blockIdx.x * {self.R} + sub;")
+                E("const bool rv = row < n;")
+                E("const u64 rowc = rv ? row : n - 1;")    # idle lanes read the last row and store nothing
+                rc = "rowc"
+            E(f"const T* __restrict__ Yr = Y + {rc} * {self.D2};")
+            E(f"const T* __restrict__ Wr = W + {rc} * {self.WN};")
+            if self.uniform_rows:
+                self.xrow_of = self.zrow_of = (lambda r: ("row", "true"))
+            else:
+                base = f"(u64)blockIdx.x * {self.R}"
+                self.xrow_of = self.zrow_of = (lambda r: (f"({base} + {r})", f"({base} + {r} < n)"))
+            return rc, rc, "row"
+        # convolution: an edge is idle when it is out of range or names a node that does not exist;
+        # idle lanes read edge/node 0 (callers never launch with zero nodes) and store nothing
+        if self.uniform_rows:
+            E("const u64 e = blockIdx.x;")
+            E("if (e >= nnz) return;")
+            E("const u64 ec = e;")
+            E("const i64 snd = cols[e], rcv = rows[e];")
+        else:
+            E(f"const u64 e = (u64)blockIdx.x * {self.R} + sub;")
+            E("const u64 ec = e < nnz ? e : nnz - 1;")
+            E("const i64 snd = cols[ec], rcv = rows[ec];")
+        E("const bool ev = (snd >= 0 && snd < (i64)node_count && rcv >= 0 && rcv < (i64)node_count);")
+        if self.uniform_rows:
+            E("const bool rv = true; (void)rv;")
+            E("if (!ev) {")                                 # whole wavefront: define dY / dW rows, then leave
+            if backward:
+                E(f"    for (int q = lane; q < {self.WN}; q += 64) Wg[e * {self.WN} + q] = (T)0;")
+                E(f"    for (int q = lane; q < {self.D2}; q += 64) Yg[e * {self.D2} + q] = (T)0;")
+            E("    return;")
+            E("}")
+            E("const u64 sndc = (u64)snd, rcvc = (u64)rcv;")
+        else:
+            E("const bool rv = ev && e < nnz;")
+            E("const u64 sndc = rv ? (u64)snd : 0, rcvc = rv ? (u64)rcv : 0;")
+        E(f"const T* __restrict__ Yr = Y + ec * {self.D2};")
+        E(f"const T* __restrict__ Wr = W + ec * {self.WN};")
+        if self.uniform_rows:
+            self.xrow_of = (lambda r: ("sndc", "true"))
+            self.zrow_of = (lambda r: ("rcvc", "true"))
+        else:
+            E("const int xsrc = rv ? (int)snd : -1;")
+            E("const int zdst = rv ? (int)rcv : -1;")
+            self.xrow_of = self._shfl_row("xsrc")
+            self.zrow_of = self._shfl_row("zdst")
+        return "sndc", "rcvc", "e"
+
+    # =============================================================== forward
+    def direct_forward_body(self) -> str:
+        E = Emitter()
+        atomic = (self.kind == "conv_atomic")
+        self.emit_lane_direct(E, lds=True)
+        xrow, zrow, _ = self._rows(E)
+        self.emit_y_load_direct(E)
+        for c in range(self.NCH):
+            self.emit_x_preload(E, c, xrow)
+            self.emit_weight_preload(E, c)
+        for c in range(self.NCH):
+            self._cur_c = c
+            E("{")
+            E.level += 1
+            E(f"const int c = {c}; (void)c;")
+            E(f"const int u = {c * self.P} + ul;")
+            self.emit_x_alias(E, c)
+            for o in self.out:
+                if o.dim == 0:
+                    continue
+                E("{")
+                E.level += 1
+                if o.idx in self.used_out:
+                    self.emit_forward_block(E, o, "Wr")
+                    self.emit_block_store(E, o, [f"z{k}" for k in range(o.D)], "Z", self.D3, zrow, self.zrow_of,
+                                          "atomic" if atomic else "store", via_lds=True)
+                elif not atomic:
+                    self.emit_record_store(E, ["(T)0"] * o.D, f"Z + (u64){zrow} * {self.D3} + {o.off} + u * {o.D}",
+                                           self.act(o))
+                E.level -= 1
+                E("}")
+            E.level -= 1
+            E("}")
+        return E.text()
+
+    # ============================================================== backward
+    def direct_backward_body(self) -> str:
+        E = Emitter()
+        atomic = (self.kind == "conv_atomic")
+        self.emit_lane_direct(E, lds=atomic)
+        xrow, zrow, srow = self._rows(E, backward=True)
+        E(f"T* __restrict__ Wgr = Wg + {srow} * {self.WN};")
+        self.emit_y_load_direct(E)
+        for f in self.used_y:
+            E(f"T dy{f} = (T)0;")
+
+        def chunk(E, c):
+            tag = c if isinstance(c, int) else "c"
+            self._cur_c = tag
+            self.emit_x_preload(E, c, xrow)
+            self.emit_weight_preload(E, c)
+            for oi in self.used_out:
+                o = self.out[oi]
+                self.emit_record_load(E, [f"G{oi}_{k}" for k in range(o.D)],
+                                      f"G + (u64){zrow} * {self.D3} + {o.off} + {self.uclamp(o, c)} * {o.D}",
+                                      self.act(o), zero=True)
+            self.emit_x_alias(E, tag)
+            for i in self.used_in1:
+                for m in range(self.in1[i].D):
+                    E(f"T dx{i}_{m} = (T)0;")
+            for oi in self.used_out:
+                o = self.out[oi]
+                E("{")
+                E.level += 1
+                for k in range(o.D):
+                    E(f"const T g{k} = G{oi}_{k};")
+
+                def sink(E, p, v, expr):
+                    E(f"  if ({self.act(p.a)}) Wgr[{self.widx(p, 'u', v)}] = {expr};")
+                self.emit_backward_block(E, o, "Wr", sink)
+                E.level -= 1
+                E("}")
+            for a in self.in1:
+                if a.dim == 0:
+                    continue
+                if a.idx in self.used_in1:
+                    self.emit_block_store(E, a, [f"dx{a.idx}_{m}" for m in range(a.D)], "Xg", self.D1, xrow,
+                                          self.xrow_of, "atomic" if atomic else "store", via_lds=atomic)
+                elif not atomic:
+                    self.emit_record_store(E, ["(T)0"] * a.D, f"Xg + (u64){xrow} * {self.D1} + {a.off} + u * {a.D}",
+                                           self.act(a))
+
+        if self.NCH <= self.unroll_bwd_chunks:
+            for c in range(self.NCH):
+                E("{")
+                E.level += 1
+                E(f"const int c = {c}; (void)c;")
+                E(f"const int u = {c * self.P} + ul;")
+                chunk(E, c)
+                E.level -= 1
+                E("}")
+        else:
+            E("#pragma unroll 1")
+            E(f"for (int c = 0; c < {self.NCH}; ++c) {{")
+            E.level += 1
+            E(f"const int u = c * {self.P} + ul;")
+            chunk(E, "c")
+            E.level -= 1
+            E("}")
+        self.emit_dy_reduce(E)
+        if self.kind == "tp":
+            E("if (rv && ul == 0) {")
+            E(f"    T* __restrict__ Ygr = Yg + row * {self.D2};")
+        else:
+            E("if (e < nnz && ul == 0) {")
+            E(f"    T* __restrict__ Ygr = Yg + e * {self.D2};")
+        for f in range(self.D2):
+            E(f"    Ygr[{f}] = " + (f"dy{f};" if f in self.used_y else "(T)0;"))
+        E("}")
+        if self.kind != "tp":
+            E("if (e < nnz && !rv) {")
+            E(f"    for (int q = ul; q < {self.WN}; q += {self.P}) Wgr[q] = (T)0;")
+            E("}")
+        return E.text()
+
+    def tp_forward_body(self) -> str:
+        return self.direct_forward_body()
+
+    def tp_backward_body(self) -> str:
+        return self.direct_backward_body()
+
+    def conv_atomic_forward_body(self) -> str:
+        return self.direct_forward_body()
+
+    def conv_atomic_backward_body(self) -> str:
+        return self.direct_backward_body()

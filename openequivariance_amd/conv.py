@@ -22,9 +22,10 @@ import torch
 
 from . import runtime as rt
 from .codegen.uvu import UVUGenerator
+from .codegen.uvu_direct import UVUDirectGenerator
 from .codegen.uvu_fast import UVUFastGenerator
 from .problem import TPProblem
-from .tensor_product import _make_steps, validate_problem
+from .tensor_product import _make_steps, schedule, validate_problem
 from .weight_order import WeightReorder
 from .wigner import wigner_3j
 
@@ -91,7 +92,10 @@ class TensorProductConv:
         if mode != "uvu":
             raise NotImplementedError("TensorProductConv supports uvu problems")
 
-        self.generator = UVUGenerator(config, "conv_det" if deterministic else "conv_atomic")
+        if deterministic or schedule() == "lds":
+            self.generator = UVUGenerator(config, "conv_det" if deterministic else "conv_atomic")
+        else:
+            self.generator = UVUDirectGenerator(config, "conv_atomic")
         self.jit_kernel = self.generator.render()
         code = rt.compile_source(self.jit_kernel)
         fwd, bwd, self._ws_bytes = self.generator.plan()
@@ -100,7 +104,7 @@ class TensorProductConv:
         self.workspace_size = 0
         self.internal_fast = None
         kind = self.generator.kind
-        if UVUFastGenerator.eligible(config, kind):
+        if schedule() == "lds" and UVUFastGenerator.eligible(config, kind):
             self.generator_fast = UVUFastGenerator(config, kind)
             ffwd, fbwd, _ = self.generator_fast.plan()
             self.internal_fast = rt.ConvImpl(rt.compile_source(self.generator_fast.render()),
@@ -149,6 +153,8 @@ class TensorProductConv:
             raise TypeError(f"tensors must be {tdt}")
 
     def _pick(self, *ptrs):
+        # (the register-direct atomic kernels have no alignment requirement: they store with
+        # scalar atomics and dword stores only)
         if self.internal_fast is not None and all(int(p) % 16 == 0 for p in ptrs):
             return self.internal_fast
         return self.internal

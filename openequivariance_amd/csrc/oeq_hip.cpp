@@ -266,6 +266,7 @@ int oeq_conv_forward(oeq_conv* c, const void* L1, const void* L2, const void* W,
                      void* workspace, const void* tperm, void* stream) {
     if (!c) return fail("null handle");
     if (c->fwd.empty()) return fail("this operator was built without a forward plan");
+    if (nnz > 0 && node_count == 0) return fail("convolution called with %llu edges but no nodes", (unsigned long long)nnz);
     void* args[] = {&L1, &L2, &W, &L3, &rows, &cols, &nnz, &node_count, &workspace, &tperm};
     for (auto& s : c->fwd)
         if (launch(s, nnz, node_count, args, stream)) return 1;
@@ -277,6 +278,7 @@ int oeq_conv_backward(oeq_conv* c, const void* L1, void* L1g, const void* L2, vo
                       uint64_t node_count, void* workspace, const void* tperm, void* stream) {
     if (!c) return fail("null handle");
     if (c->bwd.empty()) return fail("this operator was built without a backward plan");
+    if (nnz > 0 && node_count == 0) return fail("convolution called with %llu edges but no nodes", (unsigned long long)nnz);
     void* args[] = {&L1, &L1g, &L2, &L2g, &W, &Wg, &L3g, &rows, &cols, &nnz, &node_count, &workspace, &tperm};
     for (auto& s : c->bwd)
         if (launch(s, nnz, node_count, args, stream)) return 1;

@@ -12,6 +12,7 @@ import numpy as np
 
 from . import runtime as rt
 from .codegen.uvu import UVUGenerator
+from .codegen.uvu_direct import UVUDirectGenerator
 from .codegen.uvu_fast import UVUFastGenerator
 from .problem import ChannelwiseTPP, FullyConnectedTPProblem, TPProblem
 
@@ -31,8 +32,8 @@ def benchmark_generators():
             ("large/conv_atomic", UVUGenerator(ChannelwiseTPP(*LARGE), "conv_atomic")),
             ("large/conv_det", UVUGenerator(ChannelwiseTPP(*LARGE), "conv_det"))]
     for name, g in list(gens):
-        if UVUFastGenerator.eligible(g.problem, g.kind):
-            gens.append((name + "/fast", UVUFastGenerator(g.problem, g.kind)))
+        if g.kind != "conv_det" and not g.shared:
+            gens.append((name + "/direct", UVUDirectGenerator(g.problem, g.kind)))
     try:
         from .codegen.uvw import UVWGenerator
     except ImportError:

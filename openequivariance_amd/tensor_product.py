@@ -17,6 +17,7 @@ import torch
 
 from . import runtime as rt
 from .codegen.uvu import UVUGenerator
+from .codegen.uvu_direct import UVUDirectGenerator
 from .codegen.uvu_fast import UVUFastGenerator
 from .problem import TPProblem
 from .weight_order import WeightReorder, is_identity
@@ -26,6 +27,13 @@ from .wigner import wigner_3j
 def _make_steps(descs):
     return [rt.Step.make(d["kernel"], d["num_threads"], d.get("smem", 0), d.get("grid_kind", rt.GRID_PER_ROW),
                          d.get("work_per_block", 1), d.get("num_blocks", 0), d.get("grid_y", 1)) for d in descs]
+
+
+def schedule() -> str:
+    """Kernel schedule for uvu problems with per-row weights: "direct" (registers only, default)
+    or "lds" (rows staged through LDS); the environment variable exists for A/B measurements."""
+    import os
+    return os.environ.get("OEQ_AMD_SCHEDULE", "direct")
 
 
 def validate_problem(config: TPProblem) -> str:
@@ -71,8 +79,10 @@ class TensorProduct(TensorProductBase):
         if self.is_uvw:
             from .codegen.uvw import UVWGenerator
             self.generator = UVWGenerator(config)
-        else:
+        elif config.shared_weights or schedule() == "lds":
             self.generator = UVUGenerator(config, "tp")
+        else:
+            self.generator = UVUDirectGenerator(config, "tp")
         self.jit_kernel = self.generator.render()
         code = rt.compile_source(self.jit_kernel)
         fwd, bwd, ws = self.generator.plan()
@@ -82,7 +92,8 @@ class TensorProduct(TensorProductBase):
         # bandwidth-oriented schedule for 16-byte granular problems; used whenever the tensors
         # handed in are 16-byte aligned, the generic kernels otherwise
         self.internal_fast = None
-        if not self.is_uvw and UVUFastGenerator.eligible(config, "tp"):
+        self._internal_unaligned = None
+        if not self.is_uvw and schedule() == "lds" and UVUFastGenerator.eligible(config, "tp"):
             self.generator_fast = UVUFastGenerator(config, "tp")
             ffwd, fbwd, _ = self.generator_fast.plan()
             self.internal_fast = rt.TPImpl(rt.compile_source(self.generator_fast.render()),
@@ -115,8 +126,16 @@ class TensorProduct(TensorProductBase):
         return torch.cuda.current_stream().cuda_stream
 
     def _pick(self, *ptrs):
-        if self.internal_fast is not None and all(int(p) % 16 == 0 for p in ptrs):
+        aligned = all(int(p) % 16 == 0 for p in ptrs)
+        if self.internal_fast is not None and aligned:
             return self.internal_fast
+        if not aligned and isinstance(self.generator, UVUDirectGenerator):
+            # rare: a caller-supplied tensor that is not 16-byte aligned -> kernels without vector stores
+            if self._internal_unaligned is None:
+                g = UVUDirectGenerator(self.config, "tp", vector_stores=False)
+                fwd, bwd, _ = g.plan()
+                self._internal_unaligned = rt.TPImpl(rt.compile_source(g.render()), _make_steps(fwd), _make_steps(bwd))
+            return self._internal_unaligned
         return self.internal
 
     def forward_raw(self, batch, L1_in, L2_in, L3_out, weights, stream=None) -> None:
