@@ -1,0 +1,472 @@
+"""Generator of gfx950 HIP source for dense ("uvw") tensor products with shared weights.
+
+    Z[b, w, k] = sum_t sum_u  W_t[u, w] * T_t[b, u, k],    T_t[b, u, k] = c_t sum_ij C_ijk x[b, u, i] y[b, j]
+
+is a genuine dense contraction over the multiplicity ``u`` and runs on the matrix cores:
+``v_mfma_f32_16x16x4_f32`` / ``v_mfma_f64_16x16x4_f64`` (one 16x16 accumulator tile, K = 4 per
+instruction), with the sparse Clebsch-Gordan part evaluated on the vector ALU directly into
+MFMA operand registers (reference: the register-tiled CUDA-core matmul of
+openequivariance/templates/wmm.cuh:1-88 called from loop_unroll_tp.cuh:74-78, :184, :209).
+
+Tiling (lane = 16 * g + c, g = lane / 16, c = lane % 16; a batch tile is 16 rows):
+
+* forward, one wavefront per tile:  A[i=c][k=g] = T[b=c, u=4s+g] (VALU),  B[k=g][j=c] = W[u=4s+g][w]
+  from a pre-packed copy of W, accumulators = the 16 x mul_out tile of one output block; each lane
+  ends up with contiguous runs of Z, so Z is stored with vector stores straight from registers.
+* backward dX/dY, four wavefronts per tile (one 16-channel u-subtile each):
+  dT^T[u, b] = sum_w W[u][w] dZ[b][w]:  A = W (pre-packed), B = dZ held in registers for the whole
+  output block, then the CG transpose on the VALU accumulates dX (registers) and dY.
+* backward dW, four wavefronts per workgroup, persistent over batch tiles:
+  dW[u, w] = sum_{b,k} T[b,u,k] dZ[b,w,k]:  A = T (VALU), B = dZ, accumulators = this wavefront's
+  u-subtile of every path; per-workgroup partial sums go to the workspace and a last kernel adds
+  them in workgroup order (reproducible; no floating-point atomics).
+
+Nothing is staged in LDS (only the 4-wave dY sum uses 2.3 KB): operands are per-lane records of
+the ``mul x irrep`` layout, loaded straight from global memory / L2.
+
+Scope of this generator: shared weights and multiplicity 1 on the second operand (the case the
+benchmarks and MACE/NequIP-style models use).  Other uvw problems raise NotImplementedError.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Tuple
+
+import numpy as np
+
+from ..problem import TPProblem
+from ..wigner import wigner_3j
+from .common import Emitter, jinja_env, literal
+from .uvu import Block, _blocks
+
+
+def _ceil(a: int, b: int) -> int:
+    return (a + b - 1) // b
+
+
+@dataclass
+class WPath:
+    t: int
+    a: Block
+    b: Block
+    o: Block
+    coeff: float
+    woff: int                       # offset of this path's weights in the external vector
+    pairs: Dict[Tuple[int, int], List[Tuple[int, float]]] = field(default_factory=dict)
+    wb: int = 0                     # offset (elements) of the forward-packed copy
+    wa: int = 0                     # offset of the backward-packed copy
+
+    @property
+    def mu(self) -> int:
+        return self.a.mul
+
+    @property
+    def mw(self) -> int:
+        return self.o.mul
+
+    @property
+    def SU(self) -> int:            # K steps over u (forward)
+        return _ceil(self.mu, 4)
+
+    @property
+    def SW(self) -> int:            # K steps over w (backward dX)
+        return _ceil(self.mw, 4)
+
+    @property
+    def NTU(self) -> int:           # 16-wide tiles over u
+        return _ceil(self.mu, 16)
+
+    @property
+    def NTW(self) -> int:           # 16-wide tiles over w
+        return _ceil(self.mw, 16)
+
+    def ordered_pairs(self):
+        return sorted(self.pairs.items(), key=lambda kv: (kv[0][1], kv[0][0]))
+
+
+class UVWGenerator:
+    DW_WORKGROUPS = 256          # persistent dW workgroups: one per compute unit of an MI355X
+
+    def __init__(self, problem: TPProblem):
+        self.problem = problem
+        self.kind = "uvw"
+        self.T = {np.float32: "float", np.float64: "double"}[problem.irrep_dtype]
+        self.itemsize = 4 if self.T == "float" else 8
+        self.shared = bool(problem.shared_weights)
+        if not self.shared:
+            raise NotImplementedError("uvw tensor products need shared_weights=True in this implementation")
+        self.in1, self.in2, self.out = _blocks(problem.irreps_in1), _blocks(problem.irreps_in2), _blocks(problem.irreps_out)
+        self.D1, self.D2, self.D3 = problem.irreps_in1.dim, problem.irreps_in2.dim, problem.irreps_out.dim
+        self.WN = problem.weight_numel
+        self.paths: List[WPath] = []
+        woff = 0
+        for t, ins in enumerate(problem.instructions):
+            if ins.connection_mode != "uvw":
+                raise ValueError("UVWGenerator handles uvw instructions only")
+            if not ins.has_weight:
+                raise NotImplementedError("instructions without weights are not supported")
+            a, b, o = self.in1[ins.i_in1], self.in2[ins.i_in2], self.out[ins.i_out]
+            if b.mul != 1:
+                raise NotImplementedError("uvw tensor products need multiplicity 1 on the second operand")
+            c = wigner_3j(a.l, b.l, o.l) * ins.path_weight
+            p = WPath(t, a, b, o, ins.path_weight, woff)
+            for i, j, k in np.argwhere(np.abs(c) > 1e-14):
+                p.pairs.setdefault((int(i), int(j)), []).append((int(k), float(c[i, j, k])))
+            self.paths.append(p)
+            woff += a.mul * o.mul
+        if not self.paths:
+            raise ValueError("Tensor product problem has no valid instructions!")
+        self.used_in1 = sorted({p.a.idx for p in self.paths})
+        self.used_out = sorted({p.o.idx for p in self.paths})
+        self.used_y = sorted({p.b.off + j for p in self.paths for (_, j) in p.pairs})
+        # packed weight copies in the workspace
+        pos = 0
+        for p in self.paths:
+            p.wb = pos
+            pos += p.SU * 64 * p.NTW
+        self.WB_SIZE = pos
+        for p in self.paths:
+            p.wa = pos
+            pos += p.NTU * 64 * p.SW
+        self.WA_END = pos
+        self.PART_OFF = _ceil(pos, 64) * 64
+        self.ws_elems = self.PART_OFF + self.DW_WORKGROUPS * self.WN
+
+    # ------------------------------------------------------------------ helpers
+    def lit(self, v: float) -> str:
+        return literal(v, self.T)
+
+    def row(self, r: int) -> str:
+        """Row of accumulator element r held by this lane (differs between the f32 and f64 MFMA)."""
+        return f"(4 * g + {r})" if self.T == "float" else f"({4 * r} + g)"
+
+    def paths_into(self, o: int) -> List[WPath]:
+        return [p for p in self.paths if p.o.idx == o]
+
+    def paths_from(self, a: int) -> List[WPath]:
+        return [p for p in self.paths if p.a.idx == a]
+
+    def oeq_index(self, p: WPath, u: str, w: str) -> str:
+        """Position of W_t[u, w] in the external (oeq) weight vector: 32 x 32 blocks enumerated
+        (u-block, w-block), each stored [u_local][w_local] (weight_order.py)."""
+        mu, mw = p.mu, p.mw
+        if mu <= 32 and mw <= 32:
+            return f"{p.woff} + ({u}) * {mw} + ({w})"
+        ul = "32" if mu % 32 == 0 else f"min(32, {mu} - (({u}) >> 5) * 32)"
+        wl = "32" if mw % 32 == 0 else f"min(32, {mw} - (({w}) >> 5) * 32)"
+        return f"{p.woff} + (({u}) >> 5) * {32 * mw} + {ul} * ((({w}) >> 5) * 32) + (({u}) & 31) * {wl} + (({w}) & 31)"
+
+    def emit_cg_forward(self, E: Emitter, p: WPath, x: str, y: str, out: str) -> None:
+        """out{k} = sum_ij c_ijk {x}{i} * {y}{off+j}  (declares out0..)."""
+        body, seen = [], []
+        for (i, j), ks in p.ordered_pairs():
+            body.append(f"{{ const T t_ = {x}{i} * {y}{p.b.off + j};")
+            for k, val in ks:
+                if k in seen:
+                    body.append(f"  {out}{k} = oeq_fma({self.lit(val)}, t_, {out}{k});")
+                else:
+                    body.append(f"  {out}{k} = {self.lit(val)} * t_;")
+                    seen.append(k)
+            body.append("}")
+        E("T " + ", ".join(f"{out}{k}" + ("" if k in seen else " = (T)0") for k in range(p.o.D)) + ";")
+        E.extend(body)
+
+    def emit_cg_backward(self, E: Emitter, p: WPath, dt: str, x: str, y: str, dx: str, dy: str) -> None:
+        """dx_i += s_ij y_j, dy_j += s_ij x_i with s_ij = sum_k c_ijk dt_k."""
+        for (i, j), ks in p.ordered_pairs():
+            E("{")
+            for n_, (k, val) in enumerate(ks):
+                if n_ == 0:
+                    E(f"  T s_ = {self.lit(val)} * {dt}{k};")
+                else:
+                    E(f"  s_ = oeq_fma({self.lit(val)}, {dt}{k}, s_);")
+            E(f"  {dx}{i} = oeq_fma(s_, {y}{p.b.off + j}, {dx}{i});")
+            E(f"  {dy}{p.b.off + j} = oeq_fma(s_, {x}{i}, {dy}{p.b.off + j});")
+            E("}")
+
+    # ================================================================== prep
+    def prep_body(self) -> str:
+        """Packs the external weight vector into the two MFMA operand layouts (zero padded)."""
+        E = Emitter()
+        E("const int q = blockIdx.x * 256 + threadIdx.x;")
+        E("T* __restrict__ wsT = (T*)ws;")
+        for p in self.paths:
+            nb = p.SU * 64 * p.NTW
+            E(f"if (q >= {p.wb} && q < {p.wb + nb}) {{   // forward copy of path {p.t}: [s][lane][nt]")
+            E(f"    const int e = q - {p.wb};")
+            E(f"    const int nt = e % {p.NTW}; const int ln = (e / {p.NTW}) & 63; const int s = e / {64 * p.NTW};")
+            E(f"    const int u = 4 * s + (ln >> 4); const int w = {p.NTW} * (ln & 15) + nt;")
+            E(f"    wsT[q] = (u < {p.mu} && w < {p.mw}) ? W[{self.oeq_index(p, 'u', 'w')}] : (T)0;")
+            E("}")
+            na = p.NTU * 64 * p.SW
+            E(f"if (q >= {p.wa} && q < {p.wa + na}) {{   // backward copy of path {p.t}: [mt][lane][s]")
+            E(f"    const int e = q - {p.wa};")
+            E(f"    const int s = e % {p.SW}; const int ln = (e / {p.SW}) & 63; const int mt = e / {64 * p.SW};")
+            E(f"    const int u = 16 * mt + (ln & 15); const int w = 4 * s + (ln >> 4);")
+            E(f"    wsT[q] = (u < {p.mu} && w < {p.mw}) ? W[{self.oeq_index(p, 'u', 'w')}] : (T)0;")
+            E("}")
+        return E.text()
+
+    @property
+    def prep_blocks(self) -> int:
+        return _ceil(self.WA_END, 256)
+
+    # =============================================================== forward
+    def forward_body(self) -> str:
+        E = Emitter()
+        E("const int lane = threadIdx.x, c = lane & 15, g = lane >> 4;")
+        E("const u64 row0 = (u64)blockIdx.x * 16;")
+        E("if (row0 >= n) return;")
+        E("const u64 rowA = min(row0 + (u64)c, n - 1);       // rows past the end repeat the last row, never stored")
+        E("const T* __restrict__ wsT = (const T*)ws;")
+        E(f"const T* __restrict__ Xr = X + rowA * {self.D1};")
+        for f in self.used_y:
+            E(f"const T y{f} = Y[rowA * {self.D2} + {f}];")
+        for o in self.out:
+            if o.dim == 0:
+                continue
+            NT = _ceil(o.mul, 16)
+            E(f"{{ // output block {o.idx}: {o.mul}x l={o.l}")
+            E.level += 1
+            if o.idx not in self.used_out:
+                for r in range(4):
+                    E(f"{{ const u64 row = row0 + {self.row(r)}; if (row < n) for (int q = c; q < {o.dim}; q += 16) Z[row * {self.D3} + {o.off} + q] = (T)0; }}")
+                E.level -= 1
+                E("}")
+                continue
+            for k in range(o.D):
+                for nt in range(NT):
+                    E(f"V4 acc{k}_{nt} = {{0, 0, 0, 0}};")
+            for p in self.paths_into(o.idx):
+                E(f"// path {p.t}: l = {p.a.l} x {p.b.l} -> {p.o.l}, coefficient {p.coeff:.9g}")
+                E("#pragma unroll 4")
+                E(f"for (int s = 0; s < {p.SU}; ++s) {{")
+                E.level += 1
+                if p.mu % 4 == 0:
+                    E("const int u = 4 * s + g;")
+                else:
+                    E("const int uu = 4 * s + g;")
+                    E(f"const int u = min(uu, {p.mu - 1});")
+                E(f"const T* __restrict__ xp = Xr + {p.a.off} + u * {p.a.D};")
+                E("const T " + ", ".join(f"x{i} = xp[{i}]" for i in range(p.a.D)) + ";")
+                self.emit_cg_forward(E, p, "x", "y", "t")
+                if p.mu % 4 != 0:
+                    E(f"if (uu >= {p.mu}) {{ " + " ".join(f"t{k} = (T)0;" for k in range(o.D)) + " }")
+                E(f"const T* __restrict__ bp = wsT + {p.wb} + (s * 64 + lane) * {NT};")
+                E("const T " + ", ".join(f"b{nt} = bp[{nt}]" for nt in range(NT)) + ";")
+                for k in range(o.D):
+                    for nt in range(NT):
+                        E(f"acc{k}_{nt} = oeq_mfma(t{k}, b{nt}, acc{k}_{nt});")
+                E.level -= 1
+                E("}")
+            # lane holds, for each of its 4 rows, w = NT*c + nt (nt < NT) and all k: a contiguous run
+            for r in range(4):
+                E(f"{{ const u64 row = row0 + {self.row(r)};")
+                E(f"  if (row < n) {{ T* __restrict__ zp = Z + row * {self.D3} + {o.off} + {NT} * c * {o.D};")
+                for nt in range(NT):
+                    guard = "" if o.mul % 16 == 0 else f"if ({NT} * c + {nt} < {o.mul}) "
+                    E(f"    {guard}{{ " + " ".join(f"zp[{nt * o.D + k}] = acc{k}_{nt}[{r}];" for k in range(o.D)) + " }")
+                E("  } }")
+            E.level -= 1
+            E("}")
+        return E.text()
+
+    # ====================================================== backward: dX, dY
+    def backward_body(self) -> str:
+        E = Emitter()
+        E("const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;")
+        E("const u64 row0 = (u64)blockIdx.x * 16;")
+        E("if (row0 >= n) return;")
+        E("const u64 rowB = min(row0 + (u64)c, n - 1);")
+        E("const bool bvalid = row0 + c < n;")
+        E("const T* __restrict__ wsT = (const T*)ws;")
+        E(f"const T* __restrict__ Xr = X + rowB * {self.D1};")
+        E(f"const T* __restrict__ Gr = G + rowB * {self.D3};")
+        E(f"__shared__ T dyl[4 * 16 * {max(1, self.D2)}];")
+        for f in self.used_y:
+            E(f"const T y{f} = Y[rowB * {self.D2} + {f}];")
+            E(f"T dy{f} = (T)0;")
+        # dX accumulators of this wavefront: u-subtiles mt = wave + 4q
+        for ai in self.used_in1:
+            a = self.in1[ai]
+            for q in range(_ceil(_ceil(a.mul, 16), 4)):
+                for r in range(4):
+                    E("T " + ", ".join(f"dx{ai}_{q}_{r}_{i} = (T)0" for i in range(a.D)) + ";")
+        for oi in self.used_out:
+            o = self.out[oi]
+            SW = _ceil(o.mul, 4)
+            E(f"{{ // output block {oi}: dZ records of this lane, w = 4s + g")
+            E.level += 1
+            for s in range(SW):
+                if o.mul % 4 == 0:
+                    E(f"const T* __restrict__ gp{s} = Gr + {o.off} + ({4 * s} + g) * {o.D};")
+                    E("const T " + ", ".join(f"gz{s}_{k} = gp{s}[{k}]" for k in range(o.D)) + ";")
+                else:
+                    E(f"const T* __restrict__ gp{s} = Gr + {o.off} + min({4 * s} + g, {o.mul - 1}) * {o.D};")
+                    E("T " + ", ".join(f"gz{s}_{k} = gp{s}[{k}]" for k in range(o.D)) + ";")
+                    E(f"if ({4 * s} + g >= {o.mul}) {{ " + " ".join(f"gz{s}_{k} = (T)0;" for k in range(o.D)) + " }")
+            for p in self.paths_into(oi):
+                a = p.a
+                for q in range(_ceil(p.NTU, 4)):
+                    E(f"// path {p.t}, u-subtile wave + {4 * q}")
+                    E(f"if (wave + {4 * q} < {p.NTU}) {{")
+                    E.level += 1
+                    E(f"const int mt = wave + {4 * q};")
+                    E(f"const T* __restrict__ ap = wsT + {p.wa} + (mt * 64 + lane) * {SW};")
+                    for k in range(o.D):
+                        E(f"V4 acc{k} = {{0, 0, 0, 0}};")
+                    for s in range(SW):
+                        E(f"{{ const T a_ = ap[{s}]; " + " ".join(f"acc{k} = oeq_mfma(a_, gz{s}_{k}, acc{k});" for k in range(o.D)) + " }")
+                    for r in range(4):
+                        E(f"{{ // row {r} of the tile: channel u, batch row b = row0 + c")
+                        if a.mul % 16 == 0:
+                            E(f"  const int u = 16 * mt + {self.row(r)};")
+                        else:
+                            E(f"  const int u = min(16 * mt + {self.row(r)}, {a.mul - 1});")
+                        E(f"  const T* __restrict__ xp = Xr + {a.off} + u * {a.D};")
+                        E("  const T " + ", ".join(f"x{i} = xp[{i}]" for i in range(a.D)) + ";")
+                        E("  const T " + ", ".join(f"dt{k} = acc{k}[{r}]" for k in range(o.D)) + ";")
+                        E.level += 1
+                        self.emit_cg_backward(E, p, "dt", "x", "y", f"dx{a.idx}_{q}_{r}_", "dy")
+                        E.level -= 1
+                        E("}")
+                    E.level -= 1
+                    E("}")
+            E.level -= 1
+            E("}")
+        # ---- dX stores
+        for a in self.in1:
+            if a.dim == 0:
+                continue
+            if a.idx not in self.used_in1:
+                E(f"if (wave == 0 && bvalid) for (int q = g; q < {a.dim}; q += 4) Xg[(row0 + c) * {self.D1} + {a.off} + q] = (T)0;")
+                continue
+            for q in range(_ceil(_ceil(a.mul, 16), 4)):
+                E(f"if (wave + {4 * q} < {_ceil(a.mul, 16)} && bvalid) {{")
+                E(f"    const int mt = wave + {4 * q};")
+                for r in range(4):
+                    E(f"    {{ const int u = 16 * mt + {self.row(r)};")
+                    guard = "" if a.mul % 16 == 0 else f"if (u < {a.mul}) "
+                    E(f"      {guard}{{ T* __restrict__ xp = Xg + (row0 + c) * {self.D1} + {a.off} + u * {a.D}; "
+                      + " ".join(f"xp[{i}] = dx{a.idx}_{q}_{r}_{i};" for i in range(a.D)) + " } }")
+                E("}")
+        # ---- dY: sum over the 4 lane groups (channels), then over the 4 wavefronts, fixed order
+        for f in self.used_y:
+            E(f"dy{f} += oeq_shfl_xor(dy{f}, 16);")
+            E(f"dy{f} += oeq_shfl_xor(dy{f}, 32);")
+        E("if (g == 0) {")
+        for f in range(self.D2):
+            E(f"    dyl[(wave * 16 + c) * {self.D2} + {f}] = " + (f"dy{f};" if f in self.used_y else "(T)0;"))
+        E("}")
+        E("oeq_block_sync();")
+        E(f"if (wave == 0 && g == 0 && bvalid) {{")
+        E(f"    for (int f = 0; f < {self.D2}; ++f)")
+        E(f"        Yg[(row0 + c) * {self.D2} + f] = ((dyl[c * {self.D2} + f] + dyl[(16 + c) * {self.D2} + f]) + dyl[(32 + c) * {self.D2} + f]) + dyl[(48 + c) * {self.D2} + f];")
+        E("}")
+        return E.text()
+
+    # ============================================================ backward: dW
+    def backward_dw_body(self) -> str:
+        E = Emitter()
+        E("const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;")
+        E("const u64 ntiles = (n + 15) / 16;")
+        for p in self.paths:
+            for q in range(_ceil(p.NTU, 4)):
+                for nt in range(p.NTW):
+                    E(f"V4 acc{p.t}_{q}_{nt} = {{0, 0, 0, 0}};")
+        E("for (u64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {")
+        E.level += 1
+        E("const u64 row0 = tile * 16;")
+        E("#pragma unroll 1")
+        E("for (int sp = 0; sp < 4; ++sp) {")
+        E.level += 1
+        E("const u64 b = row0 + 4 * sp + g;          // batch row of this lane for both operands")
+        E("const bool bv = b < n;")
+        E("const u64 bc = bv ? b : n - 1;")
+        E(f"const T* __restrict__ Xr = X + bc * {self.D1};")
+        E(f"const T* __restrict__ Gr = G + bc * {self.D3};")
+        for f in self.used_y:
+            E(f"const T y{f} = bv ? Y[bc * {self.D2} + {f}] : (T)0;     // zero rows past the end: T = 0 there")
+        # x records: u = 16 mt + c
+        for ai in self.used_in1:
+            a = self.in1[ai]
+            for q in range(_ceil(_ceil(a.mul, 16), 4)):
+                uexp = f"16 * (wave + {4 * q}) + c"
+                ucl = uexp if a.mul % 64 == 0 else f"min({uexp}, {a.mul - 1})"
+                E(f"const T* __restrict__ xp{ai}_{q} = Xr + {a.off} + ({ucl}) * {a.D};")
+                if a.mul % 64 == 0:
+                    E("const T " + ", ".join(f"x{ai}_{q}_{i} = xp{ai}_{q}[{i}]" for i in range(a.D)) + ";")
+                else:
+                    E("T " + ", ".join(f"x{ai}_{q}_{i} = xp{ai}_{q}[{i}]" for i in range(a.D)) + ";")
+                    E(f"if ({uexp} >= {a.mul}) {{ " + " ".join(f"x{ai}_{q}_{i} = (T)0;" for i in range(a.D)) + " }")
+        for oi in self.used_out:
+            o = self.out[oi]
+            NT = _ceil(o.mul, 16)
+            E(f"{{ // output block {oi}: dZ records, w = 16 nt + c")
+            E.level += 1
+            for nt in range(NT):
+                wexp = f"{16 * nt} + c"
+                wcl = wexp if o.mul % 16 == 0 else f"min({wexp}, {o.mul - 1})"
+                E(f"const T* __restrict__ gp{nt} = Gr + {o.off} + ({wcl}) * {o.D};")
+                E("const T " + ", ".join(f"gz{nt}_{k} = gp{nt}[{k}]" for k in range(o.D)) + ";")
+            for p in self.paths_into(oi):
+                for q in range(_ceil(p.NTU, 4)):
+                    E(f"if (wave + {4 * q} < {p.NTU}) {{  // path {p.t}")
+                    E.level += 1
+                    self.emit_cg_forward(E, p, f"x{p.a.idx}_{q}_", "y", "t")
+                    for nt in range(NT):
+                        for k in range(o.D):
+                            E(f"acc{p.t}_{q}_{nt} = oeq_mfma(t{k}, gz{nt}_{k}, acc{p.t}_{q}_{nt});")
+                    E.level -= 1
+                    E("}")
+            E.level -= 1
+            E("}")
+        E.level -= 1
+        E("}")
+        E.level -= 1
+        E("}")
+        # ---- partial sums of this workgroup, laid out [t][u][w]
+        E(f"T* __restrict__ part = (T*)ws + {self.PART_OFF} + (u64)blockIdx.x * {self.WN};")
+        for p in self.paths:
+            for q in range(_ceil(p.NTU, 4)):
+                E(f"if (wave + {4 * q} < {p.NTU}) {{")
+                for nt in range(p.NTW):
+                    for r in range(4):
+                        E(f"    {{ const int u = 16 * (wave + {4 * q}) + {self.row(r)}; const int w = {16 * nt} + c;")
+                        E(f"      if (u < {p.mu} && w < {p.mw}) part[{p.woff} + u * {p.mw} + w] = acc{p.t}_{q}_{nt}[{r}]; }}")
+                E("}")
+        return E.text()
+
+    def reduce_body(self) -> str:
+        E = Emitter()
+        E("const int q = blockIdx.x * 256 + threadIdx.x;")
+        E(f"if (q >= {self.WN}) return;")
+        E(f"const T* __restrict__ part = (const T*)ws + {self.PART_OFF};")
+        E("T acc = (T)0;")
+        E(f"for (int b = 0; b < {self.DW_WORKGROUPS}; ++b) acc += part[(u64)b * {self.WN} + q];")
+        E("int dst = q;")
+        for p in self.paths:
+            E(f"if (q >= {p.woff} && q < {p.woff + p.mu * p.mw}) {{ const int e = q - {p.woff}; const int u = e / {p.mw}; const int w = e - u * {p.mw}; dst = {self.oeq_index(p, 'u', 'w')}; }}")
+        E("Wg[dst] = acc;")
+        return E.text()
+
+    # ---------------------------------------------------------------- rendering
+    def render(self, prelude: str = None) -> str:
+        env = jinja_env()
+        if prelude is None:
+            prelude = env.get_template("prelude.hip.jinja").render(T=self.T)
+        return env.get_template("tp_uvw.hip.jinja").render(g=self, prelude=prelude)
+
+    def describe(self) -> str:
+        return (f"uvw T={self.T} paths={len(self.paths)} d1={self.D1} d2={self.D2} d3={self.D3} wn={self.WN} "
+                f"mfma=16x16x4 workspace={self.ws_elems * self.itemsize}B")
+
+    def plan(self):
+        FIXED, ROW = 0, 1
+        fwd = [dict(kernel="prep_forward", num_threads=256, grid_kind=FIXED, num_blocks=self.prep_blocks),
+               dict(kernel="forward", num_threads=64, grid_kind=ROW, work_per_block=16)]
+        bwd = [dict(kernel="prep_backward", num_threads=256, grid_kind=FIXED, num_blocks=self.prep_blocks),
+               dict(kernel="backward", num_threads=256, grid_kind=ROW, work_per_block=16),
+               dict(kernel="backward_dw", num_threads=256, grid_kind=FIXED, num_blocks=self.DW_WORKGROUPS),
+               dict(kernel="backward_reduce", num_threads=256, grid_kind=FIXED, num_blocks=_ceil(self.WN, 256))]
+        return fwd, bwd, (lambda nnz=0, nodes=0: self.ws_elems * self.itemsize)

@@ -62,10 +62,30 @@ struct VT { T v[16 / sizeof(T)]; };
 static inline void oeq_dma16(const T* g, T* lds_base) { memcpy((char*)lds_base + 16 * threadIdx.x, g, 16); }
 static inline void oeq_wait_vm() {}
 static inline void oeq_wait_lds() {}
+static inline void oeq_block_sync() { pthread_barrier_wait(&g_bar); }
+// matrix-core step of one wavefront, emulated collectively by its 64 threads
+struct V4 { T v[4]; T& operator[](int i) { return v[i]; } const T& operator[](int i) const { return v[i]; } };
+static pthread_barrier_t g_wbar[16];
+static T g_mA[16][16][4], g_mB[16][4][16];
+static inline V4 oeq_mfma(T a, T b, V4 c) {
+    const int wv = threadIdx.x >> 6, l = threadIdx.x & 63;
+    g_mA[wv][l & 15][l >> 4] = a; g_mB[wv][l >> 4][l & 15] = b;
+    pthread_barrier_wait(&g_wbar[wv]);
+    V4 d = c;
+    for (int r = 0; r < 4; ++r) {
+        const int i = (sizeof(T) == 4) ? 4 * (l >> 4) + r : 4 * r + (l >> 4), j = l & 15;
+        T acc = 0;
+        for (int k = 0; k < 4; ++k) acc += g_mA[wv][i][k] * g_mB[wv][k][j];
+        d[r] = c[r] + acc;
+    }
+    pthread_barrier_wait(&g_wbar[wv]);
+    return d;
+}
 
 static void emu_run(unsigned gx, unsigned gy, unsigned block, const std::function<void()>& kernel) {
     gridDim = {gx, gy, 1}; blockDim = {block, 1, 1};
     pthread_barrier_init(&g_bar, nullptr, block);
+    for (unsigned w = 0; w < (block + 63) / 64; ++w) pthread_barrier_init(&g_wbar[w], nullptr, block < 64 ? block : 64);
     for (unsigned by = 0; by < gy; ++by)
         for (unsigned bx = 0; bx < gx; ++bx) {
             std::vector<std::thread> th;
@@ -117,6 +137,14 @@ int main(int argc, char** argv) {
     emu_write(d + "/Z.bin", Z); emu_write(d + "/Xg.bin", Xg); emu_write(d + "/Yg.bin", Yg); emu_write(d + "/Wg.bin", Wg);
     return 0;
 }
+"""
+
+TP_EXTRA_UVW = r"""
+        else if (k == "prep_forward") emu_run(gx, gy, threads, [&] { prep_forward(n, (const T*)X.data(), (const T*)Y.data(), (T*)Z.data(), (const T*)W.data(), ws.data()); });
+#define UVW_BWD(fn) emu_run(gx, gy, threads, [&] { fn(n, (const T*)X.data(), (T*)Xg.data(), (const T*)Y.data(), (T*)Yg.data(), (const T*)W.data(), (T*)Wg.data(), (const T*)G.data(), ws.data()); })
+        else if (k == "prep_backward") UVW_BWD(prep_backward);
+        else if (k == "backward_dw") UVW_BWD(backward_dw);
+        else if (k == "backward_reduce") UVW_BWD(backward_reduce);
 """
 
 TP_EXTRA_SHARED = r"""
@@ -213,7 +241,8 @@ def _run(exe: pathlib.Path, workdir: str) -> None:
 def run_tp(gen, steps: Sequence[Dict], X, Y, W, G=None, ws_bytes: int = 0):
     """Run TP steps; returns dict of outputs (Z or dX, dY, dW)."""
     dt = np.float32 if gen.T == "float" else np.float64
-    main = TP_MAIN.replace("@EXTRA@", TP_EXTRA_SHARED if gen.shared else "")
+    extra = TP_EXTRA_UVW if gen.kind == "uvw" else (TP_EXTRA_SHARED if gen.shared else "")
+    main = TP_MAIN.replace("@EXTRA@", extra)
     exe = build(gen.render(prelude=emu_prelude(gen.T)), main)
     n = X.shape[0]
     with tempfile.TemporaryDirectory() as d:
