@@ -1,0 +1,107 @@
+"""The generated kernel source, compiled for the host and run under AddressSanitizer
+(tests/host_emu): checks indexing, bounds and arithmetic of every kernel family against the
+oracle without a GPU.  Sizes are tiny because 64 host threads stand in for one wavefront."""
+import numpy as np
+import pytest
+
+import openequivariance_amd as oeq
+from openequivariance_amd.codegen.uvu import UVUGenerator
+from openequivariance_amd.codegen.uvu_direct import UVUDirectGenerator
+from openequivariance_amd.codegen.uvw import UVWGenerator
+from host_emu import emu
+from oracle import spec, tp as otp, weights as ow
+
+import common
+from common import rel_err
+
+TOL = 2e-6     # fp32 arithmetic against the fp64 oracle on O(1) data
+
+
+def _tp(gen_cls, irreps, n, seed, **kw):
+    prob, oprob = common.channelwise(irreps)
+    g = gen_cls(prob, "tp", **kw)
+    X, Y, W, G = common.tp_inputs(prob, n, seed)
+    fwd, bwd, ws = g.plan()
+    out = emu.run_tp(g, fwd, X, Y, W, ws_bytes=ws())
+    assert rel_err(out["Z"], otp.forward(oprob, X, Y, W)) < TOL
+    out = emu.run_tp(g, bwd, X, Y, W, G, ws_bytes=ws())
+    for got, ref in zip((out["Xg"], out["Yg"], out["Wg"]), otp.backward(oprob, X, Y, W, G)):
+        assert rel_err(got, ref) < TOL
+
+
+def test_direct_tp_two_rows_per_wave():
+    _tp(UVUDirectGenerator, common.NEQUIP, 5, 1)
+
+
+def test_direct_tp_ragged_two_chunks():
+    _tp(UVUDirectGenerator, ("5x0e+3x1o+70x2e", "1x0e+1x1o+1x2e", "5x0e+3x1o+70x2e+7x3o"), 3, 2)
+
+
+def test_direct_tp_record_stores_only():
+    _tp(UVUDirectGenerator, common.NEQUIP, 3, 3, vector_stores=False)
+
+
+def test_generic_tp_shared_weights():
+    ins = [(0, 0, 0, "uvu", True), (1, 1, 0, "uvu", True), (1, 0, 1, "uvu", True)]
+    a = ("24x0e+24x1o", "1x0e+1x1o", "24x0e+24x1o")
+    prob = oeq.TPProblem(*a, ins, shared_weights=True, internal_weights=False)
+    oprob = spec.Problem(*a, ins, shared_weights=True)
+    g = UVUGenerator(prob, "tp", dw_partials=3)
+    X, Y, W, G = common.tp_inputs(prob, 9, 4)
+    fwd, bwd, ws = g.plan()
+    out = emu.run_tp(g, fwd, X, Y, W, ws_bytes=ws())
+    assert rel_err(out["Z"], otp.forward(oprob, X, Y, W)) < TOL
+    out = emu.run_tp(g, bwd, X, Y, W, G, ws_bytes=ws())
+    for got, ref in zip((out["Xg"], out["Yg"], out["Wg"]), otp.backward(oprob, X, Y, W, G)):
+        assert rel_err(got, ref) < TOL
+
+
+@pytest.mark.parametrize("det", [False, True])
+def test_conv(det):
+    prob, oprob = common.channelwise(common.NEQUIP)
+    g = UVUGenerator(prob, "conv_det") if det else UVUDirectGenerator(prob, "conv_atomic")
+    nodes, nnz = 7, 19
+    rows, cols = common.random_graph(nodes, nnz, 5)
+    tperm = None
+    if det:
+        rows, cols, tperm, _ = otp.coord_graph(rows, cols)
+    X, Y, W, G = common.conv_inputs(prob, nodes, nnz, 6)
+    fwd, bwd, ws = g.plan()
+    out = emu.run_conv(g, fwd, X, Y, W, rows, cols, tperm=tperm, ws_bytes=ws(nnz, nodes))
+    assert rel_err(out["Z"], otp.conv_forward(oprob, X, Y, W, rows, cols)) < TOL
+    out = emu.run_conv(g, bwd, X, Y, W, rows, cols, G=G, tperm=tperm, ws_bytes=ws(nnz, nodes))
+    for got, ref in zip((out["Xg"], out["Yg"], out["Wg"]), otp.conv_backward(oprob, X, Y, W, G, rows, cols)):
+        assert rel_err(got, ref) < TOL
+
+
+def test_conv_det_chunked_ragged():
+    irreps = ("5x0e+3x1o+70x2e", "1x0e+1x1o+1x2e", "5x0e+3x1o+70x2e+7x3o")
+    prob, oprob = common.channelwise(irreps)
+    g = UVUGenerator(prob, "conv_det")
+    nodes, nnz = 5, 11
+    rows, cols, tperm, _ = otp.coord_graph(*common.random_graph(nodes, nnz, 7))
+    X, Y, W, G = common.conv_inputs(prob, nodes, nnz, 8)
+    fwd, bwd, ws = g.plan()
+    out = emu.run_conv(g, fwd, X, Y, W, rows, cols, tperm=tperm, ws_bytes=ws(nnz, nodes))
+    assert rel_err(out["Z"], otp.conv_forward(oprob, X, Y, W, rows, cols)) < TOL
+    out = emu.run_conv(g, bwd, X, Y, W, rows, cols, G=G, tperm=tperm, ws_bytes=ws(nnz, nodes))
+    for got, ref in zip((out["Xg"], out["Yg"], out["Wg"]), otp.conv_backward(oprob, X, Y, W, G, rows, cols)):
+        assert rel_err(got, ref) < TOL
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_uvw_matrix_core_kernels(dtype, monkeypatch):
+    monkeypatch.setattr(UVWGenerator, "DW_WORKGROUPS", 3)
+    a = ("5x0e+21x1o", "1x0e+1x1o+1x2e", "18x0e+7x1o+3x2e")
+    prob, oprob = common.fully_connected(a, shared=True, dtype=dtype)
+    g = UVWGenerator(prob)
+    X, Y, We, G = common.tp_inputs(prob, 21, 9, dtype, w_scale=0.3)
+    W = ow.e3nn_to_oeq(oprob, We)
+    fwd, bwd, ws = g.plan()
+    tol = TOL if dtype == np.float32 else 1e-13
+    out = emu.run_tp(g, fwd, X, Y, W, ws_bytes=ws())
+    assert rel_err(out["Z"], otp.forward(oprob, X, Y, We)) < tol
+    out = emu.run_tp(g, bwd, X, Y, W, G, ws_bytes=ws())
+    dX, dY, dW = otp.backward(oprob, X, Y, We, G)
+    assert rel_err(out["Xg"], dX) < tol and rel_err(out["Yg"], dY) < tol
+    assert rel_err(ow.oeq_to_e3nn(oprob, out["Wg"]), dW) < tol

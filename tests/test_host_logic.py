@@ -1,0 +1,85 @@
+"""Host-side logic that needs no GPU: validation errors, launch plans, byte/FLOP models, bench contract."""
+import json
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+import openequivariance_amd as oeq
+from openequivariance_amd import workloads
+from openequivariance_amd.codegen.uvu import UVUGenerator
+from openequivariance_amd.codegen.uvu_direct import UVUDirectGenerator
+from openequivariance_amd.codegen.uvw import UVWGenerator
+from openequivariance_amd.conv import flops_data_per_tp
+from openequivariance_amd.tensor_product import validate_problem
+
+import common
+
+
+def test_validation_mirrors_reference_constraints():
+    with pytest.raises(ValueError, match="no valid"):
+        validate_problem(oeq.TPProblem("1x0e", "1x0e", "1x0e", []))
+    mixed = oeq.TPProblem("2x0e", "1x0e", "2x0e", [(0, 0, 0, "uvu", True), (0, 0, 0, "uvw", True)])
+    with pytest.raises(AssertionError):
+        validate_problem(mixed)
+    with pytest.raises(AssertionError):
+        validate_problem(oeq.TPProblem("2x0e", "2x0e", "2x0e", [(0, 0, 0, "uuu", True)]))
+    with pytest.raises(AssertionError):
+        validate_problem(oeq.TPProblem("2x0e", "1x0e", "2x0e", [(0, 0, 0, "uvu", True)], irrep_dtype=np.float64))
+    with pytest.raises(AssertionError):                      # conv needs mul 1 on the second operand
+        UVUGenerator(oeq.TPProblem("2x0e", "2x0e", "2x0e", [(0, 0, 0, "uvu", True)], shared_weights=False,
+                                   internal_weights=False), "conv_atomic")
+
+
+def test_launch_plans():
+    prob, _ = common.channelwise(common.MACE)
+    fwd, bwd, ws = UVUDirectGenerator(prob, "tp").plan()
+    assert [s["kernel"] for s in fwd] == ["forward"] and fwd[0]["work_per_block"] == 1 and ws() == 0
+    prob, _ = common.channelwise(common.NEQUIP)
+    assert UVUDirectGenerator(prob, "tp").plan()[0][0]["work_per_block"] == 2       # two rows per wavefront
+    prob, _ = common.channelwise(common.LARGE)
+    g = UVUGenerator(prob, "conv_det")
+    fwd, bwd, ws = g.plan()
+    assert [s["kernel"] for s in fwd] == ["prep_forward", "forward"] and fwd[1]["grid_y"] == 4
+    assert [s["kernel"] for s in bwd] == ["prep_backward", "backward", "backward_dy_reduce"]
+    assert ws(1000, 10) == 2 * 11 * 8 + 4 * 1000 * 16 * 4
+    prob, _ = common.fully_connected(common.DENSE)
+    fwd, bwd, ws = UVWGenerator(prob).plan()
+    assert [s["kernel"] for s in bwd] == ["prep_backward", "backward", "backward_dw", "backward_reduce"]
+
+
+def test_generated_source_bakes_cg_constants():
+    prob, _ = common.readme_problem()
+    src = UVUDirectGenerator(prob, "tp").render()
+    assert src.count("oeq_fma(0x") + src.count("= 0x") + src.count("= -0x") >= 28      # 28 nonzeros of C(2,3,2)
+    assert "__global__" in src and "#ifdef" not in src
+
+
+def test_work_models_match_the_documented_numbers():
+    mace = workloads.get("mace_uvu")
+    assert mace.alg_bytes["forward"] == 50000 * 49728 and mace.alg_bytes["backward"] == 50000 * 63104
+    dense = workloads.get("dense_uvw_f32")
+    assert dense.alg_flops["forward"] == 100000 * 286720 and dense.alg_flops["backward"] == 100000 * 573440
+    prob, _ = common.channelwise(common.NEQUIP)
+    ops_f, bytes_f, nnz = flops_data_per_tp(prob, "forward")
+    ops_b, bytes_b, _ = flops_data_per_tp(prob, "backward")
+    assert (bytes_f, bytes_b, nnz) == (7076, 9672, 83)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    res = subprocess.run([sys.executable, "bench.py", "--gpus", "2"], capture_output=True, text=True,
+                         cwd=str(common.__file__).rsplit("/tests", 1)[0])
+    assert res.returncode != 0 and "one GPU" in res.stderr
+
+
+def test_spherical_harmonics_inputs():
+    from openequivariance_amd.sh import spherical_harmonics
+    v = np.random.default_rng(0).standard_normal((20, 3))
+    Y = spherical_harmonics(3, v)
+    assert Y.shape == (20, 16)
+    n = v / np.linalg.norm(v, axis=1, keepdims=True)
+    np.testing.assert_allclose(Y[:, 0], 1.0)
+    np.testing.assert_allclose(Y[:, 1:4], np.sqrt(3) * n, atol=1e-13)
+    for l in range(4):
+        np.testing.assert_allclose((Y[:, l * l:(l + 1) ** 2] ** 2).sum(1), 2 * l + 1, atol=1e-12)
