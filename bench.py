@@ -102,8 +102,40 @@ def cpu_baseline(wl, case, sample):
             "sample": what + "; torch CPU einsum + autograd, fp32 (e3nn itself is not installable offline)"}
 
 
+COPY_SRC = r"""
+// Plain streaming copy: reads n 16-byte vectors and writes n 16-byte vectors, nothing else.
+extern "C" __global__ __launch_bounds__(256) void oeq_copy_calibration(const float4* __restrict__ in, float4* __restrict__ out, unsigned long long n) {
+    for (unsigned long long i = (unsigned long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (unsigned long long)gridDim.x * 256)
+        out[i] = in[i];
+}
+"""
+
+
+def copy_calibration(steps):
+    """A copy kernel of known size (1 GiB read + 1 GiB written per launch), used to scale the
+    FETCH_SIZE / WRITE_SIZE counters of rocprofv3: run it under the same --pmc as the workload."""
+    import ctypes as C
+    import torch
+    from openequivariance_amd import runtime as rt
+    nbytes = 1 << 30
+    src = torch.ones(nbytes // 4, dtype=torch.float32, device="cuda")
+    dst = torch.empty_like(src)
+    mod = rt.Module(rt.compile_source(COPY_SRC))
+    stream = torch.cuda.current_stream().cuda_stream
+    for _ in range(steps):
+        mod.launch("oeq_copy_calibration", 256 * 16, 256,
+                   [C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr()), C.c_uint64(nbytes // 16)], stream=stream)
+    torch.cuda.synchronize()
+    assert torch.equal(src[:1024], dst[:1024])
+    print(json.dumps({"workload": "copy_calibration", "bytes_read_per_launch": nbytes,
+                      "bytes_written_per_launch": nbytes, "launches": steps}))
+
+
 def main():
     args = parse()
+    if args.workload == "copy_calibration":
+        copy_calibration(args.steps)
+        return
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (the path shards over rows/edges "
               "without communication, see DESIGN.md)", file=sys.stderr)
