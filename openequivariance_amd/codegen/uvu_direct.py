@@ -31,7 +31,7 @@ class UVUDirectGenerator(UVUGenerator):
 
     def __init__(self, problem: TPProblem, kind: str = "tp", waves_per_eu: int = 0, vector_stores: bool = True):
         super().__init__(problem, kind)
-        if kind == "conv_det" or self.shared:
+        if (kind == "conv_det" and not getattr(self, "_allow_det", False)) or self.shared:
             raise NotImplementedError("direct schedule: batch product with per-row weights and atomic convolution")
         self.waves_per_eu = waves_per_eu
         # False: outputs are written with dword-aligned record stores only (for callers whose

@@ -22,6 +22,7 @@ import torch
 
 from . import runtime as rt
 from .codegen.uvu import UVUGenerator
+from .codegen.uvu_det import UVUDetGenerator
 from .codegen.uvu_direct import UVUDirectGenerator
 from .codegen.uvu_fast import UVUFastGenerator
 from .problem import TPProblem
@@ -92,7 +93,9 @@ class TensorProductConv:
         if mode != "uvu":
             raise NotImplementedError("TensorProductConv supports uvu problems")
 
-        if deterministic or schedule() == "lds":
+        if deterministic and schedule() != "lds":
+            self.generator = UVUDetGenerator(config)
+        elif schedule() == "lds":
             self.generator = UVUGenerator(config, "conv_det" if deterministic else "conv_atomic")
         else:
             self.generator = UVUDirectGenerator(config, "conv_atomic")

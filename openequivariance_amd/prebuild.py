@@ -12,6 +12,7 @@ import numpy as np
 
 from . import runtime as rt
 from .codegen.uvu import UVUGenerator
+from .codegen.uvu_det import UVUDetGenerator
 from .codegen.uvu_direct import UVUDirectGenerator
 from .codegen.uvu_fast import UVUFastGenerator
 from .problem import ChannelwiseTPP, FullyConnectedTPProblem, TPProblem
@@ -34,6 +35,8 @@ def benchmark_generators():
     for name, g in list(gens):
         if g.kind != "conv_det" and not g.shared:
             gens.append((name + "/direct", UVUDirectGenerator(g.problem, g.kind)))
+        elif g.kind == "conv_det":
+            gens.append((name + "/direct", UVUDetGenerator(g.problem)))
     try:
         from .codegen.uvw import UVWGenerator
     except ImportError:
