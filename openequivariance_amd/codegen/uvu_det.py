@@ -26,8 +26,16 @@ from .uvu_direct import UVUDirectGenerator
 class UVUDetGenerator(UVUDirectGenerator):
     _allow_det = True
 
-    def __init__(self, problem: TPProblem):
+    def __init__(self, problem: TPProblem, prefetch_backward=None):
         super().__init__(problem, "conv_det")
+        # fetch the next edge's operands while the current edge is being computed; pays when the
+        # per-edge register footprint is small enough to keep several wavefronts per SIMD
+        words = sum(self.out[i].D for i in self.used_out) + len(self.paths) + len(self.used_y)
+        import os
+        env = os.environ.get("OEQ_AMD_DET_PREFETCH")          # "0" / "1": tuning override for A/B runs
+        if prefetch_backward is None and env in ("0", "1"):
+            prefetch_backward = (env == "1")
+        self.prefetch_backward = (words <= 56) if prefetch_backward is None else prefetch_backward
         self.uniform_rows = False          # validity is per lane (edge lists differ between sub-rows)
         self.chunk_in_grid = True
 
@@ -42,13 +50,13 @@ class UVUDetGenerator(UVUDirectGenerator):
 
     # ------------------------------------------------------------------ common
     def _node_setup(self, E: Emitter, ptr_off: str) -> None:
+        """One node per wavefront.  With multiplicity <= 32 the wavefront's R = 64/P lane groups walk
+        interleaved sub-lists of the node's edges (edge beg + it*R + sub) and their partial sums are
+        combined in a fixed order at the end, which shortens the serial edge loop R-fold."""
         R = self.R
         E("const int c = blockIdx.y; (void)c;")
         E(f"const int u = c * {self.P} + ul;")
-        if R == 1:
-            E("const u64 node = blockIdx.x;")
-        else:
-            E(f"const u64 node = (u64)blockIdx.x * {R} + sub;")
+        E("const u64 node = blockIdx.x;")
         E("const bool nv = node < node_count;")
         E(f"const i64* __restrict__ ptr = (const i64*)ws + {ptr_off};")
         E("i64 beg = 0, end = 0;")
@@ -57,18 +65,30 @@ class UVUDetGenerator(UVUDirectGenerator):
         E("if (end > (i64)nnz) end = (i64)nnz;")
         E("if (end < beg) end = beg;")
         E("const int len = (int)(end - beg);")
-        E("int maxlen = len;")
+        E(f"const int maxlen = (len + {R - 1}) / {R};")
+        self.noderow_of = (lambda r: ("node", "nv"))
+
+    def edge_pos(self, it: str) -> str:
+        return f"(({it}) * {self.R} + sub)" if self.R > 1 else f"({it})"
+
+    def emit_sub_sum(self, E: Emitter, names) -> None:
+        """Add the partial sums of the R lane groups (fixed order); every lane ends with the total."""
         m = 32
         while m >= self.P:
-            E(f"maxlen = max(maxlen, oeq_shfl_xor_i32(maxlen, {m}));")
+            for n in names:
+                E(f"{n} += oeq_shfl_xor({n}, {m});")
             m //= 2
-        if R == 1:
-            E("maxlen = __builtin_amdgcn_readfirstlane(maxlen);")
-        base = "node" if R == 1 else f"((u64)blockIdx.x * {R} + {{r}})"
-        if R == 1:
-            self.noderow_of = (lambda r: ("node", "nv"))
-        else:
-            self.noderow_of = (lambda r: (f"((u64)blockIdx.x * {R} + {r})", f"((u64)blockIdx.x * {R} + {r} < node_count)"))
+
+    def store_act(self, blk) -> str:
+        base = "nv" if self.R == 1 else "(nv && sub == 0)"
+        return base if self.full(blk) else f"({base} && u < {blk.mul})"
+
+    def plan(self):
+        fwd, bwd, ws = super().plan()
+        for s in fwd + bwd:
+            if s["kernel"] in ("forward", "backward"):
+                s["work_per_block"] = 1
+        return fwd, bwd, ws
 
     # ================================================================= forward
     def conv_det_forward_body(self) -> str:
@@ -78,24 +98,52 @@ class UVUDetGenerator(UVUDirectGenerator):
         self._cur_c = "e"
         for oi in self.used_out:
             E("T " + ", ".join(f"z{oi}_{k} = (T)0" for k in range(self.out[oi].D)) + ";")
+        # registers of the edge being fetched ("N" = next); the loop computes on a copy while the
+        # loads of the following edge are in flight (software pipelining hides the gather latency,
+        # which dominates when a node has few edges and few wavefronts are resident)
+        names = []
+        for i in self.used_in1:
+            names += [f"x{i}_{m}" for m in range(self.in1[i].D)]
+        names += [f"We_{p.t}_{v}" for p in self.paths for v in range(p.mv)]
+        names += [f"y{f}" for f in self.used_y]
+        E("T " + ", ".join(f"N{n} = (T)0" for n in names) + ";")
+
+        def load(E, it):
+            E("{")
+            E.level += 1
+            E(f"const bool ev = {self.edge_pos(it)} < len;")
+            E(f"const u64 e = ev ? (u64)(beg + {self.edge_pos(it)}) : (u64)(nnz - 1);   // idle lanes re-read the last edge, masked below")
+            E("const i64 snd = cols[e];")
+            E("const bool rv = ev && snd >= 0 && snd < (i64)node_count;")
+            E("const u64 sndc = rv ? (u64)snd : 0;")
+            E(f"const T* __restrict__ Yr = Y + e * {self.D2};")
+            E(f"const T* __restrict__ Wr = W + e * {self.WN};")
+            for f in self.used_y:
+                E(f"Ny{f} = Yr[{f}];")
+            for i in self.used_in1:
+                a = self.in1[i]
+                E(f"{{ const T* __restrict__ p_ = X + sndc * {self.D1} + {a.off} + {self.uclamp(a, 0)} * {a.D}; "
+                  + " ".join(f"Nx{i}_{m} = p_[{m}];" for m in range(a.D)) + " }")
+                # everything an edge adds is proportional to x: zero it for idle lanes
+                E(f"if (!({self.act(a)})) {{ " + " ".join(f"Nx{i}_{m} = (T)0;" for m in range(a.D)) + " }")
+            for p in self.paths:
+                for v in range(p.mv):
+                    E(f"NWe_{p.t}_{v} = Wr[{self.widx(p, self.uclamp(p.a, 0), v)}];")
+            E.level -= 1
+            E("}")
+        E("if (maxlen > 0) {")
+        E.level += 1
+        load(E, "0")
+        E.level -= 1
+        E("}")
         E("for (int it = 0; it < maxlen; ++it) {")
         E.level += 1
-        E("const bool ev = it < len;")
-        E("const u64 e = ev ? (u64)(beg + it) : (u64)(nnz - 1);     // idle lanes re-read the last edge, masked below")
-        E("const i64 snd = cols[e];")
-        E("const bool rv = ev && snd >= 0 && snd < (i64)node_count;")
-        E("const u64 sndc = rv ? (u64)snd : 0;")
-        E(f"const T* __restrict__ Yr = Y + e * {self.D2};")
-        E(f"const T* __restrict__ Wr = W + e * {self.WN};")
-        self.emit_y_load_direct(E)
-        # X records of the sender (zero for idle lanes: everything they add is proportional to x)
-        for i in self.used_in1:
-            a = self.in1[i]
-            self.emit_record_load(E, [f"x{i}_{m}" for m in range(a.D)],
-                                  f"X + sndc * {self.D1} + {a.off} + {self.uclamp(a, 0)} * {a.D}", self.act(a), zero=True)
-        for p in self.paths:
-            for v in range(p.mv):
-                E(f"const T We_{p.t}_{v} = Wr[{self.widx(p, self.uclamp(p.a, 0), v)}];")
+        E("const T " + ", ".join(f"{n} = N{n}" for n in names) + ";")
+        E("if (it + 1 < maxlen) {")
+        E.level += 1
+        load(E, "it + 1")
+        E.level -= 1
+        E("}")
         for oi in self.used_out:
             self.emit_forward_block(E, self.out[oi], "Wr", zname=f"z{oi}_", declare=False)
         E.level -= 1
@@ -106,11 +154,16 @@ class UVUDetGenerator(UVUDirectGenerator):
                 continue
             E("{")
             E.level += 1
-            if o.idx in self.used_out:
+            if o.idx in self.used_out and self.R == 1:
                 self.emit_block_store(E, o, [f"z{o.idx}_{k}" for k in range(o.D)], "Z", self.D3, "node",
                                       self.noderow_of, "store", via_lds=True)
+            elif o.idx in self.used_out:
+                zs = [f"z{o.idx}_{k}" for k in range(o.D)]
+                self.emit_sub_sum(E, zs)
+                self.emit_record_store(E, zs, f"Z + node * {self.D3} + {o.off} + u * {o.D}", self.store_act(o))
             else:
-                self.emit_record_store(E, ["(T)0"] * o.D, f"Z + node * {self.D3} + {o.off} + u * {o.D}", self.act(o))
+                self.emit_record_store(E, ["(T)0"] * o.D, f"Z + node * {self.D3} + {o.off} + u * {o.D}",
+                                       self.store_act(o))
             E.level -= 1
             E("}")
         return E.text()
@@ -132,29 +185,57 @@ class UVUDetGenerator(UVUDirectGenerator):
             self.emit_record_load(E, [f"x{i}_{m}" for m in range(a.D)],
                                   f"X + nodec * {self.D1} + {a.off} + {self.uclamp(a, 0)} * {a.D}", self.act(a), zero=True)
             E("T " + ", ".join(f"dx{i}_{m} = (T)0" for m in range(a.D)) + ";")
+        names = [f"G{oi}_{k}" for oi in self.used_out for k in range(self.out[oi].D)]
+        names += [f"We_{p.t}_{v}" for p in self.paths for v in range(p.mv)]
+        names += [f"y{f}" for f in self.used_y]
+        E("T " + ", ".join(f"N{n} = (T)0" for n in names) + ";")
+        E("u64 Ne = 0; bool Nrv = false;")
+
+        def load(E, it):
+            E("{")
+            E.level += 1
+            E(f"const bool ev = {self.edge_pos(it)} < len;")
+            E(f"const u64 j = ev ? (u64)(beg + {self.edge_pos(it)}) : (u64)(nnz - 1);")
+            E("const i64 e0 = tperm[j];")
+            E("const bool ok_e = ev && e0 >= 0 && e0 < (i64)nnz;")
+            E("const u64 e = ok_e ? (u64)e0 : 0;")
+            E("const i64 rcv = rows[e];")
+            E("const bool rv = ok_e && rcv >= 0 && rcv < (i64)node_count;")
+            E("const u64 rcvc = rv ? (u64)rcv : 0;")
+            E("Ne = e; Nrv = rv;")
+            E(f"const T* __restrict__ Yr = Y + e * {self.D2};")
+            E(f"const T* __restrict__ Wr = W + e * {self.WN};")
+            for f in self.used_y:
+                E(f"Ny{f} = Yr[{f}];")
+            for p in self.paths:
+                for v in range(p.mv):
+                    E(f"NWe_{p.t}_{v} = Wr[{self.widx(p, self.uclamp(p.a, 0), v)}];")
+            for oi in self.used_out:
+                o = self.out[oi]
+                E(f"{{ const T* __restrict__ p_ = G + rcvc * {self.D3} + {o.off} + {self.uclamp(o, 0)} * {o.D}; "
+                  + " ".join(f"NG{oi}_{k} = p_[{k}];" for k in range(o.D)) + " }")
+                # every gradient of an edge is proportional to dZ: zero it for idle lanes
+                E(f"if (!({self.act(o)})) {{ " + " ".join(f"NG{oi}_{k} = (T)0;" for k in range(o.D)) + " }")
+            E.level -= 1
+            E("}")
+        E("if (maxlen > 0) {")
+        E.level += 1
+        load(E, "0")
+        E.level -= 1
+        E("}")
         E("for (int it = 0; it < maxlen; ++it) {")
         E.level += 1
-        E("const bool ev = it < len;")
-        E("const u64 j = ev ? (u64)(beg + it) : (u64)(nnz - 1);")
-        E("const i64 e0 = tperm[j];")
-        E("const bool ok_e = ev && e0 >= 0 && e0 < (i64)nnz;")
-        E("const u64 e = ok_e ? (u64)e0 : 0;")
-        E("const i64 rcv = rows[e];")
-        E("rv = ok_e && rcv >= 0 && rcv < (i64)node_count;")
-        E("const u64 rcvc = rv ? (u64)rcv : 0;")
-        E(f"const T* __restrict__ Yr = Y + e * {self.D2};")
-        E(f"const T* __restrict__ Wr = W + e * {self.WN};")
+        E("const T " + ", ".join(f"{n} = N{n}" for n in names) + ";")
+        E("const u64 e = Ne; rv = Nrv;")
+        if self.prefetch_backward:
+            E("if (it + 1 < maxlen) {")
+            E.level += 1
+            load(E, "it + 1")
+            E.level -= 1
+            E("}")
         E(f"T* __restrict__ Wgr = Wg + e * {self.WN};")
-        self.emit_y_load_direct(E)
         for f in self.used_y:
             E(f"T dy{f} = (T)0;")
-        for p in self.paths:
-            for v in range(p.mv):
-                E(f"const T We_{p.t}_{v} = Wr[{self.widx(p, self.uclamp(p.a, 0), v)}];")
-        for oi in self.used_out:
-            o = self.out[oi]
-            self.emit_record_load(E, [f"G{oi}_{k}" for k in range(o.D)],
-                                  f"G + rcvc * {self.D3} + {o.off} + {self.uclamp(o, 0)} * {o.D}", self.act(o), zero=True)
         for oi in self.used_out:
             o = self.out[oi]
             E("{")
@@ -177,6 +258,12 @@ class UVUDetGenerator(UVUDirectGenerator):
         for f in range(self.D2):
             E(f"    Ygr[{f}] = " + (f"dy{f};" if f in self.used_y else "(T)0;"))
         E("}")
+        if not self.prefetch_backward:
+            E("if (it + 1 < maxlen) {")
+            E.level += 1
+            load(E, "it + 1")
+            E.level -= 1
+            E("}")
         E.level -= 1
         E("}")
         E("rv = nv;")
@@ -185,9 +272,11 @@ class UVUDetGenerator(UVUDirectGenerator):
                 continue
             dst = f"Xg + node * {self.D1} + {a.off} + u * {a.D}"
             if a.idx in self.used_in1:
-                self.emit_record_store(E, [f"dx{a.idx}_{m}" for m in range(a.D)], dst, self.act(a))
+                dxs = [f"dx{a.idx}_{m}" for m in range(a.D)]
+                self.emit_sub_sum(E, dxs)
+                self.emit_record_store(E, dxs, dst, self.store_act(a))
             else:
-                self.emit_record_store(E, ["(T)0"] * a.D, dst, self.act(a))
+                self.emit_record_store(E, ["(T)0"] * a.D, dst, self.store_act(a))
         return E.text()
 
     def emit_dy_sum(self, E: Emitter) -> None:
