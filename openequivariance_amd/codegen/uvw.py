@@ -95,6 +95,8 @@ class UVWGenerator:
         self.shared = bool(problem.shared_weights)
         if not self.shared:
             raise NotImplementedError("uvw tensor products need shared_weights=True in this implementation")
+        import os
+        self.fwd_unroll = int(os.environ.get("OEQ_AMD_UVW_UNROLL", "4"))     # K steps issued per batch of loads
         self.in1, self.in2, self.out = _blocks(problem.irreps_in1), _blocks(problem.irreps_in2), _blocks(problem.irreps_out)
         self.D1, self.D2, self.D3 = problem.irreps_in1.dim, problem.irreps_in2.dim, problem.irreps_out.dim
         self.WN = problem.weight_numel
@@ -119,6 +121,15 @@ class UVWGenerator:
         self.used_in1 = sorted({p.a.idx for p in self.paths})
         self.used_out = sorted({p.o.idx for p in self.paths})
         self.used_y = sorted({p.b.off + j for p in self.paths for (_, j) in p.pairs})
+        # dW kernel: output blocks split into two groups of similar MFMA work
+        # (f64 accumulators are twice as wide: one group, four wavefronts, the whole register file)
+        work = {o: sum(p.o.D * p.NTW * p.NTU for p in self.paths if p.o.idx == o) for o in self.used_out}
+        self.dw_groups = 2 if (self.T == "float" and len(work) > 1) else 1
+        self.dw_group, load = {}, [0, 0]
+        for o in sorted(work, key=lambda k: -work[k]):
+            gsel = 0 if (load[0] <= load[1] or self.dw_groups == 1) else 1
+            self.dw_group[o] = gsel
+            load[gsel] += work[o]
         # packed weight copies in the workspace
         pos = 0
         for p in self.paths:
@@ -239,7 +250,7 @@ class UVWGenerator:
                     E(f"V4 acc{k}_{nt} = {{0, 0, 0, 0}};")
             for p in self.paths_into(o.idx):
                 E(f"// path {p.t}: l = {p.a.l} x {p.b.l} -> {p.o.l}, coefficient {p.coeff:.9g}")
-                E("#pragma unroll 4")
+                E(f"#pragma unroll {self.fwd_unroll}")
                 E(f"for (int s = 0; s < {p.SU}; ++s) {{")
                 E.level += 1
                 if p.mu % 4 == 0:
@@ -286,11 +297,15 @@ class UVWGenerator:
         for f in self.used_y:
             E(f"const T y{f} = Y[rowB * {self.D2} + {f}];")
             E(f"T dy{f} = (T)0;")
-        # dX accumulators of this wavefront: u-subtiles mt = wave + 4q
+        # X records and dX accumulators of this wavefront: u-subtiles mt = wave + 4q, rows r of the
+        # accumulator tile.  X is read once here for all paths that consume the block.
         for ai in self.used_in1:
             a = self.in1[ai]
             for q in range(_ceil(_ceil(a.mul, 16), 4)):
                 for r in range(4):
+                    uexp = f"16 * (wave + {4 * q}) + {self.row(r)}"
+                    E(f"const T* __restrict__ xp{ai}_{q}_{r} = Xr + {a.off} + min({uexp}, {a.mul - 1}) * {a.D};")
+                    E("const T " + ", ".join(f"x{ai}_{q}_{r}_{i} = xp{ai}_{q}_{r}[{i}]" for i in range(a.D)) + ";")
                     E("T " + ", ".join(f"dx{ai}_{q}_{r}_{i} = (T)0" for i in range(a.D)) + ";")
         for oi in self.used_out:
             o = self.out[oi]
@@ -318,16 +333,10 @@ class UVWGenerator:
                     for s in range(SW):
                         E(f"{{ const T a_ = ap[{s}]; " + " ".join(f"acc{k} = oeq_mfma(a_, gz{s}_{k}, acc{k});" for k in range(o.D)) + " }")
                     for r in range(4):
-                        E(f"{{ // row {r} of the tile: channel u, batch row b = row0 + c")
-                        if a.mul % 16 == 0:
-                            E(f"  const int u = 16 * mt + {self.row(r)};")
-                        else:
-                            E(f"  const int u = min(16 * mt + {self.row(r)}, {a.mul - 1});")
-                        E(f"  const T* __restrict__ xp = Xr + {a.off} + u * {a.D};")
-                        E("  const T " + ", ".join(f"x{i} = xp[{i}]" for i in range(a.D)) + ";")
+                        E(f"{{ // row {r} of the tile: channel u = 16 mt + row, batch row b = row0 + c")
                         E("  const T " + ", ".join(f"dt{k} = acc{k}[{r}]" for k in range(o.D)) + ";")
                         E.level += 1
-                        self.emit_cg_backward(E, p, "dt", "x", "y", f"dx{a.idx}_{q}_{r}_", "dy")
+                        self.emit_cg_backward(E, p, "dt", f"x{a.idx}_{q}_{r}_", "y", f"dx{a.idx}_{q}_{r}_", "dy")
                         E.level -= 1
                         E("}")
                     E.level -= 1
@@ -368,73 +377,85 @@ class UVWGenerator:
     # ============================================================ backward: dW
     def backward_dw_body(self) -> str:
         E = Emitter()
-        E("const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;")
+        # eight wavefronts: wave & 3 selects the 16-channel u-subtile, wave >> 2 one of two groups of
+        # output blocks (balanced by MFMA count), so that two wavefronts share each SIMD and cover
+        # each other's load latency while the accumulators of one group fit half the register file.
+        # Each group is a separate copy of the loop so that its accumulators are the only ones live.
+        E("const int lane = threadIdx.x & 63, wave = (threadIdx.x >> 6) & 3, grp = threadIdx.x >> 8, c = lane & 15, g = lane >> 4;")
         E("const u64 ntiles = (n + 15) / 16;")
-        for p in self.paths:
-            for q in range(_ceil(p.NTU, 4)):
-                for nt in range(p.NTW):
-                    E(f"V4 acc{p.t}_{q}_{nt} = {{0, 0, 0, 0}};")
-        E("for (u64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {")
-        E.level += 1
-        E("const u64 row0 = tile * 16;")
-        E("#pragma unroll 1")
-        E("for (int sp = 0; sp < 4; ++sp) {")
-        E.level += 1
-        E("const u64 b = row0 + 4 * sp + g;          // batch row of this lane for both operands")
-        E("const bool bv = b < n;")
-        E("const u64 bc = bv ? b : n - 1;")
-        E(f"const T* __restrict__ Xr = X + bc * {self.D1};")
-        E(f"const T* __restrict__ Gr = G + bc * {self.D3};")
-        for f in self.used_y:
-            E(f"const T y{f} = bv ? Y[bc * {self.D2} + {f}] : (T)0;     // zero rows past the end: T = 0 there")
-        # x records: u = 16 mt + c
-        for ai in self.used_in1:
-            a = self.in1[ai]
-            for q in range(_ceil(_ceil(a.mul, 16), 4)):
-                uexp = f"16 * (wave + {4 * q}) + c"
-                ucl = uexp if a.mul % 64 == 0 else f"min({uexp}, {a.mul - 1})"
-                E(f"const T* __restrict__ xp{ai}_{q} = Xr + {a.off} + ({ucl}) * {a.D};")
-                if a.mul % 64 == 0:
-                    E("const T " + ", ".join(f"x{ai}_{q}_{i} = xp{ai}_{q}[{i}]" for i in range(a.D)) + ";")
-                else:
-                    E("T " + ", ".join(f"x{ai}_{q}_{i} = xp{ai}_{q}[{i}]" for i in range(a.D)) + ";")
-                    E(f"if ({uexp} >= {a.mul}) {{ " + " ".join(f"x{ai}_{q}_{i} = (T)0;" for i in range(a.D)) + " }")
-        for oi in self.used_out:
-            o = self.out[oi]
-            NT = _ceil(o.mul, 16)
-            E(f"{{ // output block {oi}: dZ records, w = 16 nt + c")
+        E(f"T* __restrict__ part = (T*)ws + {self.PART_OFF} + (u64)blockIdx.x * {self.WN};")
+        for grp in range(self.dw_groups):
+            outs = [oi for oi in self.used_out if self.dw_group[oi] == grp]
+            paths = [p for p in self.paths if p.o.idx in outs]
+            ins = sorted({p.a.idx for p in paths})
+            ys = sorted({p.b.off + j for p in paths for (_, j) in p.pairs})
+            E(f"if (grp == {grp}) {{")
             E.level += 1
-            for nt in range(NT):
-                wexp = f"{16 * nt} + c"
-                wcl = wexp if o.mul % 16 == 0 else f"min({wexp}, {o.mul - 1})"
-                E(f"const T* __restrict__ gp{nt} = Gr + {o.off} + ({wcl}) * {o.D};")
-                E("const T " + ", ".join(f"gz{nt}_{k} = gp{nt}[{k}]" for k in range(o.D)) + ";")
-            for p in self.paths_into(oi):
+            for p in paths:
                 for q in range(_ceil(p.NTU, 4)):
-                    E(f"if (wave + {4 * q} < {p.NTU}) {{  // path {p.t}")
-                    E.level += 1
-                    self.emit_cg_forward(E, p, f"x{p.a.idx}_{q}_", "y", "t")
-                    for nt in range(NT):
-                        for k in range(o.D):
-                            E(f"acc{p.t}_{q}_{nt} = oeq_mfma(t{k}, gz{nt}_{k}, acc{p.t}_{q}_{nt});")
-                    E.level -= 1
+                    for nt in range(p.NTW):
+                        E(f"V4 acc{p.t}_{q}_{nt} = {{0, 0, 0, 0}};")
+            E("for (u64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {")
+            E.level += 1
+            E("const u64 row0 = tile * 16;")
+            E("#pragma unroll 1")
+            E("for (int sp = 0; sp < 4; ++sp) {")
+            E.level += 1
+            E("const u64 b = row0 + 4 * sp + g;          // batch row of this lane for both operands")
+            E("const bool bv = b < n;")
+            E("const u64 bc = bv ? b : n - 1;")
+            E(f"const T* __restrict__ Xr = X + bc * {self.D1};")
+            E(f"const T* __restrict__ Gr = G + bc * {self.D3};")
+            for f in ys:
+                E(f"const T y{f} = bv ? Y[bc * {self.D2} + {f}] : (T)0;     // zero rows past the end: T = 0 there")
+            for ai in ins:
+                a_ = self.in1[ai]
+                for q in range(_ceil(_ceil(a_.mul, 16), 4)):
+                    uexp = f"16 * (wave + {4 * q}) + c"
+                    ucl = uexp if a_.mul % 64 == 0 else f"min({uexp}, {a_.mul - 1})"
+                    E(f"const T* __restrict__ xp{ai}_{q} = Xr + {a_.off} + ({ucl}) * {a_.D};")
+                    if a_.mul % 64 == 0:
+                        E("const T " + ", ".join(f"x{ai}_{q}_{i} = xp{ai}_{q}[{i}]" for i in range(a_.D)) + ";")
+                    else:
+                        E("T " + ", ".join(f"x{ai}_{q}_{i} = xp{ai}_{q}[{i}]" for i in range(a_.D)) + ";")
+                        E(f"if ({uexp} >= {a_.mul}) {{ " + " ".join(f"x{ai}_{q}_{i} = (T)0;" for i in range(a_.D)) + " }")
+            for oi in outs:
+                o = self.out[oi]
+                NT = _ceil(o.mul, 16)
+                E(f"{{ // output block {oi}: dZ records, w = 16 nt + c")
+                E.level += 1
+                for nt in range(NT):
+                    wexp = f"{16 * nt} + c"
+                    wcl = wexp if o.mul % 16 == 0 else f"min({wexp}, {o.mul - 1})"
+                    E(f"const T* __restrict__ gp{nt} = Gr + {o.off} + ({wcl}) * {o.D};")
+                    E("const T " + ", ".join(f"gz{nt}_{k} = gp{nt}[{k}]" for k in range(o.D)) + ";")
+                for p in self.paths_into(oi):
+                    for q in range(_ceil(p.NTU, 4)):
+                        E(f"if (wave + {4 * q} < {p.NTU}) {{  // path {p.t}")
+                        E.level += 1
+                        self.emit_cg_forward(E, p, f"x{p.a.idx}_{q}_", "y", "t")
+                        for nt in range(NT):
+                            for k in range(o.D):
+                                E(f"acc{p.t}_{q}_{nt} = oeq_mfma(t{k}, gz{nt}_{k}, acc{p.t}_{q}_{nt});")
+                        E.level -= 1
+                        E("}")
+                E.level -= 1
+                E("}")
+            E.level -= 1
+            E("}")
+            E.level -= 1
+            E("}")
+            # ---- partial sums of this workgroup, laid out [t][u][w]
+            for p in paths:
+                for q in range(_ceil(p.NTU, 4)):
+                    E(f"if (wave + {4 * q} < {p.NTU}) {{")
+                    for nt in range(p.NTW):
+                        for r in range(4):
+                            E(f"    {{ const int u = 16 * (wave + {4 * q}) + {self.row(r)}; const int w = {16 * nt} + c;")
+                            E(f"      if (u < {p.mu} && w < {p.mw}) part[{p.woff} + u * {p.mw} + w] = acc{p.t}_{q}_{nt}[{r}]; }}")
                     E("}")
             E.level -= 1
             E("}")
-        E.level -= 1
-        E("}")
-        E.level -= 1
-        E("}")
-        # ---- partial sums of this workgroup, laid out [t][u][w]
-        E(f"T* __restrict__ part = (T*)ws + {self.PART_OFF} + (u64)blockIdx.x * {self.WN};")
-        for p in self.paths:
-            for q in range(_ceil(p.NTU, 4)):
-                E(f"if (wave + {4 * q} < {p.NTU}) {{")
-                for nt in range(p.NTW):
-                    for r in range(4):
-                        E(f"    {{ const int u = 16 * (wave + {4 * q}) + {self.row(r)}; const int w = {16 * nt} + c;")
-                        E(f"      if (u < {p.mu} && w < {p.mw}) part[{p.woff} + u * {p.mw} + w] = acc{p.t}_{q}_{nt}[{r}]; }}")
-                E("}")
         return E.text()
 
     def reduce_body(self) -> str:
@@ -467,6 +488,7 @@ class UVWGenerator:
                dict(kernel="forward", num_threads=64, grid_kind=ROW, work_per_block=16)]
         bwd = [dict(kernel="prep_backward", num_threads=256, grid_kind=FIXED, num_blocks=self.prep_blocks),
                dict(kernel="backward", num_threads=256, grid_kind=ROW, work_per_block=16),
-               dict(kernel="backward_dw", num_threads=256, grid_kind=FIXED, num_blocks=self.DW_WORKGROUPS),
+               dict(kernel="backward_dw", num_threads=256 * self.dw_groups, grid_kind=FIXED,
+                    num_blocks=self.DW_WORKGROUPS),
                dict(kernel="backward_reduce", num_threads=256, grid_kind=FIXED, num_blocks=_ceil(self.WN, 256))]
         return fwd, bwd, (lambda nnz=0, nodes=0: self.ws_elems * self.itemsize)
