@@ -36,6 +36,7 @@ class UVUDetGenerator(UVUDirectGenerator):
         if prefetch_backward is None and env in ("0", "1"):
             prefetch_backward = (env == "1")
         self.prefetch_backward = (words <= 56) if prefetch_backward is None else prefetch_backward
+        self.nontemporal = os.environ.get("OEQ_AMD_DET_NT", "1") == "1"   # streaming hint on W / Y / dW / dY
         self.uniform_rows = False          # validity is per lane (edge lists differ between sub-rows)
         self.chunk_in_grid = True
 
@@ -67,6 +68,12 @@ class UVUDetGenerator(UVUDirectGenerator):
         E("const int len = (int)(end - beg);")
         E(f"const int maxlen = (len + {R - 1}) / {R};")
         self.noderow_of = (lambda r: ("node", "nv"))
+
+    def ld(self, ptr: str, idx) -> str:
+        return f"oeq_ldnt({ptr} + {idx})" if self.nontemporal else f"{ptr}[{idx}]"
+
+    def st(self, ptr: str, idx, val: str) -> str:
+        return f"oeq_stnt({ptr} + {idx}, {val});" if self.nontemporal else f"{ptr}[{idx}] = {val};"
 
     def edge_pos(self, it: str) -> str:
         return f"(({it}) * {self.R} + sub)" if self.R > 1 else f"({it})"
@@ -119,7 +126,7 @@ class UVUDetGenerator(UVUDirectGenerator):
             E(f"const T* __restrict__ Yr = Y + e * {self.D2};")
             E(f"const T* __restrict__ Wr = W + e * {self.WN};")
             for f in self.used_y:
-                E(f"Ny{f} = Yr[{f}];")
+                E(f"Ny{f} = {self.ld('Yr', f)};")
             for i in self.used_in1:
                 a = self.in1[i]
                 E(f"{{ const T* __restrict__ p_ = X + sndc * {self.D1} + {a.off} + {self.uclamp(a, 0)} * {a.D}; "
@@ -128,7 +135,7 @@ class UVUDetGenerator(UVUDirectGenerator):
                 E(f"if (!({self.act(a)})) {{ " + " ".join(f"Nx{i}_{m} = (T)0;" for m in range(a.D)) + " }")
             for p in self.paths:
                 for v in range(p.mv):
-                    E(f"NWe_{p.t}_{v} = Wr[{self.widx(p, self.uclamp(p.a, 0), v)}];")
+                    E(f"NWe_{p.t}_{v} = {self.ld('Wr', self.widx(p, self.uclamp(p.a, 0), v))};")
             E.level -= 1
             E("}")
         E("if (maxlen > 0) {")
@@ -206,10 +213,10 @@ class UVUDetGenerator(UVUDirectGenerator):
             E(f"const T* __restrict__ Yr = Y + e * {self.D2};")
             E(f"const T* __restrict__ Wr = W + e * {self.WN};")
             for f in self.used_y:
-                E(f"Ny{f} = Yr[{f}];")
+                E(f"Ny{f} = {self.ld('Yr', f)};")
             for p in self.paths:
                 for v in range(p.mv):
-                    E(f"NWe_{p.t}_{v} = Wr[{self.widx(p, self.uclamp(p.a, 0), v)}];")
+                    E(f"NWe_{p.t}_{v} = {self.ld('Wr', self.widx(p, self.uclamp(p.a, 0), v))};")
             for oi in self.used_out:
                 o = self.out[oi]
                 E(f"{{ const T* __restrict__ p_ = G + rcvc * {self.D3} + {o.off} + {self.uclamp(o, 0)} * {o.D}; "
@@ -244,7 +251,7 @@ class UVUDetGenerator(UVUDirectGenerator):
                 E(f"const T g{k} = G{oi}_{k};")
 
             def sink(E, p, v, expr):
-                E(f"  if ({self.act(p.a)}) Wgr[{self.widx(p, 'u', v)}] = {expr};")
+                E(f"  if ({self.act(p.a)}) {self.st('Wgr', self.widx(p, 'u', v), expr)}")
             self.emit_backward_block(E, o, "Wr", sink)
             E.level -= 1
             E("}")

@@ -63,6 +63,8 @@ static inline void oeq_dma16(const T* g, T* lds_base) { memcpy((char*)lds_base +
 static inline void oeq_wait_vm() {}
 static inline void oeq_wait_lds() {}
 static inline T oeq_wave_sum63(T v) { g_xT[threadIdx.x] = v; oeq_sync(); T t = 0; for (int i = 0; i < 64; ++i) t += g_xT[(threadIdx.x & ~63) + i]; oeq_sync(); return t; }
+static inline T oeq_ldnt(const T* p) { return *p; }
+static inline void oeq_stnt(T* p, T v) { *p = v; }
 static inline void oeq_block_sync() { pthread_barrier_wait(&g_bar); }
 // matrix-core step of one wavefront, emulated collectively by its 64 threads
 struct V4 { T v[4]; T& operator[](int i) { return v[i]; } const T& operator[](int i) const { return v[i]; } };
