@@ -93,8 +93,8 @@ class UVWGenerator:
         self.T = {np.float32: "float", np.float64: "double"}[problem.irrep_dtype]
         self.itemsize = 4 if self.T == "float" else 8
         self.shared = bool(problem.shared_weights)
-        if not self.shared:
-            raise NotImplementedError("uvw tensor products need shared_weights=True in this implementation")
+        if not self.shared and not getattr(self, "_allow_batched", False):
+            raise NotImplementedError("this generator handles shared weights; see uvw_batched.py for per-row weights")
         import os
         self.fwd_unroll = int(os.environ.get("OEQ_AMD_UVW_UNROLL", "4"))     # K steps issued per batch of loads
         self.in1, self.in2, self.out = _blocks(problem.irreps_in1), _blocks(problem.irreps_in2), _blocks(problem.irreps_out)

@@ -76,9 +76,12 @@ class TensorProduct(TensorProductBase):
         config = self.config
         mode = validate_problem(config)
         self.is_uvw = (mode == "uvw")
-        if self.is_uvw:
+        if self.is_uvw and config.shared_weights:
             from .codegen.uvw import UVWGenerator
             self.generator = UVWGenerator(config)
+        elif self.is_uvw:
+            from .codegen.uvw_batched import UVWBatchedGenerator
+            self.generator = UVWBatchedGenerator(config)
         elif config.shared_weights or schedule() == "lds":
             self.generator = UVUGenerator(config, "tp")
         else:

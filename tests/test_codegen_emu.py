@@ -6,6 +6,7 @@ import pytest
 
 import openequivariance_amd as oeq
 from openequivariance_amd.codegen.uvu import UVUGenerator
+from openequivariance_amd.codegen.uvu_det import UVUDetGenerator
 from openequivariance_amd.codegen.uvu_direct import UVUDirectGenerator
 from openequivariance_amd.codegen.uvw import UVWGenerator
 from host_emu import emu
@@ -59,7 +60,7 @@ def test_generic_tp_shared_weights():
 @pytest.mark.parametrize("det", [False, True])
 def test_conv(det):
     prob, oprob = common.channelwise(common.NEQUIP)
-    g = UVUGenerator(prob, "conv_det") if det else UVUDirectGenerator(prob, "conv_atomic")
+    g = UVUDetGenerator(prob) if det else UVUDirectGenerator(prob, "conv_atomic")
     nodes, nnz = 7, 19
     rows, cols = common.random_graph(nodes, nnz, 5)
     tperm = None
@@ -77,7 +78,7 @@ def test_conv(det):
 def test_conv_det_chunked_ragged():
     irreps = ("5x0e+3x1o+70x2e", "1x0e+1x1o+1x2e", "5x0e+3x1o+70x2e+7x3o")
     prob, oprob = common.channelwise(irreps)
-    g = UVUGenerator(prob, "conv_det")
+    g = UVUDetGenerator(prob)
     nodes, nnz = 5, 11
     rows, cols, tperm, _ = otp.coord_graph(*common.random_graph(nodes, nnz, 7))
     X, Y, W, G = common.conv_inputs(prob, nodes, nnz, 8)
@@ -105,3 +106,19 @@ def test_uvw_matrix_core_kernels(dtype, monkeypatch):
     dX, dY, dW = otp.backward(oprob, X, Y, We, G)
     assert rel_err(out["Xg"], dX) < tol and rel_err(out["Yg"], dY) < tol
     assert rel_err(ow.oeq_to_e3nn(oprob, out["Wg"]), dW) < tol
+
+
+def test_uvw_per_row_weights():
+    from openequivariance_amd.codegen.uvw_batched import UVWBatchedGenerator
+    a = ("5x0e+21x1o", "1x0e+1x1o+1x2e", "18x0e+7x1o+3x2e")
+    prob, oprob = common.fully_connected(a, shared=False)
+    g = UVWBatchedGenerator(prob)
+    X, Y, We, G = common.tp_inputs(prob, 5, 10, w_scale=0.3)
+    W = ow.e3nn_to_oeq(oprob, We)
+    fwd, bwd, ws = g.plan()
+    out = emu.run_tp(g, fwd, X, Y, W)
+    assert rel_err(out["Z"], otp.forward(oprob, X, Y, We)) < TOL
+    out = emu.run_tp(g, bwd, X, Y, W, G)
+    dX, dY, dW = otp.backward(oprob, X, Y, We, G)
+    assert rel_err(out["Xg"], dX) < TOL and rel_err(out["Yg"], dY) < TOL
+    assert rel_err(ow.oeq_to_e3nn(oprob, out["Wg"]), dW) < TOL

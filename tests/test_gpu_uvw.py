@@ -86,9 +86,50 @@ def test_dw_bit_reproducible_and_full_batch(cuda):
 
 def test_uvw_unsupported_cases_raise(cuda):
     import openequivariance_amd as oeq
-    prob, _ = common.fully_connected(("4x0e", "2x0e", "4x0e"), shared=True)
-    with pytest.raises(NotImplementedError):
-        oeq.TensorProduct(prob, torch_op=True)
-    prob, _ = common.fully_connected(("4x0e", "1x0e", "4x0e"), shared=False)
-    with pytest.raises(NotImplementedError):
-        oeq.TensorProduct(prob, torch_op=True)
+    for shared in (True, False):
+        prob, _ = common.fully_connected(("4x0e", "2x0e", "4x0e"), shared=shared)
+        with pytest.raises(NotImplementedError):
+            oeq.TensorProduct(prob, torch_op=True)
+
+
+DIFFDOCK = {"DiffDock-L=1": ("10x1o+10x1e+48x0e+48x0o", "1x0e+1x1o", "10x1o+10x1e+48x0e+48x0o"),
+            "DiffDock-L=2": ("10x1o+10x1e+48x0e+48x0o", "1x0e+1x1o+1x2e", "10x1o+10x1e+48x0e+48x0o")}
+
+
+@pytest.mark.parametrize("name", list(DIFFDOCK))
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_uvw_per_row_weights_diffdock(cuda, name, dtype):
+    """uvw with shared_weights=False (reference: benchmark/benchmark_configs.py:44-48)."""
+    import torch
+    import openequivariance_amd as oeq
+    tol = FP32_TOL if dtype == np.float32 else FP64_TOL
+    prob, oprob = common.fully_connected(DIFFDOCK[name], shared=False, dtype=dtype)
+    X, Y, We, G = common.tp_inputs(prob, 129, 45, dtype, w_scale=0.2)
+    tp = oeq.TensorProduct(prob, torch_op=True)
+    W = ow.e3nn_to_oeq(oprob, We)
+    x, y, w = (torch.tensor(a, device=cuda, requires_grad=True) for a in (X, Y, W))
+    z = tp(x, y, w)
+    z.backward(torch.tensor(G, device=cuda))
+    dXr, dYr, dWr = otp.backward(oprob, X, Y, We, G)
+    assert rel_err(z.detach().cpu().numpy(), otp.forward(oprob, X, Y, We)) <= tol
+    assert rel_err(x.grad.cpu().numpy(), dXr) <= tol
+    assert rel_err(y.grad.cpu().numpy(), dYr) <= tol
+    assert rel_err(ow.oeq_to_e3nn(oprob, w.grad.cpu().numpy()), dWr) <= tol
+
+
+def test_uvw_per_row_weights_wide(cuda):
+    """Multiplicities above 64 on both sides (several lane chunks), ragged 32-blocks in the weight order."""
+    import torch
+    import openequivariance_amd as oeq
+    prob, oprob = common.fully_connected(("70x0e+40x1o", "1x0e+1x1o", "66x0e+33x1o"), shared=False)
+    X, Y, We, G = common.tp_inputs(prob, 33, 46, w_scale=0.2)
+    tp = oeq.TensorProduct(prob, torch_op=True)
+    W = ow.e3nn_to_oeq(oprob, We)
+    x, y, w = (torch.tensor(a, device=cuda, requires_grad=True) for a in (X, Y, W))
+    z = tp(x, y, w)
+    z.backward(torch.tensor(G, device=cuda))
+    dXr, dYr, dWr = otp.backward(oprob, X, Y, We, G)
+    assert rel_err(z.detach().cpu().numpy(), otp.forward(oprob, X, Y, We)) <= FP32_TOL
+    assert rel_err(x.grad.cpu().numpy(), dXr) <= FP32_TOL
+    assert rel_err(y.grad.cpu().numpy(), dYr) <= FP32_TOL
+    assert rel_err(ow.oeq_to_e3nn(oprob, w.grad.cpu().numpy()), dWr) <= FP32_TOL

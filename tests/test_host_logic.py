@@ -39,7 +39,8 @@ def test_launch_plans():
     prob, _ = common.channelwise(common.NEQUIP)
     assert UVUDirectGenerator(prob, "tp").plan()[0][0]["work_per_block"] == 2       # two rows per wavefront
     prob, _ = common.channelwise(common.LARGE)
-    g = UVUGenerator(prob, "conv_det")
+    from openequivariance_amd.codegen.uvu_det import UVUDetGenerator
+    g = UVUDetGenerator(prob)
     fwd, bwd, ws = g.plan()
     assert [s["kernel"] for s in fwd] == ["prep_forward", "forward"] and fwd[1]["grid_y"] == 4
     assert [s["kernel"] for s in bwd] == ["prep_backward", "backward", "backward_dy_reduce"]
