@@ -173,6 +173,11 @@ class UVUGenerator:
     def lit(self, v: float) -> str:
         return literal(v, self.T)
 
+    def backward_attr(self) -> str:
+        """Extra kernel attributes of the backward kernel (occupancy hint)."""
+        w = getattr(self, "waves_per_eu", 0)
+        return f" __attribute__((amdgpu_waves_per_eu({w})))" if w else ""
+
     def widx(self, p: Path, u: str, v: int) -> str:
         """oeq-order position of weight (u, v) of path ``p`` (see weight_order.py)."""
         mu, mv = p.mu, p.mv

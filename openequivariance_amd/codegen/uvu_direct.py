@@ -33,7 +33,8 @@ class UVUDirectGenerator(UVUGenerator):
         super().__init__(problem, kind)
         if (kind == "conv_det" and not getattr(self, "_allow_det", False)) or self.shared:
             raise NotImplementedError("direct schedule: batch product with per-row weights and atomic convolution")
-        self.waves_per_eu = waves_per_eu
+        import os
+        self.waves_per_eu = waves_per_eu or int(os.environ.get("OEQ_AMD_WAVES_PER_EU", "0"))
         # False: outputs are written with dword-aligned record stores only (for callers whose
         # output tensor is not 16-byte aligned)
         self.vector_stores = vector_stores
@@ -338,12 +339,20 @@ class UVUDirectGenerator(UVUGenerator):
             chunk(E, "c")
             E.level -= 1
             E("}")
-        self.emit_dy_reduce(E)
+        # dY: sum over the lanes of the row in a fixed order (DPP row operations when a row fills the
+        # wavefront - the total lands in lane 63 - else the xor butterfly, total in every lane)
+        if self.P == 64:
+            for f in self.used_y:
+                E(f"dy{f} = oeq_wave_sum63(dy{f});")
+            writer = "lane == 63"
+        else:
+            self.emit_dy_reduce(E)
+            writer = "ul == 0"
         if self.kind == "tp":
-            E("if (rv && ul == 0) {")
+            E(f"if (rv && {writer}) {{")
             E(f"    T* __restrict__ Ygr = Yg + row * {self.D2};")
         else:
-            E("if (e < nnz && ul == 0) {")
+            E(f"if (e < nnz && {writer}) {{")
             E(f"    T* __restrict__ Ygr = Yg + e * {self.D2};")
         for f in range(self.D2):
             E(f"    Ygr[{f}] = " + (f"dy{f};" if f in self.used_y else "(T)0;"))

@@ -96,7 +96,11 @@ class UVWGenerator:
         if not self.shared and not getattr(self, "_allow_batched", False):
             raise NotImplementedError("this generator handles shared weights; see uvw_batched.py for per-row weights")
         import os
-        self.fwd_unroll = int(os.environ.get("OEQ_AMD_UVW_UNROLL", "4"))     # K steps issued per batch of loads
+        # forward K loop: steps fetched per batch of loads, and unroll factor of the batch loop
+        # (measured on MI355X: fp32 4 / 1, fp64 1 / 3)
+        dflt = ("4", "1") if self.T == "float" else ("1", "3")
+        self.fwd_group = int(os.environ.get("OEQ_AMD_UVW_GROUP", dflt[0]))
+        self.fwd_unroll = int(os.environ.get("OEQ_AMD_UVW_UNROLL", dflt[1]))
         self.in1, self.in2, self.out = _blocks(problem.irreps_in1), _blocks(problem.irreps_in2), _blocks(problem.irreps_out)
         self.D1, self.D2, self.D3 = problem.irreps_in1.dim, problem.irreps_in2.dim, problem.irreps_out.dim
         self.WN = problem.weight_numel
@@ -121,6 +125,8 @@ class UVWGenerator:
         self.used_in1 = sorted({p.a.idx for p in self.paths})
         self.used_out = sorted({p.o.idx for p in self.paths})
         self.used_y = sorted({p.b.off + j for p in self.paths for (_, j) in p.pairs})
+        cost = lambda o: sum(p.o.D * p.NTW * p.SU for p in self.paths if p.o.idx == o.idx)
+        self.fwd_order = sorted([o for o in self.out if o.dim > 0], key=lambda o: -cost(o))
         # dW kernel: output blocks split into two groups of similar MFMA work
         # (f64 accumulators are twice as wide: one group, four wavefronts, the whole register file)
         work = {o: sum(p.o.D * p.NTW * p.NTU for p in self.paths if p.o.idx == o) for o in self.used_out}
@@ -233,11 +239,12 @@ class UVWGenerator:
         E(f"const T* __restrict__ Xr = X + rowA * {self.D1};")
         for f in self.used_y:
             E(f"const T y{f} = Y[rowA * {self.D2} + {f}];")
-        for o in self.out:
-            if o.dim == 0:
-                continue
+        # One work item = (batch tile, output block): blockIdx.y walks the output blocks from the most
+        # to the least expensive, so the dispatcher fills the tail of the launch with the cheap ones
+        # (whole tiles per wavefront leave a third of the machine idle in the last round).
+        for slot, o in enumerate(self.fwd_order):
             NT = _ceil(o.mul, 16)
-            E(f"{{ // output block {o.idx}: {o.mul}x l={o.l}")
+            E(f"if (blockIdx.y == {slot}) {{ // output block {o.idx}: {o.mul}x l={o.l}")
             E.level += 1
             if o.idx not in self.used_out:
                 for r in range(4):
@@ -249,25 +256,51 @@ class UVWGenerator:
                 for nt in range(NT):
                     E(f"V4 acc{k}_{nt} = {{0, 0, 0, 0}};")
             for p in self.paths_into(o.idx):
-                E(f"// path {p.t}: l = {p.a.l} x {p.b.l} -> {p.o.l}, coefficient {p.coeff:.9g}")
-                E(f"#pragma unroll {self.fwd_unroll}")
-                E(f"for (int s = 0; s < {p.SU}; ++s) {{")
+                E(f"{{ // path {p.t}: l = {p.a.l} x {p.b.l} -> {p.o.l}, coefficient {p.coeff:.9g}")
                 E.level += 1
-                if p.mu % 4 == 0:
-                    E("const int u = 4 * s + g;")
-                else:
-                    E("const int uu = 4 * s + g;")
-                    E(f"const int u = min(uu, {p.mu - 1});")
-                E(f"const T* __restrict__ xp = Xr + {p.a.off} + u * {p.a.D};")
-                E("const T " + ", ".join(f"x{i} = xp[{i}]" for i in range(p.a.D)) + ";")
-                self.emit_cg_forward(E, p, "x", "y", "t")
-                if p.mu % 4 != 0:
-                    E(f"if (uu >= {p.mu}) {{ " + " ".join(f"t{k} = (T)0;" for k in range(o.D)) + " }")
-                E(f"const T* __restrict__ bp = wsT + {p.wb} + (s * 64 + lane) * {NT};")
-                E("const T " + ", ".join(f"b{nt} = bp[{nt}]" for nt in range(NT)) + ";")
-                for k in range(o.D):
-                    for nt in range(NT):
-                        E(f"acc{k}_{nt} = oeq_mfma(t{k}, b{nt}, acc{k}_{nt});")
+                # The K loop runs in groups of GS steps, software pipelined: the X records and weight
+                # slices of the next group are in flight while this group runs on the VALU and the
+                # matrix core.  What bounds this kernel is the L2 -> L1 stream of operands (every
+                # wavefront re-reads the packed weights), so the bytes in flight per wavefront matter
+                # more than anything else here.
+                GS = self.fwd_group
+                NG = _ceil(p.SU, GS)
+                regs = [f"nx{j}_{i}" for j in range(GS) for i in range(p.a.D)] + [f"nb{j}_{nt}" for j in range(GS) for nt in range(NT)]
+                E("T " + ", ".join(regs) + ";")
+
+                def load(E, gexp):
+                    for j in range(GS):
+                        sexp = f"({gexp}) * {GS} + {j}"
+                        need_clamp = (NG * GS != p.SU)
+                        scl = f"min({sexp}, {p.SU - 1})" if need_clamp else sexp
+                        uexp = f"4 * ({sexp}) + g"
+                        ucl = uexp if (p.mu % 4 == 0 and not need_clamp) else f"min({uexp}, {p.mu - 1})"
+                        E(f"{{ const T* __restrict__ xp = Xr + {p.a.off} + ({ucl}) * {p.a.D}; " + " ".join(f"nx{j}_{i} = xp[{i}];" for i in range(p.a.D)))
+                        E(f"  const T* __restrict__ bp = wsT + {p.wb} + (({scl}) * 64 + lane) * {NT}; " + " ".join(f"nb{j}_{nt} = bp[{nt}];" for nt in range(NT)) + " }")
+                load(E, "0")
+                E(f"#pragma unroll {self.fwd_unroll}")
+                E(f"for (int sg = 0; sg < {NG}; ++sg) {{")
+                E.level += 1
+                E("const T " + ", ".join(f"c{r} = {r}" for r in regs) + ";")
+                E(f"if (sg + 1 < {NG}) {{")
+                E.level += 1
+                load(E, "sg + 1")
+                E.level -= 1
+                E("}")
+                for j in range(GS):
+                    E("{")
+                    E.level += 1
+                    E("const T " + ", ".join(f"x{i} = cnx{j}_{i}" for i in range(p.a.D)) + ";")
+                    self.emit_cg_forward(E, p, "x", "y", "t")
+                    if p.mu % 4 != 0 or NG * GS != p.SU:
+                        E(f"if (4 * (sg * {GS} + {j}) + g >= {p.mu}) {{ " + " ".join(f"t{k} = (T)0;" for k in range(o.D)) + " }")
+                    for k in range(o.D):
+                        for nt in range(NT):
+                            E(f"acc{k}_{nt} = oeq_mfma(t{k}, cnb{j}_{nt}, acc{k}_{nt});")
+                    E.level -= 1
+                    E("}")
+                E.level -= 1
+                E("}")
                 E.level -= 1
                 E("}")
             # lane holds, for each of its 4 rows, w = NT*c + nt (nt < NT) and all k: a contiguous run
@@ -485,7 +518,7 @@ class UVWGenerator:
     def plan(self):
         FIXED, ROW = 0, 1
         fwd = [dict(kernel="prep_forward", num_threads=256, grid_kind=FIXED, num_blocks=self.prep_blocks),
-               dict(kernel="forward", num_threads=64, grid_kind=ROW, work_per_block=16)]
+               dict(kernel="forward", num_threads=64, grid_kind=ROW, work_per_block=16, grid_y=len(self.fwd_order))]
         bwd = [dict(kernel="prep_backward", num_threads=256, grid_kind=FIXED, num_blocks=self.prep_blocks),
                dict(kernel="backward", num_threads=256, grid_kind=ROW, work_per_block=16),
                dict(kernel="backward_dw", num_threads=256 * self.dw_groups, grid_kind=FIXED,
