@@ -32,6 +32,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="mace_uvu")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-cold", action="store_true", help="skip the flushed-cache timing leg")
     ap.add_argument("--cpu-sample", type=int, default=0, help="edges in the CPU sample (0 = automatic)")
     return ap.parse_args()
 
@@ -52,9 +53,20 @@ class Events:
         b.record()
         self.pairs.setdefault(name, []).append((a, b))
 
+    def times_ms(self, name):
+        return [a.elapsed_time(b) for a, b in self.pairs.get(name, [])]
+
     def mean_ms(self, name):
-        v = [a.elapsed_time(b) for a, b in self.pairs.get(name, [])]
+        v = self.times_ms(name)
         return sum(v) / len(v) if v else float("nan")
+
+    def median_min_ms(self, name):
+        v = sorted(self.times_ms(name))
+        if not v:
+            return float("nan"), float("nan")
+        mid = len(v) // 2
+        med = v[mid] if len(v) % 2 else 0.5 * (v[mid - 1] + v[mid])
+        return med, v[0]
 
 
 def load_traffic(key):
@@ -195,6 +207,27 @@ def main():
     else:
         tot = wl.alg_flops["forward"] + wl.alg_flops["backward"]
         roofline["fwd_bwd_frac"] = round(tot / ((fwd_ms + bwd_ms) * 1e-3) / 1e12 / peak, 4)
+
+    if not args.no_cold:
+        # second leg, outside the timed region: the same launches with the caches flushed before
+        # each one (a 512 MiB fill, twice the 256 MiB Infinity Cache), the protocol of the reference's
+        # timers (openequivariance/extension/util/backend_hip.hpp:65-99 clears a 100 MB buffer)
+        flush = torch.empty(512 << 20, dtype=torch.uint8, device=dev)
+        for _ in range(min(args.steps, 30)):
+            flush.fill_(1)
+            ev.wrap("forward_cold", case.forward)
+            flush.fill_(2)
+            ev.wrap("backward_cold", case.backward)
+        torch.cuda.synchronize()
+        del flush
+        fm, fmin = ev.median_min_ms("forward_cold")
+        bm, bmin = ev.median_min_ms("backward_cold")
+        work = wl.alg_bytes if wl.bound == "hbm" else wl.alg_flops
+        scale = 1e9 if wl.bound == "hbm" else 1e12
+        roofline["flushed_caches"] = {
+            "forward_ms_median": round(fm, 5), "forward_ms_min": round(fmin, 5),
+            "backward_ms_median": round(bm, 5), "backward_ms_min": round(bmin, 5),
+            "fwd_bwd_frac": round((work["forward"] + work["backward"]) / ((fm + bm) * 1e-3) / scale / peak, 4)}
 
     cpu = None
     if not args.no_cpu:

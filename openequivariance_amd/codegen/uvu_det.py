@@ -26,8 +26,8 @@ from .uvu_direct import UVUDirectGenerator
 class UVUDetGenerator(UVUDirectGenerator):
     _allow_det = True
 
-    def __init__(self, problem: TPProblem, prefetch_backward=None):
-        super().__init__(problem, "conv_det")
+    def __init__(self, problem: TPProblem, prefetch_backward=None, vector_stores: bool = True):
+        super().__init__(problem, "conv_det", vector_stores=vector_stores)
         # fetch the next edge's operands while the current edge is being computed; pays when the
         # per-edge register footprint is small enough to keep several wavefronts per SIMD
         words = sum(self.out[i].D for i in self.used_out) + len(self.paths) + len(self.used_y)

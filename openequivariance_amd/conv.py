@@ -21,12 +21,10 @@ import numpy as np
 import torch
 
 from . import runtime as rt
-from .codegen.uvu import UVUGenerator
 from .codegen.uvu_det import UVUDetGenerator
 from .codegen.uvu_direct import UVUDirectGenerator
-from .codegen.uvu_fast import UVUFastGenerator
 from .problem import TPProblem
-from .tensor_product import _make_steps, schedule, validate_problem
+from .tensor_product import _make_steps, validate_problem
 from .weight_order import WeightReorder
 from .wigner import wigner_3j
 
@@ -71,6 +69,30 @@ class CoordGraph:
         self.transpose_perm = np.lexsort((np.arange(self.nnz), self.rows, self.cols)).astype(self.rows.dtype)
 
 
+def sort_by_receiver(rows: "torch.Tensor", cols: "torch.Tensor", node_count: typing.Optional[int] = None):
+    """Graph preparation for ``deterministic=True`` on the tensors' own device (no torch_geometric):
+    returns ``(rows_sorted, cols_sorted, receiver_perm, transpose_perm)`` where ``receiver_perm``
+    sorts the edges by (receiver, sender) - apply it to the per-edge tensors Y and W - and
+    ``transpose_perm`` lists the sorted edges in (sender, receiver) order, the last argument of
+    ``TensorProductConv.forward``.  Same result as ``CoordGraph`` (reference:
+    convolution/ConvolutionBase.py:45-70) and as the ``sort_by`` recipe of the reference's README
+    (README.md:110-118); both sorts are stable, so the permutations are unique."""
+    assert rows.dtype == torch.int64 and cols.dtype == torch.int64 and rows.shape == cols.shape and rows.dim() == 1
+    if rows.numel() == 0:
+        return rows, cols, rows.clone(), rows.clone()
+    n = int(node_count) if node_count is not None else int(torch.maximum(rows.max(), cols.max()).item()) + 1
+    receiver_perm = torch.argsort(rows * n + cols, stable=True)
+    rows_s, cols_s = rows[receiver_perm], cols[receiver_perm]
+    transpose_perm = torch.argsort(cols_s * n + rows_s, stable=True)
+    return rows_s, cols_s, receiver_perm, transpose_perm
+
+
+def select_conv_generator(config: TPProblem, deterministic: bool):
+    """Kernel generator of the fused convolution: one node per wavefront with fixed summation order
+    when deterministic, register-direct kernels with coalesced atomics otherwise."""
+    return UVUDetGenerator(config) if deterministic else UVUDirectGenerator(config, "conv_atomic")
+
+
 class TensorProductConv:
     """Drop-in for ``oeq.TensorProductConv``."""
     next_conv_id = 0
@@ -93,25 +115,14 @@ class TensorProductConv:
         if mode != "uvu":
             raise NotImplementedError("TensorProductConv supports uvu problems")
 
-        if deterministic and schedule() != "lds":
-            self.generator = UVUDetGenerator(config)
-        elif schedule() == "lds":
-            self.generator = UVUGenerator(config, "conv_det" if deterministic else "conv_atomic")
-        else:
-            self.generator = UVUDirectGenerator(config, "conv_atomic")
+        self.generator = select_conv_generator(config, deterministic)
         self.jit_kernel = self.generator.render()
         code = rt.compile_source(self.jit_kernel)
         fwd, bwd, self._ws_bytes = self.generator.plan()
         self.internal = rt.ConvImpl(code, _make_steps(fwd), _make_steps(bwd))
         self.workspace_buffer = None
         self.workspace_size = 0
-        self.internal_fast = None
-        kind = self.generator.kind
-        if schedule() == "lds" and UVUFastGenerator.eligible(config, kind):
-            self.generator_fast = UVUFastGenerator(config, kind)
-            ffwd, fbwd, _ = self.generator_fast.plan()
-            self.internal_fast = rt.ConvImpl(rt.compile_source(self.generator_fast.render()),
-                                             _make_steps(ffwd), _make_steps(fbwd))
+        self._internal_unaligned = None
         self._reorder = WeightReorder(config)
         self.reorder_weights_e3nn_to_oeq = self._reorder.e3nn_to_oeq
         self.reorder_weights_oeq_to_e3nn = self._reorder.oeq_to_e3nn
@@ -156,10 +167,15 @@ class TensorProductConv:
             raise TypeError(f"tensors must be {tdt}")
 
     def _pick(self, *ptrs):
-        # (the register-direct atomic kernels have no alignment requirement: they store with
-        # scalar atomics and dword stores only)
-        if self.internal_fast is not None and all(int(p) % 16 == 0 for p in ptrs):
-            return self.internal_fast
+        """The atomic kernels use dword accesses only; the deterministic forward writes Z with 16-byte
+        vector stores and falls back to a variant without them for a misaligned tensor (rare: a view
+        with an odd storage offset)."""
+        if self.deterministic and any(int(p) % 16 for p in ptrs):
+            if self._internal_unaligned is None:
+                g = UVUDetGenerator(self.config, vector_stores=False)
+                fwd, bwd, _ = g.plan()
+                self._internal_unaligned = rt.ConvImpl(rt.compile_source(g.render()), _make_steps(fwd), _make_steps(bwd))
+            return self._internal_unaligned
         return self.internal
 
     # ---------------------------------------------------------- raw entry points

@@ -11,41 +11,26 @@ import time
 import numpy as np
 
 from . import runtime as rt
-from .codegen.uvu import UVUGenerator
-from .codegen.uvu_det import UVUDetGenerator
-from .codegen.uvu_direct import UVUDirectGenerator
-from .codegen.uvu_fast import UVUFastGenerator
+from .conv import select_conv_generator
 from .problem import ChannelwiseTPP, FullyConnectedTPProblem, TPProblem
-
-MACE = ("128x0e+128x1o+128x2e", "1x0e+1x1o+1x2e+1x3o", "128x0e+128x1o+128x2e+128x3o")
-NEQUIP = ("32x0e+32x1o+32x2e", "1x0e+1x1o+1x2e", "32x0e+32x1o+32x2e")
-LARGE = ("256x0e+256x1o+256x2e", "1x0e+1x1o+1x2e+1x3o", "256x0e+256x1o+256x2e")
-DENSE = ("64x0e+64x1o+64x2e", "1x0e+1x1o+1x2e", "64x0e+64x1o+64x2e")
+from .tensor_product import select_generator
+from .workloads import DENSE, LARGE, MACE, MACE_ALL, NEQUIP
 
 
 def benchmark_generators():
+    """(label, generator) for every kernel set the benchmark workloads and the smoke test use,
+    chosen by the same selection functions as the operators."""
     readme = TPProblem("1x2e", "1x3e", "1x2e", [(0, 0, 0, "uvu", True)], shared_weights=False, internal_weights=False)
-    gens = [("readme/tp", UVUGenerator(readme, "tp")),
-            ("mace/tp", UVUGenerator(ChannelwiseTPP(*MACE), "tp")),
-            ("nequip/tp", UVUGenerator(ChannelwiseTPP(*NEQUIP), "tp")),
-            ("nequip/conv_atomic", UVUGenerator(ChannelwiseTPP(*NEQUIP), "conv_atomic")),
-            ("nequip/conv_det", UVUGenerator(ChannelwiseTPP(*NEQUIP), "conv_det")),
-            ("large/conv_atomic", UVUGenerator(ChannelwiseTPP(*LARGE), "conv_atomic")),
-            ("large/conv_det", UVUGenerator(ChannelwiseTPP(*LARGE), "conv_det"))]
-    for name, g in list(gens):
-        if g.kind != "conv_det" and not g.shared:
-            gens.append((name + "/direct", UVUDirectGenerator(g.problem, g.kind)))
-        elif g.kind == "conv_det":
-            gens.append((name + "/direct", UVUDetGenerator(g.problem)))
-    try:
-        from .codegen.uvw import UVWGenerator
-    except ImportError:
-        UVWGenerator = None
-    if UVWGenerator is not None:
-        for dt in (np.float32, np.float64):
-            p = FullyConnectedTPProblem(*DENSE, shared_weights=True, internal_weights=False,
-                                        irrep_dtype=dt, weight_dtype=dt)
-            gens.append((f"dense/uvw/{np.dtype(dt).name}", UVWGenerator(p)))
+    gens = [("readme/tp", select_generator(readme)),
+            ("mace/tp", select_generator(ChannelwiseTPP(*MACE))),
+            ("mace-all-parities/tp", select_generator(ChannelwiseTPP(*MACE_ALL))),
+            ("nequip/tp", select_generator(ChannelwiseTPP(*NEQUIP)))]
+    for label, irreps in (("nequip", NEQUIP), ("large", LARGE)):
+        for det in (False, True):
+            gens.append((f"{label}/conv_{'det' if det else 'atomic'}", select_conv_generator(ChannelwiseTPP(*irreps), det)))
+    for dt in (np.float32, np.float64):
+        p = FullyConnectedTPProblem(*DENSE, shared_weights=True, internal_weights=False, irrep_dtype=dt, weight_dtype=dt)
+        gens.append((f"dense/uvw/{np.dtype(dt).name}", select_generator(p)))
     return gens
 
 

@@ -18,7 +18,6 @@ import torch
 from . import runtime as rt
 from .codegen.uvu import UVUGenerator
 from .codegen.uvu_direct import UVUDirectGenerator
-from .codegen.uvu_fast import UVUFastGenerator
 from .problem import TPProblem
 from .weight_order import WeightReorder, is_identity
 from .wigner import wigner_3j
@@ -29,11 +28,20 @@ def _make_steps(descs):
                          d.get("work_per_block", 1), d.get("num_blocks", 0), d.get("grid_y", 1)) for d in descs]
 
 
-def schedule() -> str:
-    """Kernel schedule for uvu problems with per-row weights: "direct" (registers only, default)
-    or "lds" (rows staged through LDS); the environment variable exists for A/B measurements."""
-    import os
-    return os.environ.get("OEQ_AMD_SCHEDULE", "direct")
+def select_generator(config: TPProblem):
+    """The kernel generator of a batch tensor product: MFMA kernels for uvw with shared weights,
+    streaming vector-ALU kernels for uvw with per-row weights, the persistent two-stage dW
+    reduction for uvu with shared weights, register-direct streaming kernels otherwise."""
+    mode = validate_problem(config)
+    if mode == "uvw" and config.shared_weights:
+        from .codegen.uvw import UVWGenerator
+        return UVWGenerator(config)
+    if mode == "uvw":
+        from .codegen.uvw_batched import UVWBatchedGenerator
+        return UVWBatchedGenerator(config)
+    if config.shared_weights:
+        return UVUGenerator(config, "tp")
+    return UVUDirectGenerator(config, "tp")
 
 
 def validate_problem(config: TPProblem) -> str:
@@ -76,31 +84,14 @@ class TensorProduct(TensorProductBase):
         config = self.config
         mode = validate_problem(config)
         self.is_uvw = (mode == "uvw")
-        if self.is_uvw and config.shared_weights:
-            from .codegen.uvw import UVWGenerator
-            self.generator = UVWGenerator(config)
-        elif self.is_uvw:
-            from .codegen.uvw_batched import UVWBatchedGenerator
-            self.generator = UVWBatchedGenerator(config)
-        elif config.shared_weights or schedule() == "lds":
-            self.generator = UVUGenerator(config, "tp")
-        else:
-            self.generator = UVUDirectGenerator(config, "tp")
+        self.generator = select_generator(config)
         self.jit_kernel = self.generator.render()
         code = rt.compile_source(self.jit_kernel)
         fwd, bwd, ws = self.generator.plan()
         self.workspace_bytes = ws()
         self.internal = rt.TPImpl(code, _make_steps(fwd), _make_steps(bwd))
         self._workspace = None
-        # bandwidth-oriented schedule for 16-byte granular problems; used whenever the tensors
-        # handed in are 16-byte aligned, the generic kernels otherwise
-        self.internal_fast = None
-        self._internal_unaligned = None
-        if not self.is_uvw and schedule() == "lds" and UVUFastGenerator.eligible(config, "tp"):
-            self.generator_fast = UVUFastGenerator(config, "tp")
-            ffwd, fbwd, _ = self.generator_fast.plan()
-            self.internal_fast = rt.TPImpl(rt.compile_source(self.generator_fast.render()),
-                                           _make_steps(ffwd), _make_steps(fbwd))
+        self._internal_unaligned = None       # kernels without 16-byte vector stores, compiled on first need
 
         self._reorder = WeightReorder(config)
         if is_identity(self._reorder.perm):
@@ -130,8 +121,6 @@ class TensorProduct(TensorProductBase):
 
     def _pick(self, *ptrs):
         aligned = all(int(p) % 16 == 0 for p in ptrs)
-        if self.internal_fast is not None and aligned:
-            return self.internal_fast
         if not aligned and isinstance(self.generator, UVUDirectGenerator):
             # rare: a caller-supplied tensor that is not 16-byte aligned -> kernels without vector stores
             if self._internal_unaligned is None:

@@ -21,6 +21,8 @@ from .sh import random_unit_vectors, spherical_harmonics
 from .tensor_product import TensorProduct
 
 MACE = ("128x0e+128x1o+128x2e", "1x0e+1x1o+1x2e+1x3o", "128x0e+128x1o+128x2e+128x3o")
+# the same inputs with every triangle-allowed output kept, also the unnatural parities 1e, 2o, 3e
+MACE_ALL = ("128x0e+128x1o+128x2e", "1x0e+1x1o+1x2e+1x3o", "128x0e+128x1o+128x1e+128x2e+128x2o+128x3o+128x3e")
 NEQUIP = ("32x0e+32x1o+32x2e", "1x0e+1x1o+1x2e", "32x0e+32x1o+32x2e")
 LARGE = ("256x0e+256x1o+256x2e", "1x0e+1x1o+1x2e+1x3o", "256x0e+256x1o+256x2e")
 DENSE = ("64x0e+64x1o+64x2e", "1x0e+1x1o+1x2e", "64x0e+64x1o+64x2e")
@@ -191,6 +193,12 @@ def get(name: str) -> Workload:
                      {"batch": 50000, "paths": 17}, sh_lmax=3)
         w.alg_bytes = _tp_bytes(w.problem(), w.units, 4)
         return w
+    if name == "mace_uvu_all_parities":
+        w = Workload(name, "per-edge uvu TP, 128x0e+128x1o+128x2e (x) SH(lmax 3) -> every triangle-allowed l3<=3 of either "
+                     "parity, 24 paths, batch 50000, fp32, forward+backward", "tp", MACE_ALL, 50000, "edges/s", "hbm",
+                     "f32", 12346, {"batch": 50000, "paths": 24}, sh_lmax=3)
+        w.alg_bytes = _tp_bytes(w.problem(), w.units, 4)
+        return w
     if name == "readme_uvu":
         w = Workload(name, "single-path uvu TP 1x2e (x) 1x3e -> 1x2e, batch 1000, fp32", "tp",
                      ("1x2e", "1x3e", "1x2e"), 1000, "rows/s", "hbm", "f32", 12345, {"batch": 1000, "paths": 1})
@@ -222,5 +230,5 @@ def get(name: str) -> Workload:
     raise KeyError(f"unknown workload {name!r}")
 
 
-ALL = ("readme_uvu", "mace_uvu", "nequip_conv_atomic", "nequip_conv_det", "dense_uvw_f32", "dense_uvw_f64",
+ALL = ("readme_uvu", "mace_uvu", "mace_uvu_all_parities", "nequip_conv_atomic", "nequip_conv_det", "dense_uvw_f32", "dense_uvw_f64",
        "large_conv_det")

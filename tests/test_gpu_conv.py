@@ -120,3 +120,28 @@ def test_deterministic_bit_reproducible(cuda):
         assert torch.equal(z1.detach(), z0)
         for a, b in zip(grads0, (x.grad, y.grad, w.grad)):
             assert torch.equal(a, b)
+
+
+def test_device_graph_preparation(cuda):
+    """The README recipe for deterministic=True without torch_geometric: an unsorted edge list is
+    sorted on the GPU with sort_by_receiver; the result equals the oracle on the unsorted graph."""
+    import torch
+    import openequivariance_amd as oeq
+    prob, oprob = common.channelwise(common.NEQUIP)
+    nodes, nnz = 200, 5000
+    rows, cols = common.random_graph(nodes, nnz, 41)
+    X, Y, W, G = common.conv_inputs(prob, nodes, nnz, 41, np.float32, 2)
+    dev = torch.device("cuda:0")
+    x, y, w = (torch.tensor(a, device=dev, requires_grad=True) for a in (X, Y, W))
+    r, c, rperm, tperm = oeq.sort_by_receiver(torch.tensor(rows, device=dev), torch.tensor(cols, device=dev), nodes)
+    conv = oeq.TensorProductConv(prob, torch_op=True, deterministic=True)
+    z = conv.forward(x, y[rperm], w[rperm], r, c, tperm)
+    z.backward(torch.tensor(G, device=dev))
+    torch.cuda.synchronize()
+    Zr = otp.conv_forward(oprob, X, Y, W, rows, cols)
+    dXr, dYr, dWr = otp.conv_backward(oprob, X, Y, W, G, rows, cols)
+    errs = dict(Z=rel_err(z.detach().cpu().numpy(), Zr), dX=rel_err(x.grad.cpu().numpy(), dXr),
+                dY=rel_err(y.grad.cpu().numpy(), dYr), dW=rel_err(w.grad.cpu().numpy(), dWr))
+    print(errs, flush=True)
+    for k, v in errs.items():
+        assert v <= FP32_TOL, f"{k}: relative error {v:.3e}"

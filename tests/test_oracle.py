@@ -160,3 +160,22 @@ def test_coord_graph_and_transpose_perm():
     import openequivariance_amd as oeq
     gph = oeq.CoordGraph(np.zeros((9, 3)), rows, cols)
     assert np.array_equal(gph.rows, r) and np.array_equal(gph.cols, c) and np.array_equal(gph.transpose_perm, tperm)
+
+
+def test_sort_by_receiver_matches_coord_graph():
+    """The torch graph preparation (any device; CPU tensors here) gives the oracle's sorted edge
+    list and transpose permutation, also with duplicate edges and isolated nodes."""
+    import torch
+    import openequivariance_amd as oeq
+    rows, cols = common.random_graph(9, 40, 11)
+    rows = np.concatenate([rows, rows[:5]])            # duplicate edges: ties broken by position
+    cols = np.concatenate([cols, cols[:5]])
+    r, c, tperm, order = otp.coord_graph(rows, cols)
+    rs, cs, rperm, tp = oeq.sort_by_receiver(torch.from_numpy(rows), torch.from_numpy(cols), 12)
+    assert np.array_equal(rs.numpy(), r) and np.array_equal(cs.numpy(), c)
+    assert np.array_equal(rows[rperm.numpy()], r) and np.array_equal(cols[rperm.numpy()], c)
+    key = list(zip(cs.numpy()[tp.numpy()], rs.numpy()[tp.numpy()]))
+    assert key == sorted(key) and sorted(tp.tolist()) == list(range(45))
+    assert np.array_equal(tp.numpy(), tperm)
+    e = torch.zeros(0, dtype=torch.int64)
+    assert all(t.numel() == 0 for t in oeq.sort_by_receiver(e, e))
