@@ -122,6 +122,62 @@ extern "C" __global__ __launch_bounds__(256) void oeq_copy_calibration(const flo
 }
 """
 
+STREAM_SRC = r"""
+// Streaming probe with a fixed read:write mix: every thread reads NR 16-byte vectors (one from each
+// of NR input streams) and writes NW (one to each of NW output streams), nothing else.
+typedef float v4 __attribute__((ext_vector_type(4)));
+extern "C" __global__ __launch_bounds__(256) void oeq_stream_probe(const v4* __restrict__ in, v4* __restrict__ out, unsigned long long n) {
+    v4 keep = {0.f, 0.f, 0.f, 0.f};
+    for (unsigned long long i = (unsigned long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (unsigned long long)gridDim.x * 256) {
+        v4 acc = {1.f, 2.f, 3.f, 4.f};
+#pragma unroll
+        for (int r = 0; r < NR; ++r) acc += __builtin_nontemporal_load(in + r * n + i);
+#pragma unroll
+        for (int w = 0; w < NW; ++w) __builtin_nontemporal_store(acc, out + w * n + i);
+        keep += acc;
+    }
+    if (NW == 0 && keep.x == 12345.678f) out[0] = keep;       // keeps the loads alive; never true for zero inputs
+}
+"""
+
+
+def stream_probe(nr, nw, total_bytes=3 << 30, reps=5):
+    """GB/s of a plain streaming kernel that reads ``nr`` and writes ``nw`` 16-byte vectors per
+    thread (best of ``reps`` launches, 3 GiB per launch so that the 256 MiB Infinity Cache does not
+    help): what HBM sustains for this read:write mix, the practical ceiling of a kernel with it."""
+    import ctypes as C
+    import torch
+    from openequivariance_amd import runtime as rt
+    n = total_bytes // 16 // (nr + nw)
+    src = torch.zeros(max(nr, 1) * n * 4, dtype=torch.float32, device="cuda")
+    dst = torch.empty(max(nw, 1) * n * 4, dtype=torch.float32, device="cuda")
+    mod = rt.Module(rt.compile_source(STREAM_SRC, options=tuple(rt.DEFAULT_OPTIONS) + (f"-DNR={nr}", f"-DNW={nw}")))
+    stream = torch.cuda.current_stream().cuda_stream
+    args = [C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr()), C.c_uint64(n)]
+    best = float("inf")
+    for r in range(reps + 2):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        mod.launch("oeq_stream_probe", 32768, 256, args, stream=stream)
+        b.record()
+        b.synchronize()
+        if r >= 2:
+            best = min(best, a.elapsed_time(b))
+    return (nr + nw) * n * 16 / (best * 1e-3) / 1e9
+
+
+def mix_of(read_bytes, write_bytes):
+    """Small-integer read:write mix closest to the given byte counts (each side at most 4)."""
+    best = None
+    for nr in range(0, 5):
+        for nw in range(0, 5):
+            if nr + nw == 0:
+                continue
+            err = abs(nr / (nr + nw) - read_bytes / (read_bytes + write_bytes))
+            if best is None or err < best[0] - 1e-12:
+                best = (err, nr, nw)
+    return best[1], best[2]
+
 
 def copy_calibration(steps):
     """A copy kernel of known size (1 GiB read + 1 GiB written per launch), used to scale the
@@ -143,10 +199,21 @@ def copy_calibration(steps):
                       "bytes_written_per_launch": nbytes, "launches": steps}))
 
 
+def stream_calibration():
+    """Sustained HBM rate of plain streaming kernels for several read:write mixes."""
+    out = {"workload": "stream_calibration", "unit": "GB/s", "peak": HBM_PEAK_GBS}
+    for nr, nw in ((1, 0), (4, 1), (1, 1), (1, 3), (0, 1)):
+        out[f"read{nr}_write{nw}"] = round(stream_probe(nr, nw), 1)
+    print(json.dumps(out))
+
+
 def main():
     args = parse()
     if args.workload == "copy_calibration":
         copy_calibration(args.steps)
+        return
+    if args.workload == "stream_calibration":
+        stream_calibration()
         return
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (the path shards over rows/edges "
@@ -207,6 +274,15 @@ def main():
     else:
         tot = wl.alg_flops["forward"] + wl.alg_flops["backward"]
         roofline["fwd_bwd_frac"] = round(tot / ((fwd_ms + bwd_ms) * 1e-3) / 1e12 / peak, 4)
+
+    if wl.bound == "hbm" and not args.no_cold:
+        # what a plain streaming kernel with the dominant kernel's read:write mix sustains on this
+        # GPU: the practical ceiling under the 8 TB/s datasheet peak
+        rd, wr = wl.read_write_split(dom)
+        nr, nw = mix_of(rd, wr)
+        ceil = stream_probe(nr, nw)
+        roofline["streaming_ceiling"] = {"mix": f"{nr} reads : {nw} writes", "GB/s": round(ceil, 1),
+                                         "frac_of_ceiling": round(achieved / ceil, 4)}
 
     if not args.no_cold:
         # second leg, outside the timed region: the same launches with the caches flushed before

@@ -69,6 +69,20 @@ class Workload:
     alg_bytes: Dict[str, int] = field(default_factory=dict)
     alg_flops: Dict[str, int] = field(default_factory=dict)
 
+    def read_write_split(self, direction: str):
+        """(bytes read, bytes written) of the algorithmic traffic of one launch."""
+        prob = self.problem()
+        s = 4 if self.dtype == "f32" else 8
+        d1, d2, d3, wn = prob.irreps_in1.dim, prob.irreps_in2.dim, prob.irreps_out.dim, prob.weight_numel
+        if self.kind == "tp":
+            n = self.units
+            w = wn if prob.shared_weights else wn * n
+            written = n * d3 * s if direction == "forward" else (n * (d1 + d2) + w) * s
+        else:
+            E, N = self.units, self.nodes
+            written = N * d3 * s if direction == "forward" else (E * (d2 + wn) + N * d1) * s
+        return self.alg_bytes[direction] - written, written
+
     # ------------------------------------------------------------------ problem
     def problem(self) -> TPProblem:
         dt = np.float32 if self.dtype == "f32" else np.float64
