@@ -26,8 +26,12 @@ from .uvu_direct import UVUDirectGenerator
 class UVUDetGenerator(UVUDirectGenerator):
     _allow_det = True
 
-    def __init__(self, problem: TPProblem, prefetch_backward=None, vector_stores: bool = True):
+    def __init__(self, problem: TPProblem, prefetch_backward=None, vector_stores: bool = True,
+                 forward_perm: bool = False):
         super().__init__(problem, "conv_det", vector_stores=vector_stores)
+        # True: the forward walks the receiver-grouped edge order listed in the workspace (built on
+        # the fly from an unsorted edge list) instead of the edge list itself
+        self.forward_perm = forward_perm
         # fetch the next edge's operands while the current edge is being computed; pays when the
         # per-edge register footprint is small enough to keep several wavefronts per SIMD
         words = sum(self.out[i].D for i in self.used_out) + len(self.paths) + len(self.used_y)
@@ -102,6 +106,8 @@ class UVUDetGenerator(UVUDirectGenerator):
         E = Emitter()
         self.emit_lane_direct(E, lds=True)
         self._node_setup(E, "0")
+        if self.forward_perm:
+            E("const i64* __restrict__ eperm = (const i64*)ws + 2 * (node_count + 1);")
         self._cur_c = "e"
         for oi in self.used_out:
             E("T " + ", ".join(f"z{oi}_{k} = (T)0" for k in range(self.out[oi].D)) + ";")
@@ -119,9 +125,17 @@ class UVUDetGenerator(UVUDirectGenerator):
             E("{")
             E.level += 1
             E(f"const bool ev = {self.edge_pos(it)} < len;")
-            E(f"const u64 e = ev ? (u64)(beg + {self.edge_pos(it)}) : (u64)(nnz - 1);   // idle lanes re-read the last edge, masked below")
-            E("const i64 snd = cols[e];")
-            E("const bool rv = ev && snd >= 0 && snd < (i64)node_count;")
+            if self.forward_perm:
+                E(f"const u64 j = ev ? (u64)(beg + {self.edge_pos(it)}) : (u64)(nnz - 1);")
+                E("const i64 e0 = eperm[j];")
+                E("const bool ok_e = ev && e0 >= 0 && e0 < (i64)nnz;")
+                E("const u64 e = ok_e ? (u64)e0 : 0;")
+                E("const i64 snd = cols[e];")
+                E("const bool rv = ok_e && snd >= 0 && snd < (i64)node_count;")
+            else:
+                E(f"const u64 e = ev ? (u64)(beg + {self.edge_pos(it)}) : (u64)(nnz - 1);   // idle lanes re-read the last edge, masked below")
+                E("const i64 snd = cols[e];")
+                E("const bool rv = ev && snd >= 0 && snd < (i64)node_count;")
             E("const u64 sndc = rv ? (u64)snd : 0;")
             E(f"const T* __restrict__ Yr = Y + e * {self.D2};")
             E(f"const T* __restrict__ Wr = W + e * {self.WN};")

@@ -23,6 +23,7 @@ import torch
 from . import runtime as rt
 from .codegen.uvu_det import UVUDetGenerator
 from .codegen.uvu_direct import UVUDirectGenerator
+from .codegen.uvu_sorted import UVUSortedGenerator
 from .problem import TPProblem
 from .tensor_product import _make_steps, validate_problem
 from .weight_order import WeightReorder
@@ -87,10 +88,16 @@ def sort_by_receiver(rows: "torch.Tensor", cols: "torch.Tensor", node_count: typ
     return rows_s, cols_s, receiver_perm, transpose_perm
 
 
-def select_conv_generator(config: TPProblem, deterministic: bool):
+def select_conv_generator(config: TPProblem, deterministic: bool, vector_stores: bool = True):
     """Kernel generator of the fused convolution: one node per wavefront with fixed summation order
-    when deterministic, register-direct kernels with coalesced atomics otherwise."""
-    return UVUDetGenerator(config) if deterministic else UVUDirectGenerator(config, "conv_atomic")
+    when deterministic; otherwise a forward that groups the edges by receiver on the fly and a
+    backward with coalesced atomics."""
+    if deterministic:
+        return UVUDetGenerator(config, vector_stores=vector_stores)
+    import os
+    if os.environ.get("OEQ_AMD_CONV_FORWARD", "sorted") == "atomic":     # A/B measurements only
+        return UVUDirectGenerator(config, "conv_atomic", vector_stores=vector_stores)
+    return UVUSortedGenerator(config, vector_stores=vector_stores)
 
 
 class TensorProductConv:
@@ -116,6 +123,8 @@ class TensorProductConv:
             raise NotImplementedError("TensorProductConv supports uvu problems")
 
         self.generator = select_conv_generator(config, deterministic)
+        # True: the forward writes every row of Z itself; False: it accumulates into a zeroed Z
+        self.forward_overwrites = not isinstance(self.generator, UVUDirectGenerator) or deterministic
         self.jit_kernel = self.generator.render()
         code = rt.compile_source(self.jit_kernel)
         fwd, bwd, self._ws_bytes = self.generator.plan()
@@ -167,12 +176,11 @@ class TensorProductConv:
             raise TypeError(f"tensors must be {tdt}")
 
     def _pick(self, *ptrs):
-        """The atomic kernels use dword accesses only; the deterministic forward writes Z with 16-byte
-        vector stores and falls back to a variant without them for a misaligned tensor (rare: a view
-        with an odd storage offset)."""
-        if self.deterministic and any(int(p) % 16 for p in ptrs):
+        """The forward kernels write Z with 16-byte vector stores; a misaligned tensor (rare: a view
+        with an odd storage offset) gets a variant without them, compiled on first need."""
+        if any(int(p) % 16 for p in ptrs):
             if self._internal_unaligned is None:
-                g = UVUDetGenerator(self.config, vector_stores=False)
+                g = select_conv_generator(self.config, self.deterministic, vector_stores=False)
                 fwd, bwd, _ = g.plan()
                 self._internal_unaligned = rt.ConvImpl(rt.compile_source(g.render()), _make_steps(fwd), _make_steps(bwd))
             return self._internal_unaligned
@@ -183,6 +191,7 @@ class TensorProductConv:
                           transpose_perm=0, stream=None):
         """reference: extension/convolution.hpp:121-147"""
         impl = self._pick(L1_in, L2_in, weights, L3_out)
+        workspace = workspace or self.workspace_ptr(int(nnz), int(node_count))     # the operator owns one
         impl.exec_conv_rawptrs(L1_in, L2_in, weights, L3_out, rows, cols, int(nnz), int(node_count),
                                workspace, transpose_perm, self._stream() if stream is None else stream)
 
@@ -190,6 +199,7 @@ class TensorProductConv:
                          node_count, workspace=0, transpose_perm=0, stream=None):
         """reference: extension/convolution.hpp:149-173"""
         impl = self._pick(L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_grad)
+        workspace = workspace or self.workspace_ptr(int(nnz), int(node_count))
         impl.backward_rawptrs(L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_grad, rows, cols,
                               int(nnz), int(node_count), workspace, transpose_perm,
                               self._stream() if stream is None else stream)
@@ -208,7 +218,7 @@ class TensorProductConv:
             self._check(x, y, w, rows, cols, tperm)
             E, N = rows.shape[0], x.shape[0]
             # the atomic kernels accumulate into Z; the deterministic ones write every row
-            out = (torch.empty if det else torch.zeros)((N, L3_dim), dtype=x.dtype, device=x.device)
+            out = (torch.empty if self.forward_overwrites else torch.zeros)((N, L3_dim), dtype=x.dtype, device=x.device)
             self.exec_conv_rawptrs(x.data_ptr(), y.data_ptr(), w.data_ptr(), out.data_ptr(), rows.data_ptr(),
                                    cols.data_ptr(), E, N, self.workspace_ptr(E, N),
                                    tperm.data_ptr() if tperm is not None else 0)

@@ -175,8 +175,8 @@ class Workload:
             det = self.deterministic
 
             def fwd():
-                if not det:
-                    t["Z"].zero_()              # the atomic kernels accumulate: part of the operator's work
+                if not op.forward_overwrites:
+                    t["Z"].zero_()              # atomic kernels accumulate: part of the operator's work
                 op.exec_conv_rawptrs(p["X"], p["Y"], p["W"], p["Z"], p["rows"], p["cols"], E, N, ws, tp_ptr, stream)
 
             def bwd():

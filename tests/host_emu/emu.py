@@ -66,6 +66,9 @@ static inline T oeq_wave_sum63(T v) { g_xT[threadIdx.x] = v; oeq_sync(); T t = 0
 static inline T oeq_ldnt(const T* p) { return *p; }
 static inline void oeq_stnt(T* p, T v) { *p = v; }
 static inline void oeq_block_sync() { pthread_barrier_wait(&g_bar); }
+static inline void __syncthreads() { pthread_barrier_wait(&g_bar); }
+#define __HIP_MEMORY_SCOPE_AGENT 0
+template <class V> static inline V __hip_atomic_fetch_add(V* p, V v, int, int) { std::lock_guard<std::mutex> g(g_atomic_mutex); V o = *p; *p += v; return o; }
 // matrix-core step of one wavefront, emulated collectively by its 64 threads
 struct V4 { T v[4]; T& operator[](int i) { return v[i]; } const T& operator[](int i) const { return v[i]; } };
 static pthread_barrier_t g_wbar[16];
@@ -193,6 +196,12 @@ CONV_EXTRA_DET = r"""
         else if (k == "prep_forward") FWD_CALL(prep_forward);
         else if (k == "prep_backward") BWD_CALL(prep_backward);
 """
+CONV_EXTRA_SORTED = r"""
+        else if (k == "group_clear") FWD_CALL(group_clear);
+        else if (k == "group_count") FWD_CALL(group_count);
+        else if (k == "group_scan") FWD_CALL(group_scan);
+        else if (k == "group_fill") FWD_CALL(group_fill);
+"""
 CONV_EXTRA_DYRED = r"""
         else if (k == "backward_dy_reduce") BWD_CALL(backward_dy_reduce);
 """
@@ -271,6 +280,8 @@ def run_conv(gen, steps: Sequence[Dict], X, Y, W, rows, cols, G=None, tperm=None
         extra += CONV_EXTRA_DET
         if gen.NCH > 1:
             extra += CONV_EXTRA_DYRED
+    elif hasattr(gen, "fwd"):
+        extra += CONV_EXTRA_SORTED
     exe = build(gen.render(prelude=emu_prelude(gen.T)), CONV_MAIN.replace("@EXTRA@", extra))
     nodes, nnz = X.shape[0], rows.shape[0]
     with tempfile.TemporaryDirectory() as d:

@@ -8,6 +8,7 @@ import openequivariance_amd as oeq
 from openequivariance_amd.codegen.uvu import UVUGenerator
 from openequivariance_amd.codegen.uvu_det import UVUDetGenerator
 from openequivariance_amd.codegen.uvu_direct import UVUDirectGenerator
+from openequivariance_amd.codegen.uvu_sorted import UVUSortedGenerator
 from openequivariance_amd.codegen.uvw import UVWGenerator
 from host_emu import emu
 from oracle import spec, tp as otp, weights as ow
@@ -57,10 +58,12 @@ def test_generic_tp_shared_weights():
         assert rel_err(got, ref) < TOL
 
 
-@pytest.mark.parametrize("det", [False, True])
-def test_conv(det):
+@pytest.mark.parametrize("variant", ["atomic", "det", "sorted"])
+def test_conv(variant):
     prob, oprob = common.channelwise(common.NEQUIP)
-    g = UVUDetGenerator(prob) if det else UVUDirectGenerator(prob, "conv_atomic")
+    det = variant == "det"
+    g = {"det": UVUDetGenerator, "sorted": UVUSortedGenerator,
+         "atomic": lambda p: UVUDirectGenerator(p, "conv_atomic")}[variant](prob)
     nodes, nnz = 7, 19
     rows, cols = common.random_graph(nodes, nnz, 5)
     tperm = None
@@ -68,7 +71,10 @@ def test_conv(det):
         rows, cols, tperm, _ = otp.coord_graph(rows, cols)
     X, Y, W, G = common.conv_inputs(prob, nodes, nnz, 6)
     fwd, bwd, ws = g.plan()
-    out = emu.run_conv(g, fwd, X, Y, W, rows, cols, tperm=tperm, ws_bytes=ws(nnz, nodes))
+    # (a transpose permutation makes the emulator start from a junk-filled Z: the deterministic and
+    # the sorted forward must write every row themselves; the sorted kernels never read it)
+    out = emu.run_conv(g, fwd, X, Y, W, rows, cols, tperm=np.arange(nnz) if variant == "sorted" else tperm,
+                       ws_bytes=ws(nnz, nodes))
     assert rel_err(out["Z"], otp.conv_forward(oprob, X, Y, W, rows, cols)) < TOL
     out = emu.run_conv(g, bwd, X, Y, W, rows, cols, G=G, tperm=tperm, ws_bytes=ws(nnz, nodes))
     for got, ref in zip((out["Xg"], out["Yg"], out["Wg"]), otp.conv_backward(oprob, X, Y, W, G, rows, cols)):
