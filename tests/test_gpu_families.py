@@ -28,6 +28,12 @@ SINGLE = [("128x1e", "1x1e", "128x1e"), ("128x2e", "1x1e", "128x2e"), ("128x3e",
 FULLY_CONNECTED = {
     "tetris-poly-1": ("1x0e+1x1o+1x2e+1x3o", "1x0e+1x1o+1x2e+1x3o", "64x0e+24x1e+24x1o+16x2e+16x2o"),
     "tetris-poly-2": ("64x0e+24x1e+24x1o+16x2e+16x2o", "1x0e+1x1o+1x2e+1x3o", "0o+6x0e"),
+    # layers of e3nn's tetris example (benchmark/benchmark_configs.py:6-33 of the reference):
+    # multiplicities that are no multiple of 16, up to 300 x 250 weight blocks, scalar second operand
+    "tetris-0-sc": ("1x0e", "1x0e", "150x0e+50x1o+50x2e"),
+    "tetris-1-sc": ("50x0e+50x1o+50x2e", "1x0e", "250x0e+50x1o+50x1e+50x2o+50x2e"),
+    "tetris-2-lin2": ("100x0o+150x0e+300x1o+250x1e+250x2o+300x2e", "1x0e", "50x0o+250x0e+50x1o+50x1e+50x2o+50x2e"),
+    "tetris-3-lin2": ("150x0o+150x0e", "1x0e", "1x0o+6x0e"),
 }
 
 
