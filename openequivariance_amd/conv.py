@@ -336,6 +336,151 @@ class TensorProductConv:
     def __call__(self, *args):
         return self.forward(*args)
 
+    # -------------------------------------------- correctness / timing (harness)
+    def _reference(self, reference_implementation):
+        if reference_implementation is None:
+            raise NotImplementedError("pass reference_implementation=...: no CPU reference ships with this package "
+                                      "(the reference's default, e3nn, is an optional third-party dependency)")
+        return reference_implementation(self.config)
+
+    def test_correctness_forward(self, graph, thresh, prng_seed, reference_implementation=None,
+                                 check_reproducible=True, torch_op=False):
+        """Output against a reference implementation on seeded buffers, and (five repeats) whether
+        the output repeats bit for bit (reference: ConvolutionBase.py:172-249)."""
+        from .benchmark.correctness_utils import check_similiarity
+        from .benchmark.random_buffer_utils import get_random_buffers_forward_conv
+        in1, in2, weights, out = get_random_buffers_forward_conv(self.config, graph.node_count, graph.nnz, prng_seed)
+        ref_out, test_out = out.copy(), out.copy()
+        self._reference(reference_implementation).forward_cpu(L1_in=in1.copy(), L2_in=in2.copy(), weights=weights.copy(),
+                                                              L3_out=ref_out, graph=graph)
+        self.forward_cpu(L1_in=in1.copy(), L2_in=in2.copy(), weights=weights.copy(), L3_out=test_out, graph=graph)
+        result = {"thresh": thresh, "output": check_similiarity("output", test_out, ref_out, thresh)}
+        if check_reproducible:
+            same = True
+            for _ in range(5):
+                again = out.copy()
+                self.forward_cpu(L1_in=in1.copy(), L2_in=in2.copy(), weights=weights.copy(), L3_out=again, graph=graph)
+                same = same and bool(np.all(again == test_out))
+            result["output"]["num_reproducibility_trials"] = 5
+            result["output"]["bitwise_reproducible"] = same
+        return result
+
+    def test_correctness_backward(self, graph, thresh, prng_seed, reference_implementation=None):
+        """reference: ConvolutionBase.py:445-494."""
+        from .benchmark.correctness_utils import check_similiarity
+        from .benchmark.random_buffer_utils import get_random_buffers_backward_conv
+        in1, in2, out_grad, weights, wg, g1, g2 = get_random_buffers_backward_conv(self.config, graph.node_count,
+                                                                                   graph.nnz, prng_seed)
+        grads = []
+        for impl in (self._reference(reference_implementation), self):
+            bufs = dict(weights_grad=wg.copy(), L1_grad=g1.copy(), L2_grad=g2.copy())
+            impl.backward_cpu(L1_in=in1.copy(), L2_in=in2.copy(), L3_grad=out_grad.copy(), weights=weights.copy(),
+                              graph=graph, **bufs)
+            grads.append(bufs)
+        result = {"thresh": thresh}
+        for name, key in (("weight_grad", "weights_grad"), ("in1_grad", "L1_grad"), ("in2_grad", "L2_grad")):
+            result[name] = check_similiarity(name, grads[1][key], grads[0][key], thresh)
+        return result
+
+    def test_correctness_double_backward(self, graph, thresh, prng_seed, reference_implementation=None):
+        """Second derivatives through the torch op against a differentiable reference
+        (reference: ConvolutionBase.py:496-557)."""
+        from .benchmark.correctness_utils import check_similiarity
+        from .benchmark.random_buffer_utils import get_random_buffers_backward_conv
+        assert self.torch_op
+        in1, in2, out_grad, weights, _, _, _ = get_random_buffers_backward_conv(self.config, graph.node_count,
+                                                                                graph.nnz, prng_seed)
+        scale = float(np.random.default_rng(seed=prng_seed * 2).standard_normal(1)[0])
+        got = []
+        for tp in (self, reference_implementation(self.config, torch_op=True) if reference_implementation
+                   else self._reference(None)):
+            dev = getattr(tp, "device", "cuda")
+            a, b, w, g = (torch.tensor(t, device=dev, requires_grad=True) for t in (in1, in2, weights, out_grad))
+            args = [a, b, w, torch.tensor(graph.rows, device=dev), torch.tensor(graph.cols, device=dev)]
+            if tp.deterministic:
+                args.append(torch.tensor(graph.transpose_perm, device=dev))
+            out = tp.forward(*args)
+            out.backward(g, create_graph=True, retain_graph=True, inputs=[a, b, w])
+            dummy = torch.norm(a.grad) + torch.norm(b.grad) + torch.norm(w.grad)
+            dummy.backward(torch.tensor(scale, device=dev, dtype=dummy.dtype), retain_graph=True, inputs=[g, a, b, w])
+            got.append([t.grad.detach().cpu().numpy() for t in (g, a, b, w)])
+        return {name: check_similiarity(name, got[0][i], got[1][i], thresh)
+                for i, name in enumerate(("output_grad", "in1_grad", "in2_grad", "weights_grad"))}
+
+    def _timed(self, num_warmup, num_iter, run, reset=lambda: None, stream=0):
+        times = np.zeros(num_iter, dtype=np.float32)
+        timer = rt.GPUTimer(stream)
+        for _ in range(num_warmup):
+            run()
+        for i in range(num_iter):
+            reset()
+            timer.clear_L2_cache()
+            timer.start()
+            run()
+            times[i] = timer.stop_clock_get_elapsed()
+        return times
+
+    def benchmark_forward(self, num_warmup, num_iter, graph, prng_seed=12345):
+        """reference: ConvolutionBase.py:251-318."""
+        from .benchmark.random_buffer_utils import get_random_buffers_forward_conv
+        assert graph.rows.dtype == self.idx_dtype and graph.cols.dtype == self.idx_dtype
+        in1, in2, weights, out = get_random_buffers_forward_conv(self.config, graph.node_count, graph.nnz, prng_seed)
+        idx = [graph.rows, graph.cols] + ([graph.transpose_perm] if self.deterministic else [])
+        if self.torch_op:
+            t = [torch.tensor(a, device="cuda") for a in (in1, in2, weights, *idx)]
+            times = self._timed(num_warmup, num_iter, lambda: self.forward(*t), stream=self._stream())
+        else:
+            bufs = [rt.DeviceBuffer(a) for a in (in1, in2, weights, out, graph.rows, graph.cols)]
+            tp = rt.DeviceBuffer(graph.transpose_perm) if self.deterministic else None
+            nbytes = self._ws_bytes(graph.nnz, graph.node_count)
+            ws = rt.DeviceBuffer(nbytes) if nbytes else None
+            ptrs = [b.data_ptr() for b in bufs]
+            zero = (lambda: None) if self.forward_overwrites else (lambda: bufs[3].zero())
+            times = self._timed(num_warmup, num_iter, lambda: self.internal.exec_conv_rawptrs(
+                *ptrs, graph.nnz, graph.node_count, ws.data_ptr() if ws else 0, tp.data_ptr() if tp else 0, 0), zero)
+        ops, data, _ = flops_data_per_tp(self.config, "forward")
+        return self.calculate_bench_stats("forward", ops + self.config.irreps_out.dim, data, times, graph, num_warmup,
+                                          num_iter, prng_seed)
+
+    def benchmark_backward(self, num_warmup, num_iter, graph, prng_seed=12345):
+        """reference: ConvolutionBase.py:321-411."""
+        from .benchmark.random_buffer_utils import get_random_buffers_backward_conv
+        assert graph.rows.dtype == self.idx_dtype and graph.cols.dtype == self.idx_dtype
+        in1, in2, out_grad, weights, wg, g1, g2 = get_random_buffers_backward_conv(self.config, graph.node_count,
+                                                                                   graph.nnz, prng_seed)
+        if self.torch_op:
+            x, y, w = (torch.tensor(a, device="cuda", requires_grad=True) for a in (in1, in2, weights))
+            idx = [torch.tensor(a, device="cuda") for a in
+                   [graph.rows, graph.cols] + ([graph.transpose_perm] if self.deterministic else [])]
+            out, g = self.forward(x, y, w, *idx), torch.tensor(out_grad, device="cuda")
+            times = self._timed(num_warmup, num_iter, lambda: out.backward(g, retain_graph=True, inputs=[x, y, w]),
+                                lambda: [t.grad.zero_() for t in (x, y, w)], stream=self._stream())
+        else:
+            bufs = [rt.DeviceBuffer(a) for a in (in1, g1, in2, g2, weights, wg, out_grad, graph.rows, graph.cols)]
+            tp = rt.DeviceBuffer(graph.transpose_perm) if self.deterministic else None
+            nbytes = self._ws_bytes(graph.nnz, graph.node_count)
+            ws = rt.DeviceBuffer(nbytes) if nbytes else None
+            ptrs = [b.data_ptr() for b in bufs]
+            zero = (lambda: None) if self.deterministic else (lambda: bufs[1].zero())
+            times = self._timed(num_warmup, num_iter, lambda: self.internal.backward_rawptrs(
+                *ptrs, graph.nnz, graph.node_count, ws.data_ptr() if ws else 0, tp.data_ptr() if tp else 0, 0), zero)
+        ops, data, _ = flops_data_per_tp(self.config, "backward")
+        return self.calculate_bench_stats("backward", ops + self.config.irreps_out.dim, data, times, graph, num_warmup,
+                                          num_iter, prng_seed)
+
+    def calculate_bench_stats(self, direction, ops_per_tp, data_per_tp, time_millis, graph, num_warmup, num_iter,
+                              prng_seed):
+        """Result record of the reference's convolution benchmarks (ConvolutionBase.py:413-443):
+        per-edge work model times the edge count over each measured time."""
+        t = np.asarray(time_millis, dtype=np.float64)
+        return {"direction": direction, "flops_per_tp": ops_per_tp, "data_per_tp": data_per_tp,
+                "time_millis": [float(v) for v in t],
+                "throughputs_gflops": [float(v) for v in graph.nnz * ops_per_tp / (t * 1e6)],
+                "bandwidth_gbps": [float(v) for v in graph.nnz * data_per_tp / (t * 1e6)],
+                "L1": str(self.config.irreps_in1), "L2": str(self.config.irreps_in2), "L3": str(self.config.irreps_out),
+                "graph_node_count": graph.node_count, "graph_adj_nnz": graph.nnz,
+                "num_warmup": num_warmup, "num_iter": num_iter, "prng_seed": prng_seed}
+
     # ---------------------------------------------------- numpy entry points (tests)
     def forward_cpu(self, L1_in, L2_in, weights, L3_out, graph) -> None:
         """Host arrays; ``graph`` has rows / cols / node_count / nnz (and transpose_perm when

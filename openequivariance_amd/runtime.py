@@ -293,6 +293,11 @@ class DeviceBuffer:
     def data_ptr(self) -> int:
         return self._p.value
 
+    def zero(self, stream: int = 0) -> None:
+        """Fill the allocation with zero bytes on ``stream``."""
+        if self.nbytes:
+            _check(lib().oeq_buffer_zero(self._p, self.nbytes, stream))
+
     def copy_to_host(self):
         if self.host is None:
             raise RuntimeError("buffer was created without a host array")

@@ -247,6 +247,60 @@ class TensorProduct(TensorProductBase):
         if x.dtype != tdt or y.dtype != tdt or w.dtype != tdt:
             raise TypeError(f"tensors must be {tdt}")
 
+    # ------------------------------------------------------------------ timing
+    def benchmark_forward(self, num_warmup: int, num_iter: int, L1_in, L2_in, L3_buffer, weights) -> np.ndarray:
+        """Milliseconds of ``num_iter`` forward passes, caches flushed before each (reference:
+        TensorProductBase.py:115-151).  With ``torch_op`` the torch operator is timed (allocation
+        and dispatch included), otherwise the C-ABI call on preallocated buffers."""
+        times = np.zeros(num_iter, dtype=np.float32)
+        if self.torch_op:
+            x, y, w = (torch.tensor(a, device="cuda") for a in (L1_in, L2_in, weights))
+            timer = rt.GPUTimer(self._stream())
+            run = lambda: self.forward(x, y, w)
+        else:
+            bufs = [rt.DeviceBuffer(a) for a in (L1_in, L2_in, L3_buffer, weights)]
+            n, ptrs = L1_in.shape[0], [b.data_ptr() for b in bufs]
+            ws = rt.DeviceBuffer(self.workspace_bytes) if self.workspace_bytes else None
+            timer = rt.GPUTimer(0)
+            run = lambda: self.internal.exec_tensor_product(n, *ptrs, ws.data_ptr() if ws else 0, 0)
+        for _ in range(num_warmup):
+            run()
+        for i in range(num_iter):
+            timer.clear_L2_cache()
+            timer.start()
+            run()
+            times[i] = timer.stop_clock_get_elapsed()
+        return times
+
+    def benchmark_backward(self, num_warmup: int, num_iter: int, L1_in, L2_in, L3_buffer, weights, L1_grad, L2_grad,
+                           weights_grad) -> np.ndarray:
+        """reference: TensorProductBase.py:153-218; ``L3_buffer`` is the output gradient."""
+        times = np.zeros(num_iter, dtype=np.float32)
+        if self.torch_op:
+            x, y, w = (torch.tensor(a, device="cuda", requires_grad=True) for a in (L1_in, L2_in, weights))
+            out, g = self.forward(x, y, w), torch.tensor(L3_buffer, device="cuda")
+            timer = rt.GPUTimer(self._stream())
+            run = lambda: out.backward(gradient=g, retain_graph=True, inputs=[x, y, w])
+            reset = lambda: [t.grad.zero_() for t in (x, y, w)]
+        else:
+            bufs = [rt.DeviceBuffer(a) for a in (L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_buffer)]
+            n, ptrs = L1_in.shape[0], [b.data_ptr() for b in bufs]
+            ws = rt.DeviceBuffer(self.workspace_bytes) if self.workspace_bytes else None
+            timer = rt.GPUTimer(0)
+            run = lambda: self.internal.backward(n, *ptrs, ws.data_ptr() if ws else 0, 0)
+            reset = lambda: None
+        for _ in range(num_warmup):
+            run()
+        for i in range(num_iter):
+            reset()
+            timer.clear_L2_cache()
+            timer.start()
+            run()
+            times[i] = timer.stop_clock_get_elapsed()
+        if self.torch_op:
+            L1_grad[:], L2_grad[:], weights_grad[:] = (t.grad.numpy(force=True) for t in (x, y, w))
+        return times
+
     # ------------------------------------------------------ work / traffic models
     def calculate_flops_forward(self, batch_size: int) -> dict:
         """FLOP model of the reference (LoopUnrollTP.py:77-91)."""
