@@ -12,8 +12,10 @@ from .irreps import Irrep, Irreps
 from .problem import (ChannelwiseTPP, FullyConnectedTPProblem, Instruction, SingleInstruction, TPProblem)
 from .wigner import wigner_3j
 from .tensor_product import LoopUnrollTP, TensorProduct
-from .conv import CoordGraph, LoopUnrollConv, TensorProductConv, sort_by_receiver
+from .conv import (CoordGraph, LoopUnrollConv, LoopUnrollConvAtomic, LoopUnrollConvDeterministic,
+                   LoopUnrollConvScatterSum, TensorProductConv, sort_by_receiver)
 
 __all__ = ["Irrep", "Irreps", "TPProblem", "Instruction", "ChannelwiseTPP", "FullyConnectedTPProblem",
            "SingleInstruction", "wigner_3j", "TensorProduct", "TensorProductConv", "LoopUnrollTP",
-           "LoopUnrollConv", "CoordGraph", "sort_by_receiver"]
+           "LoopUnrollConv", "LoopUnrollConvAtomic", "LoopUnrollConvDeterministic", "LoopUnrollConvScatterSum",
+           "CoordGraph", "sort_by_receiver"]

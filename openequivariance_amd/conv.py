@@ -519,3 +519,73 @@ class TensorProductConv:
 
 
 LoopUnrollConv = TensorProductConv
+
+
+class LoopUnrollConvDeterministic(TensorProductConv):
+    """reference: convolution/LoopUnrollConv.py:93-101"""
+
+    def __init__(self, config, idx_dtype=np.int64, torch_op=False):
+        super().__init__(config, torch_op=torch_op, deterministic=True, idx_dtype=idx_dtype)
+
+    @staticmethod
+    def name():
+        return "LoopUnrollConvDeterministic"
+
+
+class LoopUnrollConvAtomic(TensorProductConv):
+    """The variant for unsorted edge lists (reference: convolution/LoopUnrollConv.py:103-111)."""
+
+    def __init__(self, config, idx_dtype=np.int64, torch_op=False):
+        super().__init__(config, torch_op=torch_op, deterministic=False, idx_dtype=idx_dtype)
+
+    @staticmethod
+    def name():
+        return "LoopUnrollConvAtomic"
+
+
+class LoopUnrollConvScatterSum:
+    """Unfused baseline: the batch tensor product on gathered node features followed by a scatter
+    sum over the receivers (reference: convolution/LoopUnrollConv.py:113-160).  It materialises the
+    per-edge output, which the fused kernels avoid; the harness times it beside them."""
+    deterministic = False
+
+    def __init__(self, config, idx_dtype=np.int64, torch_op=True):
+        from .tensor_product import TensorProduct
+        assert torch_op, "the unfused baseline exists as a torch operator only"
+        self.config, self.torch_op, self.idx_dtype = config, True, np.int64
+        self.L1, self.L2, self.L3 = config.irreps_in1, config.irreps_in2, config.irreps_out
+        self.reference_tp = TensorProduct(config, torch_op=True)
+
+    @staticmethod
+    def name():
+        return "LoopUnrollConvScatterSum"
+
+    def forward(self, L1_in, L2_in, weights, rows, cols):
+        per_edge = self.reference_tp(L1_in[cols], L2_in, weights)
+        out = per_edge.new_zeros(L1_in.shape[0], self.L3.dim)
+        return out.index_add_(0, rows, per_edge)
+
+    __call__ = forward
+
+    def forward_cpu(self, L1_in, L2_in, weights, L3_out, graph):
+        per_edge = np.zeros((graph.nnz, self.L3.dim), dtype=L3_out.dtype)
+        self.reference_tp.forward_cpu(np.ascontiguousarray(L1_in[graph.cols]), L2_in, per_edge, weights)
+        L3_out[...] = 0
+        np.add.at(L3_out, graph.rows, per_edge)
+
+    def backward_cpu(self, L1_in, L1_grad, L2_in, L2_grad, L3_grad, weights, weights_grad, graph):
+        gathered_grad = np.zeros((graph.nnz, self.L1.dim), dtype=L1_grad.dtype)
+        self.reference_tp.backward_cpu(np.ascontiguousarray(L1_in[graph.cols]), gathered_grad, L2_in, L2_grad,
+                                       np.ascontiguousarray(L3_grad[graph.rows]), weights, weights_grad)
+        L1_grad[...] = 0
+        np.add.at(L1_grad, graph.cols, gathered_grad)
+
+    # the timing / comparison methods of the fused operator work on any object with these entry points
+    _reference = TensorProductConv._reference
+    _timed = TensorProductConv._timed
+    _stream = staticmethod(TensorProductConv._stream)
+    test_correctness_forward = TensorProductConv.test_correctness_forward
+    test_correctness_backward = TensorProductConv.test_correctness_backward
+    benchmark_forward = TensorProductConv.benchmark_forward
+    benchmark_backward = TensorProductConv.benchmark_backward
+    calculate_bench_stats = TensorProductConv.calculate_bench_stats

@@ -76,3 +76,38 @@ def test_conv_double_backward_check(cuda):
     conv = oeq.TensorProductConv(prob, torch_op=True, deterministic=True)
     r = conv.test_correctness_double_backward(graph, 5e-5, 12345, reference_implementation=TorchReferenceConv)
     assert all(v["pass"] for v in r.values()), r
+
+
+def test_conv_variants_agree(cuda):
+    """The named variants of the reference (deterministic, atomic, unfused scatter-sum) on one graph."""
+    import torch
+    prob, oprob = common.channelwise(common.NEQUIP)
+    nodes, nnz = 80, 1500
+    rows, cols = common.random_graph(nodes, nnz, 9)
+    graph = oeq.CoordGraph(np.zeros((nodes, 3)), rows, cols, "g")
+    X, Y, W, G = common.conv_inputs(prob, nodes, nnz, 9, np.float32, 2)
+    from oracle import tp as otp
+    Zr = otp.conv_forward(oprob, X, Y, W, graph.rows, graph.cols)
+    dXr, dYr, dWr = otp.conv_backward(oprob, X, Y, W, G, graph.rows, graph.cols)
+    names = []
+    for cls in (oeq.LoopUnrollConvDeterministic, oeq.LoopUnrollConvAtomic, oeq.LoopUnrollConvScatterSum):
+        conv = cls(prob, torch_op=True)
+        names.append(conv.name())
+        x, y, w = (torch.tensor(a, device=cuda, requires_grad=True) for a in (X, Y, W))
+        idx = [torch.tensor(a, device=cuda) for a in (graph.rows, graph.cols)]
+        if conv.deterministic:
+            idx.append(torch.tensor(graph.transpose_perm, device=cuda))
+        z = conv.forward(x, y, w, *idx)
+        z.backward(torch.tensor(G, device=cuda))
+        for nm, a, b in (("Z", z.detach(), Zr), ("dX", x.grad, dXr), ("dY", y.grad, dYr), ("dW", w.grad, dWr)):
+            assert common.rel_err(a.cpu().numpy(), b) <= common.FP32_TOL, (conv.name(), nm)
+        # numpy entry points of the unfused baseline
+        if cls is oeq.LoopUnrollConvScatterSum:
+            out = np.zeros_like(Zr, dtype=np.float32)
+            conv.forward_cpu(X, Y, W, out, graph)
+            assert common.rel_err(out, Zr) <= common.FP32_TOL
+            g1, g2, gw = np.zeros_like(X), np.zeros_like(Y), np.zeros_like(W)
+            conv.backward_cpu(X, g1, Y, g2, G, W, gw, graph)
+            for a, b in ((g1, dXr), (g2, dYr), (gw, dWr)):
+                assert common.rel_err(a, b) <= common.FP32_TOL
+    assert names == ["LoopUnrollConvDeterministic", "LoopUnrollConvAtomic", "LoopUnrollConvScatterSum"]
