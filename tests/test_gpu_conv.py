@@ -145,3 +145,34 @@ def test_device_graph_preparation(cuda):
     print(errs, flush=True)
     for k, v in errs.items():
         assert v <= FP32_TOL, f"{k}: relative error {v:.3e}"
+
+
+@pytest.mark.parametrize("deterministic", [False, True])
+def test_misaligned_tensors(cuda, deterministic):
+    """Every float tensor starts 4 bytes past a 16-byte boundary: kernels without vector stores."""
+    import torch
+    import openequivariance_amd as oeq
+    prob, oprob = common.channelwise(common.LARGE)          # 64-channel chunks: the vector-store path
+    nodes, nnz = 30, 400
+    rows, cols, tperm = _graph(nodes, nnz, 51, deterministic)
+    X, Y, W, G = common.conv_inputs(prob, nodes, nnz, 51, np.float32, 3)
+
+    def shifted(a):
+        flat = torch.empty(a.size + 1, dtype=torch.float32, device=cuda)
+        view = flat[1:].view(a.shape)
+        view.copy_(torch.from_numpy(a))
+        assert view.data_ptr() % 16 == 4
+        return view
+    conv = oeq.TensorProductConv(prob, torch_op=True, deterministic=deterministic)
+    x, y, w = (shifted(a).requires_grad_(True) for a in (X, Y, W))
+    idx = [torch.tensor(a, device=cuda) for a in ((rows, cols, tperm) if deterministic else (rows, cols))]
+    z = conv.forward(x, y, w, *idx)
+    z.backward(shifted(G))
+    zraw = shifted(np.zeros_like(G))
+    conv.exec_conv_rawptrs(x.data_ptr(), y.data_ptr(), w.data_ptr(), zraw.data_ptr(), idx[0].data_ptr(), idx[1].data_ptr(),
+                           nnz, nodes, 0, idx[2].data_ptr() if deterministic else 0)
+    torch.cuda.synchronize()
+    Zr = otp.conv_forward(oprob, X, Y, W, rows, cols)
+    dXr, dYr, dWr = otp.conv_backward(oprob, X, Y, W, G, rows, cols)
+    for nm, a, b in (("Z", z.detach(), Zr), ("Zraw", zraw, Zr), ("dX", x.grad, dXr), ("dY", y.grad, dYr), ("dW", w.grad, dWr)):
+        assert rel_err(a.cpu().numpy(), b) <= FP32_TOL, nm

@@ -161,3 +161,34 @@ def test_full_size_properties(cuda):
     # a slice of rows against the oracle
     sl = slice(49900, 50000)
     assert rel_err(z.detach()[sl].cpu().numpy(), otp.forward(oprob, X[sl], Y[sl], W[sl])) <= FP32_TOL
+
+
+def _misaligned(a, dev):
+    """Contiguous device copy of ``a`` whose storage starts 4 bytes past a 16-byte boundary."""
+    import torch
+    flat = torch.empty(a.size + 1, dtype=torch.float32, device=dev)
+    view = flat[1:].view(a.shape)
+    view.copy_(torch.from_numpy(a))
+    assert view.data_ptr() % 16 == 4 and view.is_contiguous()
+    return view
+
+
+def test_misaligned_tensors(cuda):
+    """Views with an odd storage offset: the operator switches to kernels without 16-byte vector
+    stores (inputs through the torch op, the output through the raw entry point)."""
+    import torch
+    import openequivariance_amd as oeq
+    prob, oprob = common.channelwise(common.MACE)
+    n = 37
+    X, Y, W, G = common.tp_inputs(prob, n, 5, sh_lmax=3)
+    tp = oeq.TensorProduct(prob, torch_op=True)
+    x, y, w = (_misaligned(a, cuda).requires_grad_(True) for a in (X, Y, W))
+    z = tp(x, y, w)
+    z.backward(_misaligned(G, cuda))
+    refs = (otp.forward(oprob, X, Y, W),) + otp.backward(oprob, X, Y, W, G)
+    for nm, a, b in zip(("Z", "dX", "dY", "dW"), (z.detach(), x.grad, y.grad, w.grad), refs):
+        assert rel_err(a.cpu().numpy(), b) <= FP32_TOL, nm
+    zraw = _misaligned(np.zeros_like(G), cuda)
+    tp.forward_raw(n, x.data_ptr(), y.data_ptr(), zraw.data_ptr(), w.data_ptr())
+    torch.cuda.synchronize()
+    assert rel_err(zraw.cpu().numpy(), refs[0]) <= FP32_TOL
