@@ -101,6 +101,8 @@ class UVWGenerator:
         dflt = ("4", "1") if self.T == "float" else ("1", "3")
         self.fwd_group = int(os.environ.get("OEQ_AMD_UVW_GROUP", dflt[0]))
         self.fwd_unroll = int(os.environ.get("OEQ_AMD_UVW_UNROLL", dflt[1]))
+        # backward dX/dY: register sets for the packed weight fragments (2 = fetched one item ahead)
+        self.bwd_a_sets = int(os.environ.get("OEQ_AMD_UVW_ASETS", "1"))
         self.in1, self.in2, self.out = _blocks(problem.irreps_in1), _blocks(problem.irreps_in2), _blocks(problem.irreps_out)
         self.D1, self.D2, self.D3 = problem.irreps_in1.dim, problem.irreps_in2.dim, problem.irreps_out.dim
         self.WN = problem.weight_numel
@@ -142,9 +144,12 @@ class UVWGenerator:
             p.wb = pos
             pos += p.SU * 64 * p.NTW
         self.WB_SIZE = pos
+        # backward copy: [u-subtile][group of VW steps][lane][VW], so that one 16-byte load per lane
+        # is a contiguous 1 KB access of the wavefront
+        self.VW = 16 // self.itemsize
         for p in self.paths:
             p.wa = pos
-            pos += p.NTU * 64 * p.SW
+            pos += p.NTU * _ceil(p.SW, self.VW) * 64 * self.VW
         self.WA_END = pos
         self.PART_OFF = _ceil(pos, 64) * 64
         self.ws_elems = self.PART_OFF + self.DW_WORKGROUPS * self.WN
@@ -215,10 +220,11 @@ class UVWGenerator:
             E(f"    const int u = 4 * s + (ln >> 4); const int w = {p.NTW} * (ln & 15) + nt;")
             E(f"    wsT[q] = (u < {p.mu} && w < {p.mw}) ? W[{self.oeq_index(p, 'u', 'w')}] : (T)0;")
             E("}")
-            na = p.NTU * 64 * p.SW
-            E(f"if (q >= {p.wa} && q < {p.wa + na}) {{   // backward copy of path {p.t}: [mt][lane][s]")
+            VW, SQ = self.VW, _ceil(p.SW, self.VW)
+            na = p.NTU * SQ * 64 * VW
+            E(f"if (q >= {p.wa} && q < {p.wa + na}) {{   // backward copy of path {p.t}: [mt][s / {VW}][lane][s % {VW}]")
             E(f"    const int e = q - {p.wa};")
-            E(f"    const int s = e % {p.SW}; const int ln = (e / {p.SW}) & 63; const int mt = e / {64 * p.SW};")
+            E(f"    const int ln = (e / {VW}) & 63; const int s = {VW} * ((e / {64 * VW}) % {SQ}) + e % {VW}; const int mt = e / {64 * VW * SQ};")
             E(f"    const int u = 16 * mt + (ln & 15); const int w = 4 * s + (ln >> 4);")
             E(f"    wsT[q] = (u < {p.mu} && w < {p.mw}) ? W[{self.oeq_index(p, 'u', 'w')}] : (T)0;")
             E("}")
@@ -340,40 +346,77 @@ class UVWGenerator:
                     E(f"const T* __restrict__ xp{ai}_{q}_{r} = Xr + {a.off} + min({uexp}, {a.mul - 1}) * {a.D};")
                     E("const T " + ", ".join(f"x{ai}_{q}_{r}_{i} = xp{ai}_{q}_{r}[{i}]" for i in range(a.D)) + ";")
                     E("T " + ", ".join(f"dx{ai}_{q}_{r}_{i} = (T)0" for i in range(a.D)) + ";")
+        # Work list of this wavefront: (output block, path, u-subtile group).  The packed weight
+        # fragments (MFMA A operand) of the next item are fetched into a second register set while
+        # the current item runs, and the dZ records of the next output block are requested as soon
+        # as the last matrix-core step of the current one is issued, so that neither L2 nor HBM
+        # latency sits between two items.
+        items = [(oi, p, q) for oi in self.used_out for p in self.paths_into(oi) for q in range(_ceil(p.NTU, 4))]
+        max_sw = max(_ceil(self.out[oi].mul, 4) for oi in self.used_out)
+        NSETS = self.bwd_a_sets
+        E("T " + ", ".join(f"af{b_}_{s_}" for b_ in range(NSETS) for s_ in range(max_sw)) + ";")
+
+        def load_a(E, j):
+            oi, p, q = items[j]
+            SW = _ceil(self.out[oi].mul, 4)
+            mt = f"wave + {4 * q}" if p.NTU % 4 == 0 else f"min(wave + {4 * q}, {p.NTU - 1})"
+            VW, SQ = self.VW, _ceil(SW, self.VW)
+            E(f"{{ const T* __restrict__ ap = wsT + {p.wa} + (({mt}) * {SQ * 64} + lane) * {VW}; "
+              + " ".join(f"af{j % NSETS}_{s_} = ap[{(s_ // VW) * 64 * VW + s_ % VW}];" for s_ in range(SW)) + " }")
+
+        def load_gz(E, oi):
+            o = self.out[oi]
+            for s_ in range(_ceil(o.mul, 4)):
+                wexp = f"{4 * s_} + g" if o.mul % 4 == 0 else f"min({4 * s_} + g, {o.mul - 1})"
+                E(f"{{ const T* __restrict__ gp = Gr + {o.off} + ({wexp}) * {o.D}; "
+                  + " ".join(f"gz{oi}_{s_}_{k} = gp[{k}];" for k in range(o.D)) + " }")
+                if o.mul % 4 != 0:
+                    E(f"if ({4 * s_} + g >= {o.mul}) {{ " + " ".join(f"gz{oi}_{s_}_{k} = (T)0;" for k in range(o.D)) + " }")
+
         for oi in self.used_out:
             o = self.out[oi]
+            E("T " + ", ".join(f"gz{oi}_{s_}_{k}" for s_ in range(_ceil(o.mul, 4)) for k in range(o.D)) + ";")
+        load_gz(E, items[0][0])
+        load_a(E, 0)
+        for j, (oi, p, q) in enumerate(items):
+            o, a = self.out[oi], p.a
             SW = _ceil(o.mul, 4)
-            E(f"{{ // output block {oi}: dZ records of this lane, w = 4s + g")
+            last_of_block = (j + 1 == len(items)) or items[j + 1][0] != oi
+            E(f"{{ // output block {oi}, path {p.t}, u-subtile wave + {4 * q}")
             E.level += 1
-            for s in range(SW):
-                if o.mul % 4 == 0:
-                    E(f"const T* __restrict__ gp{s} = Gr + {o.off} + ({4 * s} + g) * {o.D};")
-                    E("const T " + ", ".join(f"gz{s}_{k} = gp{s}[{k}]" for k in range(o.D)) + ";")
-                else:
-                    E(f"const T* __restrict__ gp{s} = Gr + {o.off} + min({4 * s} + g, {o.mul - 1}) * {o.D};")
-                    E("T " + ", ".join(f"gz{s}_{k} = gp{s}[{k}]" for k in range(o.D)) + ";")
-                    E(f"if ({4 * s} + g >= {o.mul}) {{ " + " ".join(f"gz{s}_{k} = (T)0;" for k in range(o.D)) + " }")
-            for p in self.paths_into(oi):
-                a = p.a
-                for q in range(_ceil(p.NTU, 4)):
-                    E(f"// path {p.t}, u-subtile wave + {4 * q}")
-                    E(f"if (wave + {4 * q} < {p.NTU}) {{")
-                    E.level += 1
-                    E(f"const int mt = wave + {4 * q};")
-                    E(f"const T* __restrict__ ap = wsT + {p.wa} + (mt * 64 + lane) * {SW};")
-                    for k in range(o.D):
-                        E(f"V4 acc{k} = {{0, 0, 0, 0}};")
-                    for s in range(SW):
-                        E(f"{{ const T a_ = ap[{s}]; " + " ".join(f"acc{k} = oeq_mfma(a_, gz{s}_{k}, acc{k});" for k in range(o.D)) + " }")
-                    for r in range(4):
-                        E(f"{{ // row {r} of the tile: channel u = 16 mt + row, batch row b = row0 + c")
-                        E("  const T " + ", ".join(f"dt{k} = acc{k}[{r}]" for k in range(o.D)) + ";")
-                        E.level += 1
-                        self.emit_cg_backward(E, p, "dt", f"x{a.idx}_{q}_{r}_", "y", f"dx{a.idx}_{q}_{r}_", "dy")
-                        E.level -= 1
-                        E("}")
-                    E.level -= 1
-                    E("}")
+            # The two halves of an item sit in branches of their own (taken by every wavefront that
+            # owns a u-subtile of this path): basic-block boundaries are what keeps the compiler from
+            # sinking the vector-ALU halves of all items below the matrix-core work, which would keep
+            # every accumulator alive and halve the occupancy.
+            cond = f"wave + {4 * q} < {p.NTU}"
+            if j + 1 < len(items) and NSETS == 2:
+                load_a(E, j + 1)
+            for k in range(o.D):
+                E(f"V4 acc{k} = {{0, 0, 0, 0}};")
+            E(f"if ({cond}) {{")
+            E.level += 1
+            for s_ in range(SW):
+                E(" ".join(f"acc{k} = oeq_mfma(af{j % NSETS}_{s_}, gz{oi}_{s_}_{k}, acc{k});" for k in range(o.D)))
+            E.level -= 1
+            E("}")
+            if j + 1 < len(items) and (NSETS == 1 or last_of_block):
+                # the fragment registers (one set) and, at the end of a block, the dZ registers are free
+                # from here on: request the next ones now, the vector-ALU part below covers the latency
+                if NSETS == 1:
+                    load_a(E, j + 1)
+                if last_of_block:
+                    load_gz(E, items[j + 1][0])
+            E(f"if ({cond}) {{")
+            E.level += 1
+            for r in range(4):
+                E(f"{{ // row {r} of the tile: channel u = 16 mt + row, batch row b = row0 + c")
+                E("  const T " + ", ".join(f"dt{k} = acc{k}[{r}]" for k in range(o.D)) + ";")
+                E.level += 1
+                self.emit_cg_backward(E, p, "dt", f"x{a.idx}_{q}_{r}_", "y", f"dx{a.idx}_{q}_{r}_", "dy")
+                E.level -= 1
+                E("}")
+            E.level -= 1
+            E("}")
             E.level -= 1
             E("}")
         # ---- dX stores

@@ -66,6 +66,7 @@ static inline T oeq_wave_sum63(T v) { g_xT[threadIdx.x] = v; oeq_sync(); T t = 0
 static inline T oeq_ldnt(const T* p) { return *p; }
 static inline void oeq_stnt(T* p, T v) { *p = v; }
 static inline void oeq_block_sync() { pthread_barrier_wait(&g_bar); }
+static inline void oeq_sched_fence() {}
 static inline void __syncthreads() { pthread_barrier_wait(&g_bar); }
 #define __HIP_MEMORY_SCOPE_AGENT 0
 template <class V> static inline V __hip_atomic_fetch_add(V* p, V v, int, int) { std::lock_guard<std::mutex> g(g_atomic_mutex); V o = *p; *p += v; return o; }
