@@ -444,7 +444,12 @@ class UVUGenerator:
 
     # ------------------------------------------------------------- dY reduction
     def emit_dy_reduce(self, E: Emitter) -> None:
-        """Butterfly sum of dy* over the P lanes of each sub-row (fixed order -> deterministic)."""
+        """Sum of dy* over the P lanes of each sub-row (fixed order -> deterministic): DPP row
+        operations for groups of up to 32 lanes, a shuffle butterfly for a full wavefront."""
+        if self.P <= 32:
+            for f in self.used_y:
+                E(f"dy{f} = oeq_group_sum<{self.P}>(dy{f});")
+            return
         m = self.P // 2
         while m >= 1:
             for f in self.used_y:

@@ -119,9 +119,7 @@ class UVUDetGenerator(UVUDirectGenerator):
             names += [f"x{i}_{m}" for m in range(self.in1[i].D)]
         names += [f"We_{p.t}_{v}" for p in self.paths for v in range(p.mv)]
         names += [f"y{f}" for f in self.used_y]
-        E("T " + ", ".join(f"N{n} = (T)0" for n in names) + ";")
-
-        def load(E, it):
+        def load(E, it, h):
             E("{")
             E.level += 1
             E(f"const bool ev = {self.edge_pos(it)} < len;")
@@ -140,35 +138,23 @@ class UVUDetGenerator(UVUDirectGenerator):
             E(f"const T* __restrict__ Yr = Y + e * {self.D2};")
             E(f"const T* __restrict__ Wr = W + e * {self.WN};")
             for f in self.used_y:
-                E(f"Ny{f} = {self.ld('Yr', f)};")
+                E(f"S{h}y{f} = {self.ld('Yr', f)};")
             for i in self.used_in1:
                 a = self.in1[i]
                 E(f"{{ const T* __restrict__ p_ = X + sndc * {self.D1} + {a.off} + {self.uclamp(a, 0)} * {a.D}; "
-                  + " ".join(f"Nx{i}_{m} = p_[{m}];" for m in range(a.D)) + " }")
+                  + " ".join(f"S{h}x{i}_{m} = p_[{m}];" for m in range(a.D)) + " }")
                 # everything an edge adds is proportional to x: zero it for idle lanes
-                E(f"if (!({self.act(a)})) {{ " + " ".join(f"Nx{i}_{m} = (T)0;" for m in range(a.D)) + " }")
+                E(f"if (!({self.act(a)})) {{ " + " ".join(f"S{h}x{i}_{m} = (T)0;" for m in range(a.D)) + " }")
             for p in self.paths:
                 for v in range(p.mv):
-                    E(f"NWe_{p.t}_{v} = {self.ld('Wr', self.widx(p, self.uclamp(p.a, 0), v))};")
+                    E(f"S{h}We_{p.t}_{v} = {self.ld('Wr', self.widx(p, self.uclamp(p.a, 0), v))};")
             E.level -= 1
             E("}")
-        E("if (maxlen > 0) {")
-        E.level += 1
-        load(E, "0")
-        E.level -= 1
-        E("}")
-        E("for (int it = 0; it < maxlen; ++it) {")
-        E.level += 1
-        E("const T " + ", ".join(f"{n} = N{n}" for n in names) + ";")
-        E("if (it + 1 < maxlen) {")
-        E.level += 1
-        load(E, "it + 1")
-        E.level -= 1
-        E("}")
-        for oi in self.used_out:
-            self.emit_forward_block(E, self.out[oi], "Wr", zname=f"z{oi}_", declare=False)
-        E.level -= 1
-        E("}")
+
+        def compute(E, h):
+            for oi in self.used_out:
+                self.emit_forward_block(E, self.out[oi], "Wr", zname=f"z{oi}_", declare=False)
+        self.emit_pingpong_loop(E, names, load, compute)
         E("const bool rv = nv;")
         for o in self.out:
             if o.dim == 0:
@@ -192,6 +178,59 @@ class UVUDetGenerator(UVUDirectGenerator):
     def uclamp(self, blk, c) -> str:
         return "u" if self.full(blk) else f"min(u, {blk.mul - 1})"
 
+    def emit_pingpong_loop(self, E: Emitter, names, load, compute, scalars: str = "", prefetch_first: bool = True) -> None:
+        """The edge loop, software pipelined over two register sets: while the edge held in one set is
+        computed, the operands of the following edge are in flight into the other set.  The loop body is
+        emitted twice (one copy per set) so that no register is copied from "next" to "current" at the
+        loop head.  ``load(E, it, h)`` fills set h for iteration ``it``; ``compute(E, h)`` sees the names
+        without prefix.  ``prefetch_first=False`` (large register footprints) keeps one set and requests the
+        next edge after the arithmetic."""
+        for h in (0, 1):
+            E("T " + ", ".join(f"S{h}{n} = (T)0" for n in names) + ";")
+        if scalars:
+            E(scalars)
+        E("if (maxlen > 0) {")
+        E.level += 1
+        load(E, "0", 0)
+        E.level -= 1
+        E("}")
+        if not prefetch_first:
+            # one register set is enough: it is refilled once the arithmetic on it is done
+            E("for (int it = 0; it < maxlen; ++it) {")
+            E.level += 1
+            E("const T " + ", ".join(f"{n} = S0{n}" for n in names) + ";")
+            compute(E, 0)
+            E("if (it + 1 < maxlen) {")
+            E.level += 1
+            load(E, "it + 1", 0)
+            E.level -= 1
+            E("}")
+            E.level -= 1
+            E("}")
+            return
+        E("for (int it = 0; it < maxlen; it += 2) {")
+        E.level += 1
+        for h in (0, 1):
+            nxt = f"it + {h + 1}"
+            if h == 1:
+                E("if (it + 1 >= maxlen) break;")
+            E("{")
+            E.level += 1
+            E("const T " + ", ".join(f"{n} = S{h}{n}" for n in names) + ";")
+
+            def prefetch():
+                E(f"if ({nxt} < maxlen) {{")
+                E.level += 1
+                load(E, nxt, 1 - h)
+                E.level -= 1
+                E("}")
+            prefetch()
+            compute(E, h)
+            E.level -= 1
+            E("}")
+        E.level -= 1
+        E("}")
+
     # ================================================================ backward
     def conv_det_backward_body(self) -> str:
         E = Emitter()
@@ -209,10 +248,7 @@ class UVUDetGenerator(UVUDirectGenerator):
         names = [f"G{oi}_{k}" for oi in self.used_out for k in range(self.out[oi].D)]
         names += [f"We_{p.t}_{v}" for p in self.paths for v in range(p.mv)]
         names += [f"y{f}" for f in self.used_y]
-        E("T " + ", ".join(f"N{n} = (T)0" for n in names) + ";")
-        E("u64 Ne = 0; bool Nrv = false;")
-
-        def load(E, it):
+        def load(E, it, h):
             E("{")
             E.level += 1
             E(f"const bool ev = {self.edge_pos(it)} < len;")
@@ -223,70 +259,52 @@ class UVUDetGenerator(UVUDirectGenerator):
             E("const i64 rcv = rows[e];")
             E("const bool rv = ok_e && rcv >= 0 && rcv < (i64)node_count;")
             E("const u64 rcvc = rv ? (u64)rcv : 0;")
-            E("Ne = e; Nrv = rv;")
+            E(f"S{h}e = e; S{h}rv = rv;")
             E(f"const T* __restrict__ Yr = Y + e * {self.D2};")
             E(f"const T* __restrict__ Wr = W + e * {self.WN};")
             for f in self.used_y:
-                E(f"Ny{f} = {self.ld('Yr', f)};")
+                E(f"S{h}y{f} = {self.ld('Yr', f)};")
             for p in self.paths:
                 for v in range(p.mv):
-                    E(f"NWe_{p.t}_{v} = {self.ld('Wr', self.widx(p, self.uclamp(p.a, 0), v))};")
+                    E(f"S{h}We_{p.t}_{v} = {self.ld('Wr', self.widx(p, self.uclamp(p.a, 0), v))};")
             for oi in self.used_out:
                 o = self.out[oi]
                 E(f"{{ const T* __restrict__ p_ = G + rcvc * {self.D3} + {o.off} + {self.uclamp(o, 0)} * {o.D}; "
-                  + " ".join(f"NG{oi}_{k} = p_[{k}];" for k in range(o.D)) + " }")
+                  + " ".join(f"S{h}G{oi}_{k} = p_[{k}];" for k in range(o.D)) + " }")
                 # every gradient of an edge is proportional to dZ: zero it for idle lanes
-                E(f"if (!({self.act(o)})) {{ " + " ".join(f"NG{oi}_{k} = (T)0;" for k in range(o.D)) + " }")
+                E(f"if (!({self.act(o)})) {{ " + " ".join(f"S{h}G{oi}_{k} = (T)0;" for k in range(o.D)) + " }")
             E.level -= 1
             E("}")
-        E("if (maxlen > 0) {")
-        E.level += 1
-        load(E, "0")
-        E.level -= 1
-        E("}")
-        E("for (int it = 0; it < maxlen; ++it) {")
-        E.level += 1
-        E("const T " + ", ".join(f"{n} = N{n}" for n in names) + ";")
-        E("const u64 e = Ne; rv = Nrv;")
-        if self.prefetch_backward:
-            E("if (it + 1 < maxlen) {")
-            E.level += 1
-            load(E, "it + 1")
-            E.level -= 1
-            E("}")
-        E(f"T* __restrict__ Wgr = Wg + e * {self.WN};")
-        for f in self.used_y:
-            E(f"T dy{f} = (T)0;")
-        for oi in self.used_out:
-            o = self.out[oi]
-            E("{")
-            E.level += 1
-            for k in range(o.D):
-                E(f"const T g{k} = G{oi}_{k};")
 
-            def sink(E, p, v, expr):
-                E(f"  if ({self.act(p.a)}) {self.st('Wgr', self.widx(p, 'u', v), expr)}")
-            self.emit_backward_block(E, o, "Wr", sink)
-            E.level -= 1
+        def compute(E, h):
+            E(f"const u64 e = S{h}e; rv = S{h}rv;")
+            E(f"T* __restrict__ Wgr = Wg + e * {self.WN};")
+            for f in self.used_y:
+                E(f"T dy{f} = (T)0;")
+            for oi in self.used_out:
+                o = self.out[oi]
+                E("{")
+                E.level += 1
+                for k in range(o.D):
+                    E(f"const T g{k} = G{oi}_{k};")
+
+                def sink(E, p, v, expr):
+                    E(f"  if ({self.act(p.a)}) {self.st('Wgr', self.widx(p, 'u', v), expr)}")
+                self.emit_backward_block(E, o, "Wr", sink)
+                E.level -= 1
+                E("}")
+            self.emit_dy_sum(E)
+            writer = "ul == 0" if self.P < 64 else "lane == 63"
+            E(f"if (rv && {writer}) {{")
+            if self.NCH > 1:
+                E(f"    T* __restrict__ Ygr = (T*)((char*)ws + DYPART_OFF) + ((u64)c * nnz + e) * {self.D2};")
+            else:
+                E(f"    T* __restrict__ Ygr = Yg + e * {self.D2};")
+            for f in range(self.D2):
+                E(f"    Ygr[{f}] = " + (f"dy{f};" if f in self.used_y else "(T)0;"))
             E("}")
-        self.emit_dy_sum(E)
-        writer = "ul == 0" if self.P < 64 else "lane == 63"
-        E(f"if (rv && {writer}) {{")
-        if self.NCH > 1:
-            E(f"    T* __restrict__ Ygr = (T*)((char*)ws + DYPART_OFF) + ((u64)c * nnz + e) * {self.D2};")
-        else:
-            E(f"    T* __restrict__ Ygr = Yg + e * {self.D2};")
-        for f in range(self.D2):
-            E(f"    Ygr[{f}] = " + (f"dy{f};" if f in self.used_y else "(T)0;"))
-        E("}")
-        if not self.prefetch_backward:
-            E("if (it + 1 < maxlen) {")
-            E.level += 1
-            load(E, "it + 1")
-            E.level -= 1
-            E("}")
-        E.level -= 1
-        E("}")
+        self.emit_pingpong_loop(E, names, load, compute, scalars="u64 S0e = 0, S1e = 0; bool S0rv = false, S1rv = false;",
+                                prefetch_first=self.prefetch_backward)
         E("rv = nv;")
         for a in self.in1:
             if a.dim == 0:

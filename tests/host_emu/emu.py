@@ -63,6 +63,7 @@ static inline void oeq_dma16(const T* g, T* lds_base) { memcpy((char*)lds_base +
 static inline void oeq_wait_vm() {}
 static inline void oeq_wait_lds() {}
 static inline T oeq_wave_sum63(T v) { g_xT[threadIdx.x] = v; oeq_sync(); T t = 0; for (int i = 0; i < 64; ++i) t += g_xT[(threadIdx.x & ~63) + i]; oeq_sync(); return t; }
+template <int P> static inline T oeq_group_sum(T v) { g_xT[threadIdx.x] = v; oeq_sync(); T t = 0; for (int i = 0; i < P; ++i) t += g_xT[(threadIdx.x & ~(P - 1)) + i]; oeq_sync(); return t; }
 static inline T oeq_ldnt(const T* p) { return *p; }
 static inline void oeq_stnt(T* p, T v) { *p = v; }
 static inline void oeq_block_sync() { pthread_barrier_wait(&g_bar); }
