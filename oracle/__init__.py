@@ -19,7 +19,7 @@ How each function is pinned (a function with no such check would be marked
                        sympy's Clebsch-Gordan coefficients; closed-form special
                        cases; ``|C| = 1``; rotation invariance
 ``spec.Problem``       golden path coefficients from the reference's
-                       ``TPProblem`` (tests/golden/problems.json); hand values
+                       ``TPProblem`` (tests/golden/tpproblem.json, all normalisation modes); hand values
                        (sqrt 5; sqrt(2l3+1); sqrt(1/192), sqrt(3/256), sqrt(5/256))
 ``spec.channelwise``   path counts / dims / weight counts of the five benchmark
 ``spec.fully_conn..``  configurations and the explicit column tables

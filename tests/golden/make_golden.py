@@ -1,4 +1,5 @@
-"""Writes tests/golden/wigner_3j.npz from the reference's own ``wigner_3j``.
+"""Writes tests/golden/wigner_3j.npz from the reference's own ``wigner_3j`` and
+tests/golden/tpproblem.json from the reference's own ``TPProblem``.
 
 The sign convention of the real-basis coupling tensors is the one thing about
 the oracle that no invariant, special case or third-party library fixes (a
@@ -6,15 +7,94 @@ global sign per (l1, l2, l3) survives all of them), so these vectors are taken
 from the reference itself.  The reference file is numpy-only and is loaded by
 path, in the build container only; the output is plain data.
 
+The second fixture pins the normalisation: for literal instruction lists (written out below, no
+reference enumeration helper is used) it records what the reference's ``TPProblem`` computes - the
+final coefficient of every instruction, its weight shape, ``weight_numel`` and the irreps' sizes -
+for the default and the non-default normalisation modes, variances and user path weights.
+
     python tests/golden/make_golden.py [/root/reference]
 """
 import importlib.util
+import json
 import pathlib
 import sys
 
 import numpy as np
 
 LMAX = 4
+
+SH2, SH3 = "1x0e+1x1o+1x2e", "1x0e+1x1o+1x2e+1x3o"
+
+
+def _parse(irreps):
+    out = []
+    for tok in irreps.replace(" ", "").split("+"):
+        mul, ir = tok.split("x") if "x" in tok else ("1", tok)
+        out.append((int(mul), int(ir[:-1]), 1 if ir[-1] == "e" else -1))
+    return out
+
+
+def _channelwise(in1, in2, lmax_out, natural):
+    """Instruction list of a channelwise product: every allowed (i1, i2) -> l3 <= lmax_out path gets an
+    output slot of its own; slots sorted by (l, parity) then creation order, parity -1 first."""
+    a, b = _parse(in1), _parse(in2)
+    slots = []
+    for i, (m1, l1, p1) in enumerate(a):
+        for j, (_, l2, p2) in enumerate(b):
+            for l3 in range(abs(l1 - l2), l1 + l2 + 1):
+                p3 = p1 * p2
+                if l3 <= lmax_out and (not natural or p3 == (-1) ** l3):
+                    slots.append((l3, p3, len(slots), i, j, m1))
+    slots.sort(key=lambda t: (t[0], t[1], t[2]))
+    out = "+".join(f"{m}x{l}{'e' if p == 1 else 'o'}" for l, p, _, _, _, m in slots)
+    ins = [(i, j, k, "uvu", True) for k, (_, _, _, i, j, _) in enumerate(slots)]
+    return out, ins
+
+
+def _fully_connected(in1, in2, out):
+    a, b, c = _parse(in1), _parse(in2), _parse(out)
+    return [(i, j, k, "uvw", True, 1.0) for i, (_, l1, p1) in enumerate(a) for j, (_, l2, p2) in enumerate(b)
+            for k, (_, l3, p3) in enumerate(c) if p3 == p1 * p2 and abs(l1 - l2) <= l3 <= l1 + l2]
+
+
+def problem_cases():
+    cases = [dict(name="readme", in1="1x2e", in2="1x3e", out="1x2e", ins=[(0, 0, 0, "uvu", True)], kw={})]
+    for name, in1, in2, lmax in (("mace", "128x0e+128x1o+128x2e", SH3, 3), ("nequip", "32x0e+32x1o+32x2e", SH2, 2),
+                                 ("large", "256x0e+256x1o+256x2e", SH3, 2)):
+        out, ins = _channelwise(in1, in2, lmax, natural=True)
+        cases.append(dict(name=name, in1=in1, in2=in2, out=out, ins=ins, kw={}))
+    out, ins = _channelwise("128x0e+128x1o+128x2e", SH3, 3, natural=False)
+    cases.append(dict(name="mace_all_parities", in1="128x0e+128x1o+128x2e", in2=SH3, out=out, ins=ins, kw={}))
+    d = "64x0e+64x1o+64x2e"
+    cases.append(dict(name="dense_uvw", in1=d, in2=SH2, out=d, ins=_fully_connected(d, SH2, d), kw=dict(shared_weights=True)))
+    # non-default modes on a small mixed problem, with user path weights and variances
+    in1, in2, out = "3x0e+2x1o", "2x0e+1x1o", "4x0e+3x1o+2x1e"
+    ins = [(0, 0, 0, "uvw", True, 1.0), (1, 1, 0, "uvw", True, 2.5), (0, 1, 1, "uvw", True, 0.5),
+           (1, 0, 1, "uvw", True, 1.0), (1, 1, 2, "uvw", True, 3.0)]
+    for irn in ("component", "norm", "none"):
+        for pn in ("element", "path", "none"):
+            cases.append(dict(name=f"modes_{irn}_{pn}", in1=in1, in2=in2, out=out, ins=ins,
+                              kw=dict(irrep_normalization=irn, path_normalization=pn)))
+    cases.append(dict(name="variances", in1=in1, in2=in2, out=out, ins=ins,
+                      kw=dict(in1_var=[1.0, 0.5], in2_var=[2.0, 0.25], out_var=[3.0, 0.125, 1.5])))
+    cases.append(dict(name="uvu_mul2", in1="4x0e+4x1o", in2="2x0e+2x1o", out="4x0e+4x1o+4x1o",
+                      ins=[(0, 0, 0, "uvu", True), (0, 1, 1, "uvu", True, 2.0), (1, 0, 2, "uvu", True), (1, 1, 0, "uvu", True)], kw={}))
+    return cases
+
+
+def write_problem_fixture(mod, dest):
+    out = []
+    for c in problem_cases():
+        tpp = mod.TPProblem(c["in1"], c["in2"], c["out"], [tuple(t) for t in c["ins"]], **c["kw"])
+        out.append(dict(name=c["name"], irreps_in1=c["in1"], irreps_in2=c["in2"], irreps_out=c["out"],
+                        instructions=[list(t) for t in c["ins"]], kwargs=c["kw"],
+                        expect=dict(path_weights=[float(i.path_weight) for i in tpp.instructions],
+                                    path_shapes=[list(i.path_shape) for i in tpp.instructions],
+                                    weight_numel=int(tpp.weight_numel),
+                                    dims=[int(tpp.irreps_in1.dim), int(tpp.irreps_in2.dim), int(tpp.irreps_out.dim)],
+                                    shared_weights=bool(tpp.shared_weights), internal_weights=bool(tpp.internal_weights))))
+    dest.write_text(json.dumps(out, indent=1) + "\n")
+    print(f"wrote {len(out)} problems to {dest}")
 
 
 def main():
@@ -31,6 +111,7 @@ def main():
     dest = pathlib.Path(__file__).with_name("wigner_3j.npz")
     np.savez_compressed(dest, **out)
     print(f"wrote {len(out)} tensors to {dest}")
+    write_problem_fixture(mod, pathlib.Path(__file__).with_name("tpproblem.json"))
 
 
 if __name__ == "__main__":

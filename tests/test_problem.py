@@ -100,3 +100,56 @@ def test_constructor_errors():
     p = oeq.TPProblem("1x0e", "1x0e", "1x0e", [(0, 0, 0, "uvu", False)])
     with pytest.raises(ValueError):
         p.weight_range_and_shape_for_instruction(0)
+
+
+# ------------------------------------------------------------------ golden vectors of the reference's TPProblem
+import json
+import pathlib
+
+GOLDEN_PROBLEMS = json.loads((pathlib.Path(__file__).parent / "golden" / "tpproblem.json").read_text())
+
+
+@pytest.mark.parametrize("case", GOLDEN_PROBLEMS, ids=[c["name"] for c in GOLDEN_PROBLEMS])
+def test_normalisation_matches_reference_golden(case):
+    """Final path coefficients, weight shapes and sizes as computed by the reference's own TPProblem
+    (tests/golden/make_golden.py), for the product's TPProblem and for the oracle's restatement."""
+    from oracle import spec
+    ins = [tuple(t) for t in case["instructions"]]
+    exp = case["expect"]
+    tpp = oeq.TPProblem(case["irreps_in1"], case["irreps_in2"], case["irreps_out"], ins, **case["kwargs"])
+    assert [list(t.path_shape) for t in tpp.instructions] == exp["path_shapes"]
+    assert np.allclose([t.path_weight for t in tpp.instructions], exp["path_weights"], rtol=1e-14, atol=0)
+    assert tpp.weight_numel == exp["weight_numel"]
+    assert [tpp.irreps_in1.dim, tpp.irreps_in2.dim, tpp.irreps_out.dim] == exp["dims"]
+    assert bool(tpp.shared_weights) == exp["shared_weights"] and bool(tpp.internal_weights) == exp["internal_weights"]
+    kw = {k: v for k, v in case["kwargs"].items() if k != "shared_weights"}
+    op = spec.Problem(case["irreps_in1"], case["irreps_in2"], case["irreps_out"], ins,
+                      shared_weights=exp["shared_weights"], **kw)
+    assert np.allclose([p["coeff"] for p in op.paths], exp["path_weights"], rtol=1e-14, atol=0)
+    assert [list(p["shape"]) for p in op.paths] == exp["path_shapes"]
+    assert op.weight_numel == exp["weight_numel"] and [op.d1, op.d2, op.d3] == exp["dims"]
+
+
+@pytest.mark.parametrize("name,irreps", [("mace", common.MACE), ("nequip", common.NEQUIP), ("large", common.LARGE),
+                                         ("mace_all_parities", ("128x0e+128x1o+128x2e", "1x0e+1x1o+1x2e+1x3o",
+                                                                "128x0e+128x1o+128x1e+128x2e+128x2o+128x3o+128x3e"))])
+def test_channelwise_enumeration_matches_the_fixture(name, irreps):
+    """The instruction order and output layout spelled out in the fixture (a literal enumeration,
+    accepted by the reference's TPProblem) are what ChannelwiseTPP and the oracle produce."""
+    from oracle import spec
+    case = next(c for c in GOLDEN_PROBLEMS if c["name"] == name)
+    prob = oeq.ChannelwiseTPP(*irreps)
+    got = [(t.i_in1, t.i_in2, t.i_out) for t in prob.instructions]
+    assert got == [tuple(t[:3]) for t in case["instructions"]]
+    assert str(prob.irreps_out).replace(" ", "") == case["irreps_out"]
+    op = spec.channelwise(*irreps)
+    assert [(p["i1"], p["i2"], p["io"]) for p in op.paths] == got
+
+
+def test_fully_connected_enumeration_matches_the_fixture():
+    from oracle import spec
+    case = next(c for c in GOLDEN_PROBLEMS if c["name"] == "dense_uvw")
+    prob = oeq.FullyConnectedTPProblem(*common.DENSE, shared_weights=True, internal_weights=False)
+    got = [(t.i_in1, t.i_in2, t.i_out, t.connection_mode) for t in prob.instructions]
+    assert got == [tuple(t[:4]) for t in case["instructions"]]
+    assert [(p["i1"], p["i2"], p["io"], p["mode"]) for p in spec.fully_connected(*common.DENSE, shared_weights=True).paths] == got
