@@ -103,6 +103,9 @@ class UVWGenerator:
         self.fwd_unroll = int(os.environ.get("OEQ_AMD_UVW_UNROLL", dflt[1]))
         # backward dX/dY: register sets for the packed weight fragments (2 = fetched one item ahead)
         self.bwd_a_sets = int(os.environ.get("OEQ_AMD_UVW_ASETS", "1"))
+        self._bwd_lds_env = os.environ.get("OEQ_AMD_UVW_BWD_LDS", "1") == "1"
+        # backward dW: fetch the operands of the next step while the current one runs (two register sets)
+        self.dw_prefetch = os.environ.get("OEQ_AMD_UVW_DW_PREFETCH", "1" if self.T == "float" else "0") == "1"
         self.in1, self.in2, self.out = _blocks(problem.irreps_in1), _blocks(problem.irreps_in2), _blocks(problem.irreps_out)
         self.D1, self.D2, self.D3 = problem.irreps_in1.dim, problem.irreps_in2.dim, problem.irreps_out.dim
         self.WN = problem.weight_numel
@@ -138,6 +141,10 @@ class UVWGenerator:
             gsel = 0 if (load[0] <= load[1] or self.dw_groups == 1) else 1
             self.dw_group[o] = gsel
             load[gsel] += work[o]
+        # backward dX/dY: the 16-row dZ tile is staged in LDS when it fits (row stride padded against bank
+        # conflicts of the B-operand reads: lanes c = 0..15 read 16 different rows at the same column)
+        self.bwd_rs = self._pick_row_stride()
+        self.bwd_lds = self._bwd_lds_env and 16 * self.bwd_rs * self.itemsize <= 80 * 1024    # gfx950: 160 KB per CU
         # packed weight copies in the workspace
         pos = 0
         for p in self.paths:
@@ -155,6 +162,27 @@ class UVWGenerator:
         self.ws_elems = self.PART_OFF + self.DW_WORKGROUPS * self.WN
 
     # ------------------------------------------------------------------ helpers
+    def _pick_row_stride(self) -> int:
+        """Row stride (elements) of the dZ tile in LDS: the smallest padding for which the 32 lanes of
+        one LDS pass (16 rows x 2 adjacent records) spread best over the 32 four-byte banks."""
+        words = self.itemsize // 4
+        best = None
+        for pad in range(0, 33):
+            rs = self.D3 + pad
+            worst = 0
+            for d in {o.D for o in self.out if o.dim}:
+                hits = {}
+                for c in range(16):
+                    for g in range(2):
+                        bank = ((c * rs + g * d) * words) % 32
+                        hits[bank] = hits.get(bank, 0) + 1
+                worst = max(worst, max(hits.values()))
+            if best is None or worst < best[0]:
+                best = (worst, rs)
+            if worst == 1:
+                break
+        return best[1]
+
     def lit(self, v: float) -> str:
         return literal(v, self.T)
 
@@ -333,6 +361,35 @@ class UVWGenerator:
         E(f"const T* __restrict__ Xr = X + rowB * {self.D1};")
         E(f"const T* __restrict__ Gr = G + rowB * {self.D3};")
         E(f"__shared__ T dyl[4 * 16 * {max(1, self.D2)}];")
+        if self.bwd_lds:
+            # the dZ tile goes to LDS once per workgroup (coalesced, one HBM round trip), and every
+            # wavefront reads its MFMA B operands from there
+            RS = self.bwd_rs
+            E(f"__shared__ T gl[16 * {RS}];")
+            VW = self.VW
+            if self.D3 % VW == 0:
+                # 16-byte vectors, all requested before the first one is written to LDS
+                NV, RV = 16 * self.D3 // VW, self.D3 // VW
+                NQ = _ceil(NV, 256)
+                E("if ((((unsigned long long)G) & 15ull) == 0) {")
+                E.level += 1
+                E(f"VT gv[{NQ}];")
+                for q in range(NQ):
+                    idx = f"(int)threadIdx.x + {256 * q}"
+                    guard = "" if 256 * (q + 1) <= NV else f"if ({idx} < {NV}) "
+                    E(f"{guard}{{ const int r_ = ({idx}) / {RV}, v_ = ({idx}) - r_ * {RV}; "
+                      f"gv[{q}] = *(const VT*)(G + min(row0 + (u64)r_, n - 1) * {self.D3} + v_ * {VW}); }}")
+                for q in range(NQ):
+                    idx = f"(int)threadIdx.x + {256 * q}"
+                    guard = "" if 256 * (q + 1) <= NV else f"if ({idx} < {NV}) "
+                    E(f"{guard}{{ const int r_ = ({idx}) / {RV}, v_ = ({idx}) - r_ * {RV}; T* __restrict__ d_ = gl + r_ * {RS} + v_ * {VW}; "
+                      + " ".join(f"d_[{i}] = gv[{q}][{i}];" for i in range(VW)) + " }")
+                E.level -= 1
+                E("} else")
+            E(f"for (int q = threadIdx.x; q < 16 * {self.D3}; q += 256) {{")
+            E(f"    const int r_ = q / {self.D3}, col_ = q - r_ * {self.D3};")
+            E(f"    gl[r_ * {RS} + col_] = G[min(row0 + (u64)r_, n - 1) * {self.D3} + col_];")
+            E("}")
         for f in self.used_y:
             E(f"const T y{f} = Y[rowB * {self.D2} + {f}];")
             E(f"T dy{f} = (T)0;")
@@ -373,10 +430,13 @@ class UVWGenerator:
                 if o.mul % 4 != 0:
                     E(f"if ({4 * s_} + g >= {o.mul}) {{ " + " ".join(f"gz{oi}_{s_}_{k} = (T)0;" for k in range(o.D)) + " }")
 
-        for oi in self.used_out:
-            o = self.out[oi]
-            E("T " + ", ".join(f"gz{oi}_{s_}_{k}" for s_ in range(_ceil(o.mul, 4)) for k in range(o.D)) + ";")
-        load_gz(E, items[0][0])
+        if self.bwd_lds:
+            E("oeq_block_sync();")
+        else:
+            for oi in self.used_out:
+                o = self.out[oi]
+                E("T " + ", ".join(f"gz{oi}_{s_}_{k}" for s_ in range(_ceil(o.mul, 4)) for k in range(o.D)) + ";")
+            load_gz(E, items[0][0])
         load_a(E, 0)
         for j, (oi, p, q) in enumerate(items):
             o, a = self.out[oi], p.a
@@ -395,16 +455,26 @@ class UVWGenerator:
                 E(f"V4 acc{k} = {{0, 0, 0, 0}};")
             E(f"if ({cond}) {{")
             E.level += 1
+            if self.bwd_lds:
+                E(f"const T* __restrict__ gb = gl + c * {self.bwd_rs} + {o.off} + g * {o.D};")
             for s_ in range(SW):
-                E(" ".join(f"acc{k} = oeq_mfma(af{j % NSETS}_{s_}, gz{oi}_{s_}_{k}, acc{k});" for k in range(o.D)))
+                if self.bwd_lds:
+                    if o.mul % 4 == 0:
+                        E("{ const T " + ", ".join(f"b{k} = gb[{4 * s_ * o.D + k}]" for k in range(o.D)) + ";")
+                    else:
+                        E(f"{{ const bool in_ = {4 * s_} + g < {o.mul}; const T* __restrict__ gq = in_ ? gb + {4 * s_ * o.D} : gl;")
+                        E("  const T " + ", ".join(f"b{k} = in_ ? gq[{k}] : (T)0" for k in range(o.D)) + ";")
+                    E("  " + " ".join(f"acc{k} = oeq_mfma(af{j % NSETS}_{s_}, b{k}, acc{k});" for k in range(o.D)) + " }")
+                else:
+                    E(" ".join(f"acc{k} = oeq_mfma(af{j % NSETS}_{s_}, gz{oi}_{s_}_{k}, acc{k});" for k in range(o.D)))
             E.level -= 1
             E("}")
-            if j + 1 < len(items) and (NSETS == 1 or last_of_block):
+            if j + 1 < len(items) and (NSETS == 1 or (last_of_block and not self.bwd_lds)):
                 # the fragment registers (one set) and, at the end of a block, the dZ registers are free
                 # from here on: request the next ones now, the vector-ALU part below covers the latency
                 if NSETS == 1:
                     load_a(E, j + 1)
-                if last_of_block:
+                if last_of_block and not self.bwd_lds:
                     load_gz(E, items[j + 1][0])
             E(f"if ({cond}) {{")
             E.level += 1
@@ -471,56 +541,155 @@ class UVWGenerator:
                 for q in range(_ceil(p.NTU, 4)):
                     for nt in range(p.NTW):
                         E(f"V4 acc{p.t}_{q}_{nt} = {{0, 0, 0, 0}};")
-            E("for (u64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {")
-            E.level += 1
-            E("const u64 row0 = tile * 16;")
-            E("#pragma unroll 1")
-            E("for (int sp = 0; sp < 4; ++sp) {")
-            E.level += 1
-            E("const u64 b = row0 + 4 * sp + g;          // batch row of this lane for both operands")
-            E("const bool bv = b < n;")
-            E("const u64 bc = bv ? b : n - 1;")
-            E(f"const T* __restrict__ Xr = X + bc * {self.D1};")
-            E(f"const T* __restrict__ Gr = G + bc * {self.D3};")
-            for f in ys:
-                E(f"const T y{f} = bv ? Y[bc * {self.D2} + {f}] : (T)0;     // zero rows past the end: T = 0 there")
-            for ai in ins:
-                a_ = self.in1[ai]
-                for q in range(_ceil(_ceil(a_.mul, 16), 4)):
-                    uexp = f"16 * (wave + {4 * q}) + c"
-                    ucl = uexp if a_.mul % 64 == 0 else f"min({uexp}, {a_.mul - 1})"
-                    E(f"const T* __restrict__ xp{ai}_{q} = Xr + {a_.off} + ({ucl}) * {a_.D};")
-                    if a_.mul % 64 == 0:
-                        E("const T " + ", ".join(f"x{ai}_{q}_{i} = xp{ai}_{q}[{i}]" for i in range(a_.D)) + ";")
-                    else:
-                        E("T " + ", ".join(f"x{ai}_{q}_{i} = xp{ai}_{q}[{i}]" for i in range(a_.D)) + ";")
-                        E(f"if ({uexp} >= {a_.mul}) {{ " + " ".join(f"x{ai}_{q}_{i} = (T)0;" for i in range(a_.D)) + " }")
-            for oi in outs:
-                o = self.out[oi]
-                NT = _ceil(o.mul, 16)
-                E(f"{{ // output block {oi}: dZ records, w = 16 nt + c")
+            if self.dw_prefetch:
+                # One step = 4 batch rows (the K of one MFMA) of one tile.  The steps of all tiles of this
+                # workgroup form one loop, software pipelined over two register sets when the registers
+                # allow it: the operands of the next step are in flight while this one is computed (X and
+                # dZ stream from HBM here, so the latency to cover is the long one).
+                names = [f"y{f}" for f in ys]
+                for ai in ins:
+                    a_ = self.in1[ai]
+                    names += [f"x{ai}_{q}_{i}" for q in range(_ceil(_ceil(a_.mul, 16), 4)) for i in range(a_.D)]
+                for oi in outs:
+                    o = self.out[oi]
+                    names += [f"gz{oi}_{nt}_{k}" for nt in range(_ceil(o.mul, 16)) for k in range(o.D)]
+
+                def load(E, it, h, ys=ys, ins=ins, outs=outs):
+                    E("{")
+                    E.level += 1
+                    E(f"const u64 b = (blockIdx.x + (u64)(({it}) >> 2) * gridDim.x) * 16 + 4 * (({it}) & 3) + g;   // batch row of this lane for both operands")
+                    E("const bool bv = b < n;")
+                    E("const u64 bc = bv ? b : n - 1;")
+                    E(f"const T* __restrict__ Xr = X + bc * {self.D1};")
+                    E(f"const T* __restrict__ Gr = G + bc * {self.D3};")
+                    for f in ys:
+                        E(f"S{h}y{f} = Y[bc * {self.D2} + {f}];")
+                    E("if (!bv) { " + " ".join(f"S{h}y{f} = (T)0;" for f in ys) + " }     // rows past the end: T = 0 there")
+                    for ai in ins:
+                        a_ = self.in1[ai]
+                        for q in range(_ceil(_ceil(a_.mul, 16), 4)):
+                            uexp = f"16 * (wave + {4 * q}) + c"
+                            ucl = uexp if a_.mul % 64 == 0 else f"min({uexp}, {a_.mul - 1})"
+                            E(f"{{ const T* __restrict__ xp = Xr + {a_.off} + ({ucl}) * {a_.D}; "
+                              + " ".join(f"S{h}x{ai}_{q}_{i} = xp[{i}];" for i in range(a_.D)) + " }")
+                            if a_.mul % 64 != 0:
+                                E(f"if ({uexp} >= {a_.mul}) {{ " + " ".join(f"S{h}x{ai}_{q}_{i} = (T)0;" for i in range(a_.D)) + " }")
+                    for oi in outs:
+                        o = self.out[oi]
+                        for nt in range(_ceil(o.mul, 16)):
+                            wexp = f"{16 * nt} + c"
+                            wcl = wexp if o.mul % 16 == 0 else f"min({wexp}, {o.mul - 1})"
+                            E(f"{{ const T* __restrict__ gp = Gr + {o.off} + ({wcl}) * {o.D}; "
+                              + " ".join(f"S{h}gz{oi}_{nt}_{k} = gp[{k}];" for k in range(o.D)) + " }")
+                    E.level -= 1
+                    E("}")
+
+                def compute(E, outs=outs):
+                    for oi in outs:
+                        o = self.out[oi]
+                        NT = _ceil(o.mul, 16)
+                        for p in self.paths_into(oi):
+                            for q in range(_ceil(p.NTU, 4)):
+                                E(f"if (wave + {4 * q} < {p.NTU}) {{  // path {p.t}")
+                                E.level += 1
+                                self.emit_cg_forward(E, p, f"x{p.a.idx}_{q}_", "y", "t")
+                                for nt in range(NT):
+                                    for k in range(o.D):
+                                        E(f"acc{p.t}_{q}_{nt} = oeq_mfma(t{k}, gz{oi}_{nt}_{k}, acc{p.t}_{q}_{nt});")
+                                E.level -= 1
+                                E("}")
+
+                E("const int nsteps = blockIdx.x < ntiles ? 4 * (int)((ntiles - blockIdx.x + gridDim.x - 1) / gridDim.x) : 0;")
+                nsets = 2
+                for h in range(nsets):
+                    E("T " + ", ".join(f"S{h}{nm} = (T)0" for nm in names) + ";")
+                E("if (nsteps > 0) {")
                 E.level += 1
-                for nt in range(NT):
-                    wexp = f"{16 * nt} + c"
-                    wcl = wexp if o.mul % 16 == 0 else f"min({wexp}, {o.mul - 1})"
-                    E(f"const T* __restrict__ gp{nt} = Gr + {o.off} + ({wcl}) * {o.D};")
-                    E("const T " + ", ".join(f"gz{nt}_{k} = gp{nt}[{k}]" for k in range(o.D)) + ";")
-                for p in self.paths_into(oi):
-                    for q in range(_ceil(p.NTU, 4)):
-                        E(f"if (wave + {4 * q} < {p.NTU}) {{  // path {p.t}")
-                        E.level += 1
-                        self.emit_cg_forward(E, p, f"x{p.a.idx}_{q}_", "y", "t")
-                        for nt in range(NT):
-                            for k in range(o.D):
-                                E(f"acc{p.t}_{q}_{nt} = oeq_mfma(t{k}, gz{nt}_{k}, acc{p.t}_{q}_{nt});")
-                        E.level -= 1
-                        E("}")
+                load(E, "0", 0)
                 E.level -= 1
                 E("}")
-            E.level -= 1
-            E("}")
-            E.level -= 1
-            E("}")
+                if nsets == 1:
+                    E("#pragma unroll 1")
+                    E("for (int it = 0; it < nsteps; ++it) {")
+                    E.level += 1
+                    E("const T " + ", ".join(f"{nm} = S0{nm}" for nm in names) + ";")
+                    compute(E)
+                    E("if (it + 1 < nsteps) {")
+                    E.level += 1
+                    load(E, "it + 1", 0)
+                    E.level -= 1
+                    E("}")
+                    E.level -= 1
+                    E("}")
+                else:
+                    E("#pragma unroll 1")
+                    E("for (int it = 0; it < nsteps; it += 2) {")     # nsteps is a multiple of 4
+                    E.level += 1
+                    for h in (0, 1):
+                        E("{")
+                        E.level += 1
+                        E("const T " + ", ".join(f"{nm} = S{h}{nm}" for nm in names) + ";")
+                        E(f"if (it + {h + 1} < nsteps) {{")
+                        E.level += 1
+                        load(E, f"it + {h + 1}", 1 - h)
+                        E.level -= 1
+                        E("}")
+                        compute(E)
+                        E.level -= 1
+                        E("}")
+                    E.level -= 1
+                    E("}")
+            else:
+                E("for (u64 tile = blockIdx.x; tile < ntiles; tile += gridDim.x) {")
+                E.level += 1
+                E("const u64 row0 = tile * 16;")
+                E("#pragma unroll 1")
+                E("for (int sp = 0; sp < 4; ++sp) {")
+                E.level += 1
+                E("const u64 b = row0 + 4 * sp + g;          // batch row of this lane for both operands")
+                E("const bool bv = b < n;")
+                E("const u64 bc = bv ? b : n - 1;")
+                E(f"const T* __restrict__ Xr = X + bc * {self.D1};")
+                E(f"const T* __restrict__ Gr = G + bc * {self.D3};")
+                for f in ys:
+                    E(f"const T y{f} = bv ? Y[bc * {self.D2} + {f}] : (T)0;     // zero rows past the end: T = 0 there")
+                for ai in ins:
+                    a_ = self.in1[ai]
+                    for q in range(_ceil(_ceil(a_.mul, 16), 4)):
+                        uexp = f"16 * (wave + {4 * q}) + c"
+                        ucl = uexp if a_.mul % 64 == 0 else f"min({uexp}, {a_.mul - 1})"
+                        E(f"const T* __restrict__ xp{ai}_{q} = Xr + {a_.off} + ({ucl}) * {a_.D};")
+                        if a_.mul % 64 == 0:
+                            E("const T " + ", ".join(f"x{ai}_{q}_{i} = xp{ai}_{q}[{i}]" for i in range(a_.D)) + ";")
+                        else:
+                            E("T " + ", ".join(f"x{ai}_{q}_{i} = xp{ai}_{q}[{i}]" for i in range(a_.D)) + ";")
+                            E(f"if ({uexp} >= {a_.mul}) {{ " + " ".join(f"x{ai}_{q}_{i} = (T)0;" for i in range(a_.D)) + " }")
+                for oi in outs:
+                    o = self.out[oi]
+                    NT = _ceil(o.mul, 16)
+                    E(f"{{ // output block {oi}: dZ records, w = 16 nt + c")
+                    E.level += 1
+                    for nt in range(NT):
+                        wexp = f"{16 * nt} + c"
+                        wcl = wexp if o.mul % 16 == 0 else f"min({wexp}, {o.mul - 1})"
+                        E(f"const T* __restrict__ gp{nt} = Gr + {o.off} + ({wcl}) * {o.D};")
+                        E("const T " + ", ".join(f"gz{nt}_{k} = gp{nt}[{k}]" for k in range(o.D)) + ";")
+                    for p in self.paths_into(oi):
+                        for q in range(_ceil(p.NTU, 4)):
+                            E(f"if (wave + {4 * q} < {p.NTU}) {{  // path {p.t}")
+                            E.level += 1
+                            self.emit_cg_forward(E, p, f"x{p.a.idx}_{q}_", "y", "t")
+                            for nt in range(NT):
+                                for k in range(o.D):
+                                    E(f"acc{p.t}_{q}_{nt} = oeq_mfma(t{k}, gz{nt}_{k}, acc{p.t}_{q}_{nt});")
+                            E.level -= 1
+                            E("}")
+                    E.level -= 1
+                    E("}")
+                E.level -= 1
+                E("}")
+                E.level -= 1
+                E("}")
             # ---- partial sums of this workgroup, laid out [t][u][w]
             for p in paths:
                 for q in range(_ceil(p.NTU, 4)):

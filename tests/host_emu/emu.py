@@ -58,7 +58,7 @@ static inline T oeq_shfl_xor(T v, int mask) { g_xT[threadIdx.x] = v; oeq_sync();
 static inline int oeq_shfl_i32(int v, int src) { g_xi[threadIdx.x] = v; oeq_sync(); int r = g_xi[src & 63]; oeq_sync(); return r; }
 static inline int oeq_shfl_xor_i32(int v, int mask) { g_xi[threadIdx.x] = v; oeq_sync(); int r = g_xi[threadIdx.x ^ mask]; oeq_sync(); return r; }
 #define __builtin_amdgcn_readfirstlane(x) oeq_shfl_i32((x), 0)
-struct VT { T v[16 / sizeof(T)]; };
+struct VT { T v[16 / sizeof(T)]; T& operator[](int i) { return v[i]; } const T& operator[](int i) const { return v[i]; } };
 static inline void oeq_dma16(const T* g, T* lds_base) { memcpy((char*)lds_base + 16 * threadIdx.x, g, 16); }
 static inline void oeq_wait_vm() {}
 static inline void oeq_wait_lds() {}
