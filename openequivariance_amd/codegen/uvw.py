@@ -65,8 +65,8 @@ class WPath:
         return self.o.mul
 
     @property
-    def SU(self) -> int:            # K steps over u (forward)
-        return _ceil(self.mu, 4)
+    def SU(self) -> int:            # K steps over u (forward): whole blocks of 16 channels, 4 steps each
+        return 4 * _ceil(self.mu, 16)
 
     @property
     def SW(self) -> int:            # K steps over w (backward dX)
@@ -104,6 +104,7 @@ class UVWGenerator:
         # backward dX/dY: register sets for the packed weight fragments (2 = fetched one item ahead)
         self.bwd_a_sets = int(os.environ.get("OEQ_AMD_UVW_ASETS", "1"))
         self._bwd_lds_env = os.environ.get("OEQ_AMD_UVW_BWD_LDS", "1") == "1"
+        self.fwd_xcd_map = os.environ.get("OEQ_AMD_UVW_FWD_XCD", "1") == "1"
         # backward dW: fetch the operands of the next step while the current one runs (two register sets)
         self.dw_prefetch = os.environ.get("OEQ_AMD_UVW_DW_PREFETCH", "1" if self.T == "float" else "0") == "1"
         self.in1, self.in2, self.out = _blocks(problem.irreps_in1), _blocks(problem.irreps_in2), _blocks(problem.irreps_out)
@@ -245,7 +246,7 @@ class UVWGenerator:
             E(f"if (q >= {p.wb} && q < {p.wb + nb}) {{   // forward copy of path {p.t}: [s][lane][nt]")
             E(f"    const int e = q - {p.wb};")
             E(f"    const int nt = e % {p.NTW}; const int ln = (e / {p.NTW}) & 63; const int s = e / {64 * p.NTW};")
-            E(f"    const int u = 4 * s + (ln >> 4); const int w = {p.NTW} * (ln & 15) + nt;")
+            E(f"    const int u = 16 * (s >> 2) + 4 * (ln >> 4) + (s & 3); const int w = {p.NTW} * (ln & 15) + nt;   // K order of forward_body")
             E(f"    wsT[q] = (u < {p.mu} && w < {p.mw}) ? W[{self.oeq_index(p, 'u', 'w')}] : (T)0;")
             E("}")
             VW, SQ = self.VW, _ceil(p.SW, self.VW)
@@ -265,8 +266,22 @@ class UVWGenerator:
     # =============================================================== forward
     def forward_body(self) -> str:
         E = Emitter()
+        NO = len(self.fwd_order)
         E("const int lane = threadIdx.x, c = lane & 15, g = lane >> 4;")
-        E("const u64 row0 = (u64)blockIdx.x * 16;")
+        if self.fwd_xcd_map:
+            # Work item = (batch tile, output block).  Workgroups are handed to the 8 XCDs round robin by
+            # their linear id, and every XCD has an L2 of its own: the items of one tile get ids 8 apart,
+            # i.e. consecutive turns of the same XCD, so that the X rows fetched for the first output
+            # block are still in that L2 for the others.  The tiles beyond the last multiple of 8 are
+            # mapped plainly.
+            E("const u64 ntiles = gridDim.x, lin = blockIdx.x + (u64)blockIdx.y * gridDim.x;")
+            E(f"const u64 full = (ntiles >> 3) * {8 * NO};")
+            E("u64 tile; int slot;")
+            E(f"if (lin < full) {{ const u64 j = lin >> 3; slot = (int)(j % {NO}); tile = (j / {NO}) * 8 + (lin & 7); }}")
+            E("else { const u64 rem = ntiles & 7, l2 = lin - full; slot = (int)(l2 / rem); tile = (ntiles & ~(u64)7) + l2 % rem; }")
+        else:
+            E("const u64 tile = blockIdx.x; const int slot = blockIdx.y;")
+        E("const u64 row0 = tile * 16;")
         E("if (row0 >= n) return;")
         E("const u64 rowA = min(row0 + (u64)c, n - 1);       // rows past the end repeat the last row, never stored")
         E("const T* __restrict__ wsT = (const T*)ws;")
@@ -278,7 +293,7 @@ class UVWGenerator:
         # (whole tiles per wavefront leave a third of the machine idle in the last round).
         for slot, o in enumerate(self.fwd_order):
             NT = _ceil(o.mul, 16)
-            E(f"if (blockIdx.y == {slot}) {{ // output block {o.idx}: {o.mul}x l={o.l}")
+            E(f"if (slot == {slot}) {{ // output block {o.idx}: {o.mul}x l={o.l}")
             E.level += 1
             if o.idx not in self.used_out:
                 for r in range(4):
@@ -307,8 +322,10 @@ class UVWGenerator:
                         sexp = f"({gexp}) * {GS} + {j}"
                         need_clamp = (NG * GS != p.SU)
                         scl = f"min({sexp}, {p.SU - 1})" if need_clamp else sexp
-                        uexp = f"4 * ({sexp}) + g"
-                        ucl = uexp if (p.mu % 4 == 0 and not need_clamp) else f"min({uexp}, {p.mu - 1})"
+                        # K index -> channel: step s of lane group g is u = 16 (s / 4) + 4 g + s % 4, so that the
+                        # four steps of a group read four adjacent records of a row (one wide load per lane)
+                        uexp = f"16 * (({sexp}) >> 2) + 4 * g + (({sexp}) & 3)"
+                        ucl = uexp if (p.mu % 16 == 0 and not need_clamp) else f"min({uexp}, {p.mu - 1})"
                         E(f"{{ const T* __restrict__ xp = Xr + {p.a.off} + ({ucl}) * {p.a.D}; " + " ".join(f"nx{j}_{i} = xp[{i}];" for i in range(p.a.D)))
                         E(f"  const T* __restrict__ bp = wsT + {p.wb} + (({scl}) * 64 + lane) * {NT}; " + " ".join(f"nb{j}_{nt} = bp[{nt}];" for nt in range(NT)) + " }")
                 load(E, "0")
@@ -326,8 +343,8 @@ class UVWGenerator:
                     E.level += 1
                     E("const T " + ", ".join(f"x{i} = cnx{j}_{i}" for i in range(p.a.D)) + ";")
                     self.emit_cg_forward(E, p, "x", "y", "t")
-                    if p.mu % 4 != 0 or NG * GS != p.SU:
-                        E(f"if (4 * (sg * {GS} + {j}) + g >= {p.mu}) {{ " + " ".join(f"t{k} = (T)0;" for k in range(o.D)) + " }")
+                    if p.mu % 16 != 0 or NG * GS != p.SU:
+                        E(f"if (16 * ((sg * {GS} + {j}) >> 2) + 4 * g + ((sg * {GS} + {j}) & 3) >= {p.mu}) {{ " + " ".join(f"t{k} = (T)0;" for k in range(o.D)) + " }")
                     for k in range(o.D):
                         for nt in range(NT):
                             E(f"acc{k}_{nt} = oeq_mfma(t{k}, cnb{j}_{nt}, acc{k}_{nt});")
