@@ -1,12 +1,13 @@
 """Generator of gfx950 HIP source for channel-wise ("uvu") tensor products.
 
-One generator serves three operator families that share the per-row arithmetic:
-
-* ``tp``          - batch tensor product (forward; backward -> dX, dY, dW)
-* ``conv_atomic`` - fused gather/product/scatter over unsorted edges, scatter by atomics
-* ``conv_det``    - deterministic fused convolution over receiver-sorted edges: one
-                    wavefront owns a node (and a 64-channel chunk) and walks its edge list,
-                    so sums are formed in a fixed order without atomics
+This class holds what every uvu kernel shares - the lane mapping, the unrolled Clebsch-Gordan
+arithmetic of one output block (forward and backward), the weight indexing and the launch plans -
+and generates the LDS-staged batch product itself, which is the schedule used for *shared* weights
+(persistent wavefronts and an ordered dW reduction).  The kernels for per-row weights and for the
+convolutions derive from it: ``uvu_direct.py`` (register-direct loads), ``uvu_det.py`` (one node per
+wavefront), ``uvu_sorted.py`` (on-the-fly grouping by receiver).  ``kind`` names the operator family
+a subclass generates for: ``tp``, ``conv_atomic`` (per-edge kernels, scatter by atomics) or
+``conv_det`` (segmented, no atomics).
 
 Mapping to the hardware (the arithmetic follows the reference's kernels,
 openequivariance/templates/loop_unroll_tp.cuh:20-97 forward and :107-252 backward, but the
@@ -97,6 +98,8 @@ class UVUGenerator:
     def __init__(self, problem: TPProblem, kind: str = "tp", dw_partials: int = 1024):
         if kind not in ("tp", "conv_atomic", "conv_det"):
             raise ValueError(kind)
+        if type(self) is UVUGenerator and kind != "tp":
+            raise NotImplementedError("the convolution kernels come from uvu_direct / uvu_det / uvu_sorted")
         self.problem, self.kind = problem, kind
         self.T = {np.float32: "float", np.float64: "double"}[problem.irrep_dtype]
         self.itemsize = 4 if self.T == "float" else 8
@@ -612,260 +615,12 @@ class UVUGenerator:
                         E(f"  if (sub == 0 && u < {p.mu}) part[{self.widx(p, 'u', v)}] = dws{p.t}_{c}_{v}; }}")
         return E.text()
 
-    # =========================================================== atomic convolution
-    def _edge_prologue(self, E: Emitter, need_recv_rows: bool = True) -> None:
-        """Edge-parallel kernels: sub-row r handles edge e0 + r."""
-        R = self.R
-        E(f"const u64 e0 = (u64)blockIdx.x * {R};")
-        E("const u64 e = e0 + sub;")
-        E("i64 snd = -1, rcv = -1;")
-        E("if (e < nnz) { snd = cols[e]; rcv = rows[e]; }")
-        E("const bool rv = (snd >= 0 && snd < (i64)node_count && rcv >= 0 && rcv < (i64)node_count);")
-        E("const int xsrc = rv ? (int)snd : -1;")
-        E("const int zdst = rv ? (int)rcv : -1;")
-        if R == 1:
-            E("const int xsrc_u = __builtin_amdgcn_readfirstlane(xsrc);")
-            E("const int zdst_u = __builtin_amdgcn_readfirstlane(zdst);")
-        E(f"const T* __restrict__ Yr = Y + e * {self.D2};")
-        E(f"const T* __restrict__ Wr = W + e * {self.WN};")
-
+    # ------------------------------------------------ row indices shared inside a wavefront
     def _shfl_row(self, var: str):
         if self.R == 1:
             return lambda r: (f"{var}_u", f"({var}_u >= 0)")
         return lambda r: (f"oeq_shfl_i32({var}, ({r}) << {self.LOGP})", f"(oeq_shfl_i32({var}, ({r}) << {self.LOGP}) >= 0)")
 
-    def conv_atomic_forward_body(self) -> str:
-        E = Emitter()
-        self.emit_lane(E)
-        self._edge_prologue(E)
-        self.emit_y_load(E, "Yr", "rv")
-        self.emit_x_stage(E)
-        E("oeq_sync();")
-        own = ("zdst", "rv")
-        row_of = self._shfl_row("zdst")
-
-        def body(E):
-            self.emit_x_regs(E)
-            for oi in self.used_out:
-                o = self.out[oi]
-                E("{")
-                E.level += 1
-                self.emit_forward_block(E, o, "Wr")
-                self.emit_block_out(E, o, "z", "Z", self.D3, own, row_of, op="atomic")
-                E.level -= 1
-                E("}")
-        self.chunk_loop(E, body)
-        return E.text()
-
-    def conv_atomic_backward_body(self) -> str:
-        E = Emitter()
-        self.emit_lane(E)
-        self._edge_prologue(E)
-        E(f"T* __restrict__ Wgr = Wg + e * {self.WN};")
-        self.emit_y_load(E, "Yr", "rv")
-        for f in self.used_y:
-            E(f"T dy{f} = (T)0;")
-        self.emit_x_stage(E)
-        E("oeq_sync();")
-        own_z = ("zdst", "rv")
-        own_x = ("xsrc", "rv")
-        zrow_of = self._shfl_row("zdst")
-        xrow_of = self._shfl_row("xsrc")
-
-        def body(E):
-            self.emit_x_regs(E)
-            for i in self.used_in1:
-                for m in range(self.in1[i].D):
-                    E(f"T dx{i}_{m} = (T)0;")
-            for oi in self.used_out:
-                o = self.out[oi]
-                E("{")
-                E.level += 1
-                self.emit_block_in(E, o, "g", "G", self.D3, own_z, zrow_of)
-
-                def sink(E, p, v, expr):
-                    E(f"  if ({self.act(p.a)}) Wgr[{self.widx(p, 'u', v)}] = {expr};")
-                self.emit_backward_block(E, o, "Wr", sink)
-                E.level -= 1
-                E("}")
-            for i in self.used_in1:
-                a = self.in1[i]
-                E("{")
-                E.level += 1
-                self.emit_block_out(E, a, f"dx{a.idx}_", "Xg", self.D1, own_x, xrow_of, op="atomic")
-                E.level -= 1
-                E("}")
-        self.chunk_loop(E, body)
-        self.emit_dy_reduce(E)
-        E("if (e < nnz && ul == 0) {")
-        E(f"    T* __restrict__ Ygr = Yg + e * {self.D2};")
-        for f in range(self.D2):
-            E(f"    Ygr[{f}] = " + (f"dy{f};" if f in self.used_y else "(T)0;"))
-        E("}")
-        # weights of idle lanes / invalid edges: dW rows must still be defined
-        E("if (e < nnz && !rv) {")
-        E(f"    for (int q = ul; q < {self.WN}; q += {self.P}) Wgr[q] = (T)0;")
-        E("}")
-        return E.text()
-
-    # ==================================================== deterministic convolution
-    def _node_prologue(self, E: Emitter, ptr_name: str) -> None:
-        """Node-parallel kernels: sub-row r owns node node0 + r and the edge positions
-        [ptr[node], ptr[node+1]) of the sorted edge list."""
-        R = self.R
-        E(f"const u64 node0 = (u64)blockIdx.x * {R};")
-        E("const u64 node = node0 + sub;")
-        E("const bool nv = node < node_count;")
-        E(f"const i64* __restrict__ ptr = (const i64*)ws + {ptr_name};")
-        E("i64 beg = 0, end = 0;")
-        E("if (nv && nnz > 0) { beg = ptr[node]; end = ptr[node + 1]; }")
-        E("if (beg < 0) beg = 0;")
-        E("if (end > (i64)nnz) end = (i64)nnz;")
-        E("if (end < beg) end = beg;")
-        E("int len = (int)(end - beg);")
-        E("int maxlen = len;")
-        m = 32
-        while m >= self.P:
-            E(f"maxlen = max(maxlen, oeq_shfl_xor_i32(maxlen, {m}));")
-            m //= 2
-        if R == 1:
-            E("maxlen = __builtin_amdgcn_readfirstlane(maxlen);")
-
-    def conv_det_forward_body(self) -> str:
-        """Z[node] = sum over the node's incoming edges, in edge order."""
-        E = Emitter()
-        self.emit_lane(E)
-        self._node_prologue(E, "0")
-        own_z = ("node", "nv")
-        zrow_of = lambda r: (f"(node0 + {r})", f"(node0 + {r} < node_count)")
-
-        def body(E):
-            for oi in self.used_out:
-                for k in range(self.out[oi].D):
-                    E(f"T z{oi}_{k} = (T)0;")
-            E("for (int it = 0; it < maxlen; ++it) {")
-            E.level += 1
-            E("const bool ev = it < len;")
-            E("const u64 e = (u64)(beg + it);")
-            E("i64 snd = -1;")
-            E("if (ev) snd = cols[e];")
-            E("const bool rv = ev && snd >= 0 && snd < (i64)node_count;")
-            E("const int xsrc = rv ? (int)snd : -1;")
-            if self.R == 1:
-                E("const int xsrc_u = __builtin_amdgcn_readfirstlane(xsrc);")
-            E(f"const T* __restrict__ Yr = Y + e * {self.D2};")
-            E(f"const T* __restrict__ Wr = W + e * {self.WN};")
-            self.emit_y_load(E, "Yr", "rv")
-            E("oeq_sync();")
-            self.emit_x_stage(E)
-            E("oeq_sync();")
-            self.emit_x_regs(E)
-            for oi in self.used_out:
-                self.emit_forward_block(E, self.out[oi], "Wr", zname=f"z{oi}_", declare=False)
-            E.level -= 1
-            E("}")
-            E("const bool rv = nv;")
-            for o in self.out:
-                if o.dim == 0:
-                    continue
-                E("{")
-                E.level += 1
-                if o.idx in self.used_out:
-                    self.emit_block_out(E, o, f"z{o.idx}_", "Z", self.D3, own_z, zrow_of)
-                else:
-                    if o.D > 1:
-                        E("oeq_sync();")
-                    self.emit_block_zero(E, o, "Z", self.D3, own_z, zrow_of)
-                E.level -= 1
-                E("}")
-        self.chunk_loop(E, body)
-        return E.text()
-
-    def conv_det_backward_body(self) -> str:
-        """dX[node] = sum over the node's outgoing edges (walked in sender-sorted order through
-        the transpose permutation); dW[e] chunk and dY[e] (partial per chunk) written per edge."""
-        E = Emitter()
-        self.emit_lane(E)
-        self._node_prologue(E, "PTR_STRIDE")
-        own_x = ("node", "nv")
-        xrow_of = lambda r: (f"(node0 + {r})", f"(node0 + {r} < node_count)")
-
-        def body(E):
-            # this node's own X chunk is staged once
-            E("{")
-            E("    const bool rv = nv;")
-            E("    const int xsrc = nv ? (int)node : -1;")
-            if self.R == 1:
-                E("    const int xsrc_u = __builtin_amdgcn_readfirstlane(xsrc);")
-            E.level += 1
-            self.emit_x_stage(E)
-            E.level -= 1
-            E("}")
-            E("oeq_sync();")
-            E("bool rv = nv;")
-            self.emit_x_regs(E)
-            for i in self.used_in1:
-                for m in range(self.in1[i].D):
-                    E(f"T dx{i}_{m} = (T)0;")
-            E("for (int it = 0; it < maxlen; ++it) {")
-            E.level += 1
-            E("const bool ev = it < len;")
-            E("i64 e = -1, rcv = -1;")
-            E("if (ev) { e = tperm[beg + it]; }")
-            E("if (e >= 0 && e < (i64)nnz) rcv = rows[e];")
-            E("rv = ev && rcv >= 0 && rcv < (i64)node_count;")
-            E("const int zdst = rv ? (int)rcv : -1;")
-            if self.R == 1:
-                E("const int zdst_u = __builtin_amdgcn_readfirstlane(zdst);")
-            E("const u64 eu = rv ? (u64)e : 0;")
-            E(f"const T* __restrict__ Yr = Y + eu * {self.D2};")
-            E(f"const T* __restrict__ Wr = W + eu * {self.WN};")
-            E(f"T* __restrict__ Wgr = Wg + eu * {self.WN};")
-            self.emit_y_load(E, "Yr", "rv")
-            for f in self.used_y:
-                E(f"T dy{f} = (T)0;")
-            own_z = ("zdst", "rv")
-            zrow_of = self._shfl_row("zdst")
-            for oi in self.used_out:
-                o = self.out[oi]
-                E("{")
-                E.level += 1
-                self.emit_block_in(E, o, "g", "G", self.D3, own_z, zrow_of)
-
-                def sink(E, p, v, expr):
-                    E(f"  if ({self.act(p.a)}) Wgr[{self.widx(p, 'u', v)}] = {expr};")
-                self.emit_backward_block(E, o, "Wr", sink)
-                E.level -= 1
-                E("}")
-            self.emit_dy_reduce(E)
-            E("if (rv && ul == 0) {")
-            if self.NCH > 1:
-                E(f"    T* __restrict__ Ygr = (T*)((char*)ws + DYPART_OFF) + ((u64)c * nnz + eu) * {self.D2};")
-            else:
-                E(f"    T* __restrict__ Ygr = Yg + eu * {self.D2};")
-            for f in range(self.D2):
-                E(f"    Ygr[{f}] = " + (f"dy{f};" if f in self.used_y else "(T)0;"))
-            E("}")
-            E.level -= 1
-            E("}")
-            E("rv = nv;")
-            for a in self.in1:
-                if a.dim == 0:
-                    continue
-                E("{")
-                E.level += 1
-                if a.idx in self.used_in1:
-                    self.emit_block_out(E, a, f"dx{a.idx}_", "Xg", self.D1, own_x, xrow_of)
-                else:
-                    if a.D > 1:
-                        E("oeq_sync();")
-                    self.emit_block_zero(E, a, "Xg", self.D1, own_x, xrow_of)
-                E.level -= 1
-                E("}")
-        self.chunk_loop(E, body)
-        return E.text()
-
-    # ---------------------------------------------------------------- rendering
     def render(self, prelude: str = None) -> str:
         env = jinja_env()
         if prelude is None:

@@ -28,8 +28,8 @@ def test_validation_mirrors_reference_constraints():
     with pytest.raises(AssertionError):
         validate_problem(oeq.TPProblem("2x0e", "1x0e", "2x0e", [(0, 0, 0, "uvu", True)], irrep_dtype=np.float64))
     with pytest.raises(AssertionError):                      # conv needs mul 1 on the second operand
-        UVUGenerator(oeq.TPProblem("2x0e", "2x0e", "2x0e", [(0, 0, 0, "uvu", True)], shared_weights=False,
-                                   internal_weights=False), "conv_atomic")
+        UVUDirectGenerator(oeq.TPProblem("2x0e", "2x0e", "2x0e", [(0, 0, 0, "uvu", True)], shared_weights=False,
+                                         internal_weights=False), "conv_atomic")
 
 
 def test_launch_plans():
