@@ -32,6 +32,8 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Dict, List, Tuple
 
+import os
+
 import numpy as np
 
 from ..problem import TPProblem
@@ -163,6 +165,14 @@ class UVWGenerator:
         self.ws_elems = self.PART_OFF + self.DW_WORKGROUPS * self.WN
 
     # ------------------------------------------------------------------ helpers
+    def backward_attr(self) -> str:
+        """Occupancy target of the dX/dY kernel: as many workgroups per CU (one wavefront per SIMD
+        each) as the LDS tile allows; the register allocator then stays within that budget."""
+        if not self.bwd_lds or os.environ.get("OEQ_AMD_UVW_BWD_OCC", "1") != "1":
+            return ""
+        per_cu = max(1, min(4, (160 * 1024) // (16 * self.bwd_rs * self.itemsize + 4 * 16 * max(1, self.D2) * self.itemsize)))
+        return f" __attribute__((amdgpu_waves_per_eu({per_cu}, {per_cu})))" if per_cu >= 3 else ""
+
     def _pick_row_stride(self) -> int:
         """Row stride (elements) of the dZ tile in LDS: the smallest padding for which the 32 lanes of
         one LDS pass (16 rows x 2 adjacent records) spread best over the 32 four-byte banks."""
@@ -411,21 +421,50 @@ class UVWGenerator:
             E(f"const T y{f} = Y[rowB * {self.D2} + {f}];")
             E(f"T dy{f} = (T)0;")
         # X records and dX accumulators of this wavefront: u-subtiles mt = wave + 4q, rows r of the
-        # accumulator tile.  X is read once here for all paths that consume the block.
+        # accumulator tile.  X is read once for all paths that consume the block.  With the dZ tile in
+        # LDS the work is ordered by in1 block, so only one block's X and dX are live at a time (plus the
+        # next block's X, requested one block ahead); otherwise everything is loaded here.
         for ai in self.used_in1:
             a = self.in1[ai]
             for q in range(_ceil(_ceil(a.mul, 16), 4)):
                 for r in range(4):
-                    uexp = f"16 * (wave + {4 * q}) + {self.row(r)}"
-                    E(f"const T* __restrict__ xp{ai}_{q}_{r} = Xr + {a.off} + min({uexp}, {a.mul - 1}) * {a.D};")
-                    E("const T " + ", ".join(f"x{ai}_{q}_{r}_{i} = xp{ai}_{q}_{r}[{i}]" for i in range(a.D)) + ";")
+                    E("T " + ", ".join(f"x{ai}_{q}_{r}_{i}" for i in range(a.D)) + ";")
                     E("T " + ", ".join(f"dx{ai}_{q}_{r}_{i} = (T)0" for i in range(a.D)) + ";")
+
+        def load_x(E, ai):
+            a = self.in1[ai]
+            for q in range(_ceil(_ceil(a.mul, 16), 4)):
+                for r in range(4):
+                    uexp = f"16 * (wave + {4 * q}) + {self.row(r)}"
+                    E(f"{{ const T* __restrict__ xp = Xr + {a.off} + min({uexp}, {a.mul - 1}) * {a.D}; "
+                      + " ".join(f"x{ai}_{q}_{r}_{i} = xp[{i}];" for i in range(a.D)) + " }")
+
+        def store_dx(E, ai):
+            a = self.in1[ai]
+            for q in range(_ceil(_ceil(a.mul, 16), 4)):
+                E(f"if (wave + {4 * q} < {_ceil(a.mul, 16)} && bvalid) {{")
+                E(f"    const int mt = wave + {4 * q};")
+                for r in range(4):
+                    E(f"    {{ const int u = 16 * mt + {self.row(r)};")
+                    guard = "" if a.mul % 16 == 0 else f"if (u < {a.mul}) "
+                    E(f"      {guard}{{ T* __restrict__ xp = Xg + (row0 + c) * {self.D1} + {a.off} + u * {a.D}; "
+                      + " ".join(f"xp[{i}] = dx{a.idx}_{q}_{r}_{i};" for i in range(a.D)) + " } }")
+                E("}")
+        by_in1 = self.bwd_lds
+        if by_in1:
+            load_x(E, self.used_in1[0])
+        else:
+            for ai in self.used_in1:
+                load_x(E, ai)
         # Work list of this wavefront: (output block, path, u-subtile group).  The packed weight
         # fragments (MFMA A operand) of the next item are fetched into a second register set while
         # the current item runs, and the dZ records of the next output block are requested as soon
         # as the last matrix-core step of the current one is issued, so that neither L2 nor HBM
         # latency sits between two items.
-        items = [(oi, p, q) for oi in self.used_out for p in self.paths_into(oi) for q in range(_ceil(p.NTU, 4))]
+        if by_in1:
+            items = [(p.o.idx, p, q) for ai in self.used_in1 for p in self.paths_from(ai) for q in range(_ceil(p.NTU, 4))]
+        else:
+            items = [(oi, p, q) for oi in self.used_out for p in self.paths_into(oi) for q in range(_ceil(p.NTU, 4))]
         max_sw = max(_ceil(self.out[oi].mul, 4) for oi in self.used_out)
         NSETS = self.bwd_a_sets
         E("T " + ", ".join(f"af{b_}_{s_}" for b_ in range(NSETS) for s_ in range(max_sw)) + ";")
@@ -466,6 +505,10 @@ class UVWGenerator:
             # sinking the vector-ALU halves of all items below the matrix-core work, which would keep
             # every accumulator alive and halve the occupancy.
             cond = f"wave + {4 * q} < {p.NTU}"
+            if by_in1 and (j == 0 or items[j - 1][1].a.idx != a.idx):
+                nxt = self.used_in1.index(a.idx) + 1
+                if nxt < len(self.used_in1):
+                    load_x(E, self.used_in1[nxt])
             if j + 1 < len(items) and NSETS == 2:
                 load_a(E, j + 1)
             for k in range(o.D):
@@ -506,22 +549,16 @@ class UVWGenerator:
             E("}")
             E.level -= 1
             E("}")
+            if by_in1 and (j + 1 == len(items) or items[j + 1][1].a.idx != a.idx):
+                store_dx(E, a.idx)
         # ---- dX stores
         for a in self.in1:
             if a.dim == 0:
                 continue
             if a.idx not in self.used_in1:
                 E(f"if (wave == 0 && bvalid) for (int q = g; q < {a.dim}; q += 4) Xg[(row0 + c) * {self.D1} + {a.off} + q] = (T)0;")
-                continue
-            for q in range(_ceil(_ceil(a.mul, 16), 4)):
-                E(f"if (wave + {4 * q} < {_ceil(a.mul, 16)} && bvalid) {{")
-                E(f"    const int mt = wave + {4 * q};")
-                for r in range(4):
-                    E(f"    {{ const int u = 16 * mt + {self.row(r)};")
-                    guard = "" if a.mul % 16 == 0 else f"if (u < {a.mul}) "
-                    E(f"      {guard}{{ T* __restrict__ xp = Xg + (row0 + c) * {self.D1} + {a.off} + u * {a.D}; "
-                      + " ".join(f"xp[{i}] = dx{a.idx}_{q}_{r}_{i};" for i in range(a.D)) + " } }")
-                E("}")
+            elif not by_in1:
+                store_dx(E, a.idx)
         # ---- dY: sum over the 4 lane groups (channels), then over the 4 wavefronts, fixed order
         for f in self.used_y:
             E(f"dy{f} += oeq_shfl_xor(dy{f}, 16);")
