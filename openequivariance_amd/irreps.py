@@ -187,7 +187,7 @@ class Irreps(tuple):
     def lmax(self) -> int:
         if len(self) == 0:
             raise ValueError("Cannot get lmax of empty Irreps")
-        return max(b.ir.l for b in self)
+        return max(self.ls)          # blocks of multiplicity 0 do not count (reference: e3nn_lite.py:346-349)
 
     def slices(self) -> List[slice]:
         out, start = [], 0

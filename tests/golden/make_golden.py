@@ -82,6 +82,28 @@ def problem_cases():
     return cases
 
 
+IRREPS_CASES = ["1x0e", "0e + 1o + 2e", "32x0e+32x1o+32x2e", "2x1o + 3x0e + 2x1o + 0x2e + 1x1e", "4x0o+4x0e+4x1o",
+                "128x0e+128x1o+128x2e+128x3o", "10x1o + 10x1e + 48x0e + 48x0o", "3x2e+0x0e+3x2e", "7x5o"]
+
+
+def write_irreps_fixture(mod, dest):
+    """What the reference's Irreps reports for a few strings: text form, sizes and the derived forms."""
+    out = []
+    for text in IRREPS_CASES:
+        ir = mod.Irreps(text)
+        srt = ir.sort()
+        out.append(dict(text=text, repr=repr(ir), dim=int(ir.dim), num_irreps=int(ir.num_irreps), ls=[int(l) for l in ir.ls],
+                        lmax=int(ir.lmax), length=len(ir), muls=[int(m) for m, _ in ir], parities=[int(i.p) for _, i in ir],
+                        slices=[[sl.start, sl.stop] for sl in ir.slices()], simplify=repr(ir.simplify()),
+                        remove_zero=repr(ir.remove_zero_multiplicities()), sort=repr(srt.irreps), sort_p=list(srt.p),
+                        sort_inv=list(srt.inv), regroup=repr(ir.regroup()), count_1o=int(ir.count("1o")),
+                        contains_2e=bool("2e" in ir), times2=repr(ir * 2), plus=repr(ir + mod.Irreps("1x3e"))))
+    sh = {str(l): repr(mod.Irreps.spherical_harmonics(l)) for l in range(4)}
+    prod = {f"{a}*{b}": [repr(x) for x in mod.Irrep(a) * mod.Irrep(b)] for a, b in (("1o", "1o"), ("2e", "1o"), ("0e", "3o"), ("2o", "2e"))}
+    dest.write_text(json.dumps(dict(irreps=out, spherical_harmonics=sh, products=prod), indent=1) + "\n")
+    print(f"wrote {len(out)} irreps cases to {dest}")
+
+
 def write_problem_fixture(mod, dest):
     out = []
     for c in problem_cases():
@@ -92,7 +114,10 @@ def write_problem_fixture(mod, dest):
                                     path_shapes=[list(i.path_shape) for i in tpp.instructions],
                                     weight_numel=int(tpp.weight_numel),
                                     dims=[int(tpp.irreps_in1.dim), int(tpp.irreps_in2.dim), int(tpp.irreps_out.dim)],
-                                    shared_weights=bool(tpp.shared_weights), internal_weights=bool(tpp.internal_weights))))
+                                    shared_weights=bool(tpp.shared_weights), internal_weights=bool(tpp.internal_weights),
+                                    text=str(tpp), repr=repr(tpp),
+                                    weight_ranges=[[int(a), int(b), list(sh)] for a, b, sh in
+                                                   (tpp.weight_range_and_shape_for_instruction(i) for i in range(len(tpp.instructions)))])))
     dest.write_text(json.dumps(out, indent=1) + "\n")
     print(f"wrote {len(out)} problems to {dest}")
 
@@ -112,6 +137,7 @@ def main():
     np.savez_compressed(dest, **out)
     print(f"wrote {len(out)} tensors to {dest}")
     write_problem_fixture(mod, pathlib.Path(__file__).with_name("tpproblem.json"))
+    write_irreps_fixture(mod, pathlib.Path(__file__).with_name("irreps.json"))
 
 
 if __name__ == "__main__":

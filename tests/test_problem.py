@@ -153,3 +153,41 @@ def test_fully_connected_enumeration_matches_the_fixture():
     got = [(t.i_in1, t.i_in2, t.i_out, t.connection_mode) for t in prob.instructions]
     assert got == [tuple(t[:4]) for t in case["instructions"]]
     assert [(p["i1"], p["i2"], p["io"], p["mode"]) for p in spec.fully_connected(*common.DENSE, shared_weights=True).paths] == got
+
+
+GOLDEN_IRREPS = json.loads((pathlib.Path(__file__).parent / "golden" / "irreps.json").read_text())
+
+
+@pytest.mark.parametrize("case", GOLDEN_IRREPS["irreps"], ids=[c["text"] for c in GOLDEN_IRREPS["irreps"]])
+def test_irreps_behave_like_the_reference(case):
+    """Text form, sizes, slices and derived forms recorded from the reference's Irreps."""
+    ir = oeq.Irreps(case["text"])
+    assert repr(ir) == case["repr"] and ir.dim == case["dim"] and ir.num_irreps == case["num_irreps"]
+    assert list(ir.ls) == case["ls"] and ir.lmax == case["lmax"] and len(ir) == case["length"]
+    assert [m for m, _ in ir] == case["muls"] and [i.p for _, i in ir] == case["parities"]
+    assert [[s.start, s.stop] for s in ir.slices()] == case["slices"]
+    assert repr(ir.simplify()) == case["simplify"] and repr(ir.remove_zero_multiplicities()) == case["remove_zero"]
+    srt = ir.sort()
+    assert repr(srt.irreps) == case["sort"] and list(srt.p) == case["sort_p"] and list(srt.inv) == case["sort_inv"]
+    assert repr(ir.regroup()) == case["regroup"]
+    assert ir.count("1o") == case["count_1o"] and ("2e" in ir) == case["contains_2e"]
+    assert repr(ir * 2) == case["times2"] and repr(ir + oeq.Irreps("1x3e")) == case["plus"]
+
+
+def test_irrep_products_and_spherical_harmonics_like_the_reference():
+    from openequivariance_amd.irreps import Irrep
+    for key, want in GOLDEN_IRREPS["products"].items():
+        a, b = key.split("*")
+        assert [repr(x) for x in Irrep(a) * Irrep(b)] == want
+    for l, want in GOLDEN_IRREPS["spherical_harmonics"].items():
+        assert repr(oeq.Irreps.spherical_harmonics(int(l))) == want
+
+
+@pytest.mark.parametrize("case", GOLDEN_PROBLEMS, ids=[c["name"] for c in GOLDEN_PROBLEMS])
+def test_problem_text_and_weight_ranges_like_the_reference(case):
+    tpp = oeq.TPProblem(case["irreps_in1"], case["irreps_in2"], case["irreps_out"], [tuple(t) for t in case["instructions"]],
+                        **case["kwargs"])
+    exp = case["expect"]
+    assert str(tpp) == exp["text"]
+    got = [tpp.weight_range_and_shape_for_instruction(i) for i in range(len(tpp.instructions))]
+    assert [[a, b, list(sh)] for a, b, sh in got] == exp["weight_ranges"]
