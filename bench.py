@@ -217,7 +217,7 @@ def main():
         return
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (the path shards over rows/edges "
-              "without communication, see DESIGN.md)", file=sys.stderr)
+              "without communication and is measured on one)", file=sys.stderr)
         sys.exit(2)
 
     import numpy as np

@@ -43,14 +43,14 @@ def _run(prob, oprob, nodes, nnz, seed, deterministic, dtype=np.float32, sh_lmax
 
 @pytest.mark.parametrize("deterministic", [False, True])
 def test_nequip_conv(cuda, deterministic):
-    """BASELINE config 3 problem on a scaled-down random graph (no self loops)."""
+    """benchmark configuration 3 problem on a scaled-down random graph (no self loops)."""
     prob, oprob = common.channelwise(common.NEQUIP)
     _run(prob, oprob, 300, 9001, 31, deterministic, sh_lmax=2)
 
 
 @pytest.mark.parametrize("deterministic", [False, True])
 def test_large_conv(cuda, deterministic):
-    """BASELINE config 5 problem (mul 256 = four chunks) on a small graph."""
+    """benchmark configuration 5 problem (mul 256 = four chunks) on a small graph."""
     prob, oprob = common.channelwise(common.LARGE)
     _run(prob, oprob, 40, 700, 32, deterministic, sh_lmax=3)
 

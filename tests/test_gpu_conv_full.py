@@ -112,10 +112,10 @@ def _full_size(name, irreps, sh_lmax, cuda, n_nodes):
 
 
 def test_nequip_conv_full_size(cuda):
-    """BASELINE config 3: 5 000 nodes, 150 000 edges."""
+    """benchmark configuration 3: 5 000 nodes, 150 000 edges."""
     _full_size("nequip_conv_det", common.NEQUIP, 2, cuda, 40)
 
 
 def test_large_conv_full_size(cuda):
-    """BASELINE config 5: 20 000 nodes, Poisson(40) in-degree (about 800 000 edges)."""
+    """benchmark configuration 5: 20 000 nodes, Poisson(40) in-degree (about 800 000 edges)."""
     _full_size("large_conv_det", common.LARGE, 3, cuda, 6)

@@ -31,7 +31,7 @@ def _run(prob, oprob, n, seed, dtype, sh_lmax=None):
 
 
 def test_readme_single_path(cuda):
-    """BASELINE config 1: 1x2e (x) 1x3e -> 1x2e, batch 1000, inputs U[0,1), forward."""
+    """benchmark configuration 1: 1x2e (x) 1x3e -> 1x2e, batch 1000, inputs U[0,1), forward."""
     import torch
     import openequivariance_amd as oeq
     prob, oprob = common.readme_problem()
@@ -52,7 +52,7 @@ def test_readme_fwd_bwd(cuda, n):
 
 @pytest.mark.parametrize("n", [1, 130])
 def test_mace_uvu(cuda, n):
-    """BASELINE config 2 problem (17 paths, mul 128 = two 64-channel chunks)."""
+    """benchmark configuration 2 problem (17 paths, mul 128 = two 64-channel chunks)."""
     prob, oprob = common.channelwise(common.MACE)
     _run(prob, oprob, n, 2, np.float32, sh_lmax=3)
 
@@ -140,7 +140,7 @@ def test_empty_batch(cuda):
 
 
 def test_full_size_properties(cuda):
-    """BASELINE config 2 at its full batch (50 000): size-independent checks.
+    """benchmark configuration 2 at its full batch (50 000): size-independent checks.
     Tri-linearity in W, and the adjoint identity <G, Z> = <X, dX> = <Y, dY> = <W, dW>."""
     import torch
     import openequivariance_amd as oeq

@@ -39,7 +39,7 @@ def _run(irreps, n, seed, dtype, w_scale=0.125, sh_lmax=None):
 
 @pytest.mark.parametrize("n", [1, 16, 1000])
 def test_dense_uvw_fp32(cuda, n):
-    """BASELINE config 4 problem: 64x0e+64x1o+64x2e (x) SH(lmax 2) -> same, 11 paths, shared W ~ N(0, 1/64)."""
+    """benchmark configuration 4 problem: 64x0e+64x1o+64x2e (x) SH(lmax 2) -> same, 11 paths, shared W ~ N(0, 1/64)."""
     _run(common.DENSE, n, 40 + n, np.float32, sh_lmax=2)
 
 
