@@ -107,6 +107,8 @@ class UVWGenerator:
         self.bwd_a_sets = int(os.environ.get("OEQ_AMD_UVW_ASETS", "1"))
         self._bwd_lds_env = os.environ.get("OEQ_AMD_UVW_BWD_LDS", "1") == "1"
         self.fwd_xcd_map = os.environ.get("OEQ_AMD_UVW_FWD_XCD", "1") == "1"
+        # forward: contract the CG tensor with the row's Y once per path and apply the small matrix per channel
+        self.fwd_row_matrix = os.environ.get("OEQ_AMD_UVW_FWD_MATRIX", "1") == "1"
         # backward dW: fetch the operands of the next step while the current one runs (two register sets)
         self.dw_prefetch = os.environ.get("OEQ_AMD_UVW_DW_PREFETCH", "1" if self.T == "float" else "0") == "1"
         self.in1, self.in2, self.out = _blocks(problem.irreps_in1), _blocks(problem.irreps_in2), _blocks(problem.irreps_out)
@@ -232,6 +234,33 @@ class UVWGenerator:
         E("T " + ", ".join(f"{out}{k}" + ("" if k in seen else " = (T)0") for k in range(p.o.D)) + ";")
         E.extend(body)
 
+    def emit_cg_matrix(self, E: Emitter, p: WPath, y: str, m: str) -> None:
+        """{m}{i}_{k} = sum_j c_ijk {y}{off+j}: the CG tensor contracted with this row's second operand.
+        It depends on the batch row only, so one evaluation serves every channel of the row."""
+        terms = {}
+        for (i, j), ks in p.ordered_pairs():
+            for k, val in ks:
+                terms.setdefault((i, k), []).append((j, val))
+        for (i, k), lst in sorted(terms.items()):
+            expr = " + ".join(f"{self.lit(val)} * {y}{p.b.off + j}" for j, val in lst)
+            E(f"const T {m}{i}_{k} = {expr};")
+
+    def emit_cg_apply(self, E: Emitter, p: WPath, x: str, m: str, out: str) -> None:
+        """out{k} = sum_i {m}{i}_{k} * {x}{i}  (declares out0..)."""
+        by_k = {}
+        for (i, j), ks in p.ordered_pairs():
+            for k, _ in ks:
+                by_k.setdefault(k, set()).add(i)
+        for k in range(p.o.D):
+            if k not in by_k:
+                E(f"T {out}{k} = (T)0;")
+                continue
+            idx = sorted(by_k[k])
+            expr = f"{m}{idx[0]}_{k} * {x}{idx[0]}"
+            for i in idx[1:]:
+                expr = f"oeq_fma({m}{i}_{k}, {x}{i}, {expr})"
+            E(f"T {out}{k} = {expr};")
+
     def emit_cg_backward(self, E: Emitter, p: WPath, dt: str, x: str, y: str, dx: str, dy: str) -> None:
         """dx_i += s_ij y_j, dy_j += s_ij x_i with s_ij = sum_k c_ijk dt_k."""
         for (i, j), ks in p.ordered_pairs():
@@ -326,6 +355,8 @@ class UVWGenerator:
                 NG = _ceil(p.SU, GS)
                 regs = [f"nx{j}_{i}" for j in range(GS) for i in range(p.a.D)] + [f"nb{j}_{nt}" for j in range(GS) for nt in range(NT)]
                 E("T " + ", ".join(regs) + ";")
+                if self.fwd_row_matrix:
+                    self.emit_cg_matrix(E, p, "y", "m")
 
                 def load(E, gexp):
                     for j in range(GS):
@@ -352,7 +383,10 @@ class UVWGenerator:
                     E("{")
                     E.level += 1
                     E("const T " + ", ".join(f"x{i} = cnx{j}_{i}" for i in range(p.a.D)) + ";")
-                    self.emit_cg_forward(E, p, "x", "y", "t")
+                    if self.fwd_row_matrix:
+                        self.emit_cg_apply(E, p, "x", "m", "t")
+                    else:
+                        self.emit_cg_forward(E, p, "x", "y", "t")
                     if p.mu % 16 != 0 or NG * GS != p.SU:
                         E(f"if (16 * ((sg * {GS} + {j}) >> 2) + 4 * g + ((sg * {GS} + {j}) & 3) >= {p.mu}) {{ " + " ".join(f"t{k} = (T)0;" for k in range(o.D)) + " }")
                     for k in range(o.D):
