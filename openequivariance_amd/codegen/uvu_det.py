@@ -39,7 +39,7 @@ class UVUDetGenerator(UVUDirectGenerator):
         env = os.environ.get("OEQ_AMD_DET_PREFETCH")          # "0" / "1": tuning override for A/B runs
         if prefetch_backward is None and env in ("0", "1"):
             prefetch_backward = (env == "1")
-        self.prefetch_backward = (words <= 56) if prefetch_backward is None else prefetch_backward
+        self.prefetch_backward = (words <= 80) if prefetch_backward is None else prefetch_backward
         self.nontemporal = os.environ.get("OEQ_AMD_DET_NT", "1") == "1"   # streaming hint on W / Y / dW / dY
         self.uniform_rows = False          # validity is per lane (edge lists differ between sub-rows)
         self.chunk_in_grid = True
@@ -119,7 +119,8 @@ class UVUDetGenerator(UVUDirectGenerator):
             names += [f"x{i}_{m}" for m in range(self.in1[i].D)]
         names += [f"We_{p.t}_{v}" for p in self.paths for v in range(p.mv)]
         names += [f"y{f}" for f in self.used_y]
-        def load(E, it, h):
+        def load_idx(E, it, q):
+            """Edge position, sender (clamped) and validity of iteration ``it`` into index set q."""
             E("{")
             E.level += 1
             E(f"const bool ev = {self.edge_pos(it)} < len;")
@@ -134,7 +135,15 @@ class UVUDetGenerator(UVUDirectGenerator):
                 E(f"const u64 e = ev ? (u64)(beg + {self.edge_pos(it)}) : (u64)(nnz - 1);   // idle lanes re-read the last edge, masked below")
                 E("const i64 snd = cols[e];")
                 E("const bool rv = ev && snd >= 0 && snd < (i64)node_count;")
-            E("const u64 sndc = rv ? (u64)snd : 0;")
+            E(f"I{q}e = e; I{q}rv = rv; I{q}n = rv ? (u64)snd : 0;")
+            E.level -= 1
+            E("}")
+
+        def load(E, h, q):
+            """Operands of the edge described by index set q into register set h."""
+            E("{")
+            E.level += 1
+            E(f"const u64 e = I{q}e, sndc = I{q}n; const bool rv = I{q}rv;")
             E(f"const T* __restrict__ Yr = Y + e * {self.D2};")
             E(f"const T* __restrict__ Wr = W + e * {self.WN};")
             for f in self.used_y:
@@ -154,7 +163,7 @@ class UVUDetGenerator(UVUDirectGenerator):
         def compute(E, h):
             for oi in self.used_out:
                 self.emit_forward_block(E, self.out[oi], "Wr", zname=f"z{oi}_", declare=False)
-        self.emit_pingpong_loop(E, names, load, compute)
+        self.emit_pingpong_loop(E, names, load_idx, load, compute)
         E("const bool rv = nv;")
         for o in self.out:
             if o.dim == 0:
@@ -178,54 +187,66 @@ class UVUDetGenerator(UVUDirectGenerator):
     def uclamp(self, blk, c) -> str:
         return "u" if self.full(blk) else f"min(u, {blk.mul - 1})"
 
-    def emit_pingpong_loop(self, E: Emitter, names, load, compute, scalars: str = "", prefetch_first: bool = True) -> None:
-        """The edge loop, software pipelined over two register sets: while the edge held in one set is
-        computed, the operands of the following edge are in flight into the other set.  The loop body is
-        emitted twice (one copy per set) so that no register is copied from "next" to "current" at the
-        loop head.  ``load(E, it, h)`` fills set h for iteration ``it``; ``compute(E, h)`` sees the names
-        without prefix.  ``prefetch_first=False`` (large register footprints) keeps one set and requests the
-        next edge after the arithmetic."""
-        for h in (0, 1):
+    def emit_pingpong_loop(self, E: Emitter, names, load_idx, load, compute, prefetch_first: bool = True) -> None:
+        """The edge loop as a three-stage software pipeline.  Stage 1 (two iterations ahead) resolves
+        the indices of an edge - a chain of dependent loads: position list, edge id, neighbour row - into
+        one of two index sets; stage 2 (one iteration ahead) requests the edge's operands into one of two
+        register sets; stage 3 computes.  With the index chain inside stage 2 an iteration lasted three
+        memory round trips, whatever the amount of arithmetic.  The loop body is emitted twice (one copy
+        per register set), so nothing is copied from "next" to "current".  ``load_idx(E, it, q)`` fills
+        index set q for iteration ``it``, ``load(E, h, q)`` register set h from index set q, and
+        ``compute(E, h)`` sees the operand names without prefix and the edge as ``cur_e`` / ``cur_rv``.
+        ``prefetch_first=False`` (large register footprints) keeps one register set and requests the next
+        edge's operands after the arithmetic; its indices are still resolved an iteration early."""
+        nsets = 2 if prefetch_first else 1
+        for h in range(nsets):
             E("T " + ", ".join(f"S{h}{n} = (T)0" for n in names) + ";")
-        if scalars:
-            E(scalars)
+        E("u64 I0e = 0, I1e = 0, I0n = 0, I1n = 0; bool I0rv = false, I1rv = false;")
         E("if (maxlen > 0) {")
         E.level += 1
-        load(E, "0", 0)
+        load_idx(E, "0", 0)
+        load(E, 0, 0)
         E.level -= 1
         E("}")
-        if not prefetch_first:
-            # one register set is enough: it is refilled once the arithmetic on it is done
-            E("for (int it = 0; it < maxlen; ++it) {")
-            E.level += 1
-            E("const T " + ", ".join(f"{n} = S0{n}" for n in names) + ";")
-            compute(E, 0)
-            E("if (it + 1 < maxlen) {")
-            E.level += 1
-            load(E, "it + 1", 0)
-            E.level -= 1
-            E("}")
-            E.level -= 1
-            E("}")
-            return
+        E("if (maxlen > 1) {")
+        E.level += 1
+        load_idx(E, "1", 1)
+        E.level -= 1
+        E("}")
         E("for (int it = 0; it < maxlen; it += 2) {")
         E.level += 1
         for h in (0, 1):
-            nxt = f"it + {h + 1}"
             if h == 1:
                 E("if (it + 1 >= maxlen) break;")
             E("{")
             E.level += 1
-            E("const T " + ", ".join(f"{n} = S{h}{n}" for n in names) + ";")
-
-            def prefetch():
-                E(f"if ({nxt} < maxlen) {{")
+            hs = h if prefetch_first else 0
+            E("const T " + ", ".join(f"{n} = S{hs}{n}" for n in names) + ";")
+            E(f"const u64 cur_e = I{h}e; const bool cur_rv = I{h}rv; (void)cur_e; (void)cur_rv;")
+            if prefetch_first:
+                E(f"if (it + {h + 1} < maxlen) {{")
                 E.level += 1
-                load(E, nxt, 1 - h)
+                load(E, 1 - h, 1 - h)
                 E.level -= 1
                 E("}")
-            prefetch()
-            compute(E, h)
+                E(f"if (it + {h + 2} < maxlen) {{")
+                E.level += 1
+                load_idx(E, f"it + {h + 2}", h)
+                E.level -= 1
+                E("}")
+                compute(E, h)
+            else:
+                compute(E, h)
+                E(f"if (it + {h + 1} < maxlen) {{")
+                E.level += 1
+                load(E, 0, 1 - h)
+                E.level -= 1
+                E("}")
+                E(f"if (it + {h + 2} < maxlen) {{")
+                E.level += 1
+                load_idx(E, f"it + {h + 2}", h)
+                E.level -= 1
+                E("}")
             E.level -= 1
             E("}")
         E.level -= 1
@@ -248,7 +269,9 @@ class UVUDetGenerator(UVUDirectGenerator):
         names = [f"G{oi}_{k}" for oi in self.used_out for k in range(self.out[oi].D)]
         names += [f"We_{p.t}_{v}" for p in self.paths for v in range(p.mv)]
         names += [f"y{f}" for f in self.used_y]
-        def load(E, it, h):
+        def load_idx(E, it, q):
+            """Edge id, receiver (clamped) and validity of iteration ``it`` into index set q: a chain of two
+            dependent loads (position list, then the edge's receiver), kept off the data loads' critical path."""
             E("{")
             E.level += 1
             E(f"const bool ev = {self.edge_pos(it)} < len;")
@@ -258,8 +281,14 @@ class UVUDetGenerator(UVUDirectGenerator):
             E("const u64 e = ok_e ? (u64)e0 : 0;")
             E("const i64 rcv = rows[e];")
             E("const bool rv = ok_e && rcv >= 0 && rcv < (i64)node_count;")
-            E("const u64 rcvc = rv ? (u64)rcv : 0;")
-            E(f"S{h}e = e; S{h}rv = rv;")
+            E(f"I{q}e = e; I{q}rv = rv; I{q}n = rv ? (u64)rcv : 0;")
+            E.level -= 1
+            E("}")
+
+        def load(E, h, q):
+            E("{")
+            E.level += 1
+            E(f"const u64 e = I{q}e, rcvc = I{q}n; const bool rv = I{q}rv;")
             E(f"const T* __restrict__ Yr = Y + e * {self.D2};")
             E(f"const T* __restrict__ Wr = W + e * {self.WN};")
             for f in self.used_y:
@@ -277,7 +306,7 @@ class UVUDetGenerator(UVUDirectGenerator):
             E("}")
 
         def compute(E, h):
-            E(f"const u64 e = S{h}e; rv = S{h}rv;")
+            E("const u64 e = cur_e; rv = cur_rv;")
             E(f"T* __restrict__ Wgr = Wg + e * {self.WN};")
             for f in self.used_y:
                 E(f"T dy{f} = (T)0;")
@@ -303,8 +332,7 @@ class UVUDetGenerator(UVUDirectGenerator):
             for f in range(self.D2):
                 E(f"    Ygr[{f}] = " + (f"dy{f};" if f in self.used_y else "(T)0;"))
             E("}")
-        self.emit_pingpong_loop(E, names, load, compute, scalars="u64 S0e = 0, S1e = 0; bool S0rv = false, S1rv = false;",
-                                prefetch_first=self.prefetch_backward)
+        self.emit_pingpong_loop(E, names, load_idx, load, compute, prefetch_first=self.prefetch_backward)
         E("rv = nv;")
         for a in self.in1:
             if a.dim == 0:
