@@ -10,6 +10,11 @@ walks the node's edge list in order, so every sum has a fixed order and nothing 
   and Y, writes dW[e] (coalesced) and dY[e] (per-chunk partial when the multiplicity spans several
   chunks), and accumulates dX[node] in registers.
 
+The edge loop is software-pipelined: operands of the next edge are requested while the current one is
+computed, either into a second register set (emit_pingpong_loop) or, for fp32 problems whose
+multiplicity fits one chunk, through LDS by LDS-DMA (emit_staged_loop), which needs one register set
+and so keeps more wavefronts resident.
+
 All loads are unconditional from clamped, range-checked indices (see uvu_direct.py); an edge
 that is out of range for its lane, or names a node that does not exist, contributes zero.  The
 CSR pointers come from the prep kernels of the template (workspace).  The backward reads sender
@@ -19,7 +24,7 @@ kernel reads both at the unpermuted position: templates/loop_unroll_conv_det.cuh
 from __future__ import annotations
 
 from ..problem import TPProblem
-from .common import Emitter
+from .common import Emitter, WAVE
 from .uvu_direct import UVUDirectGenerator
 
 
@@ -41,6 +46,21 @@ class UVUDetGenerator(UVUDirectGenerator):
             prefetch_backward = (env == "1")
         self.prefetch_backward = (words <= 80) if prefetch_backward is None else prefetch_backward
         self.nontemporal = os.environ.get("OEQ_AMD_DET_NT", "1") == "1"   # streaming hint on W / Y / dW / dY
+        # backward operands of the next edge travel global -> LDS without passing through registers
+        # (LDS-DMA), which leaves room for a third wavefront per SIMD; see emit_staged_loop
+        self.stage_words = WAVE * (sum(self.dma_stride(w) for i in self.used_out for _, w in self.dma_pieces(self.out[i].D))
+                                   + sum(p.mv for p in self.paths) + 1)
+        env = os.environ.get("OEQ_AMD_DET_LDS")
+        fits = (self.T == "float" and self.P >= self.D2 and self.prefetch_backward
+                and 12 * self.stage_words * 4 <= 160 * 1024)
+        self.lds_backward = fits and env != "0"
+        if self.lds_backward:
+            self.waves_per_eu = 3
+        # the forward likewise when the multiplicity fits one chunk: few wavefronts per node, so the
+        # registers saved buy a fifth wavefront per SIMD (with several chunks per node it measured 1 % slower)
+        fwd_words = self._forward_slabs()[1]
+        self.lds_forward = (self.T == "float" and self.P >= self.D2 and self.NCH == 1 and env != "0"
+                            and 16 * (fwd_words + self.lds_elems) * 4 <= 160 * 1024)
         self.uniform_rows = False          # validity is per lane (edge lists differ between sub-rows)
         self.chunk_in_grid = True
 
@@ -111,9 +131,9 @@ class UVUDetGenerator(UVUDirectGenerator):
         self._cur_c = "e"
         for oi in self.used_out:
             E("T " + ", ".join(f"z{oi}_{k} = (T)0" for k in range(self.out[oi].D)) + ";")
-        # registers of the edge being fetched ("N" = next); the loop computes on a copy while the
-        # loads of the following edge are in flight (software pipelining hides the gather latency,
-        # which dominates when a node has few edges and few wavefronts are resident)
+        # operands of one edge; the loop computes on one set while the loads of the following edge are
+        # in flight (software pipelining hides the gather latency, which dominates when a node has few
+        # edges and few wavefronts are resident)
         names = []
         for i in self.used_in1:
             names += [f"x{i}_{m}" for m in range(self.in1[i].D)]
@@ -163,7 +183,10 @@ class UVUDetGenerator(UVUDirectGenerator):
         def compute(E, h):
             for oi in self.used_out:
                 self.emit_forward_block(E, self.out[oi], "Wr", zname=f"z{oi}_", declare=False)
-        self.emit_pingpong_loop(E, names, load_idx, load, compute)
+        if self.lds_forward:
+            self._emit_staged_forward(E, compute)
+        else:
+            self.emit_pingpong_loop(E, names, load_idx, load, compute)
         E("const bool rv = nv;")
         for o in self.out:
             if o.dim == 0:
@@ -252,6 +275,100 @@ class UVUDetGenerator(UVUDirectGenerator):
         E.level -= 1
         E("}")
 
+    # ------------------------------------------------------- LDS-staged operands
+    @staticmethod
+    def dma_pieces(D: int):
+        """Split a record of D words into LDS-DMA transfers (the hardware moves 1, 3 or 4 words per lane):
+        list of (first word, words), as few as possible."""
+        best = {0: []}
+        for n in range(1, D + 1):
+            best[n] = min(([*best[n - w], (n - w, w)] for w in (4, 3, 1) if n - w >= 0), key=len)
+        return best[D]
+
+    @staticmethod
+    def dma_stride(words: int) -> int:
+        """Words between the LDS destinations of consecutive lanes: a 3-word transfer lands at a 4-word
+        lane stride (measured on gfx950), 1- and 4-word transfers are packed."""
+        return 4 if words == 3 else words
+
+    def emit_staged_loop(self, E: Emitter, pos_of, pos_list, nbr_list: str, dma, readback, compute, flush=None) -> None:
+        """The edge loop with the operands of the next edge in flight to LDS while the current edge is
+        computed.  An LDS-DMA load holds no registers while it is outstanding, so this pipeline needs one
+        register set where emit_pingpong_loop needs two.  Four stages, none of which consumes a load
+        issued in the same iteration (the vector-memory counter retires in order, so waiting for a load
+        in the middle of an iteration would drain everything requested before it): the edge id of
+        iteration it+3 (``pos_list``[``pos_of``(it+3)], or the position itself without a list), the neighbour
+        row of it+2 (``nbr_list``[edge id]),
+        the operands of it+1 into the stage (``dma``), and the arithmetic of ``it``.  The values the first
+        two return are range-checked at the top of the following iteration.  Per iteration: read the
+        staged operands into registers, wait until every lane has them (the stage is then free), check
+        last iteration's indices, store last iteration's per-edge results (``flush``), issue the three
+        requests, compute.  The compiler does not order LDS reads after an outstanding LDS-DMA write by
+        itself, hence the explicit wait at the top; it waits for every earlier vector-memory access, which
+        is why the per-edge stores are issued in front of the requests and not from inside the
+        arithmetic, where they would be the youngest accesses at the next wait."""
+        def pos(it):
+            return f"(({pos_of(it)}) < len ? (u64)(beg + {pos_of(it)}) : (u64)(nnz - 1))"
+
+        def fetch(it):
+            return f"{pos_list}[{pos(it)}]" if pos_list else f"(i64){pos(it)}"
+
+        def edge_ok(raw, it):
+            return f"(({pos_of(it)}) < len && {raw} >= 0 && {raw} < (i64)nnz)"
+
+        def nbr_ok(raw):
+            return f"({raw} >= 0 && {raw} < (i64)node_count)"
+        E("u64 e0 = 0, e1 = 0, e2 = 0, n1 = 0; bool v0 = false, v1 = false, v2 = false; i64 rawE = 0, rawN = 0;")
+        # prologue: dependent loads, paid once per node
+        E("if (maxlen > 0) {")
+        E.level += 1
+        E(f"const i64 t_ = {fetch('0')}; v0 = {edge_ok('t_', '0')}; e0 = v0 ? (u64)t_ : 0;")
+        E(f"const i64 r_ = {nbr_list}[e0]; v0 = v0 && {nbr_ok('r_')}; n1 = v0 ? (u64)r_ : 0;")
+        dma(E, "e0", "n1")
+        E.level -= 1
+        E("}")
+        E("if (maxlen > 1) {")
+        E.level += 1
+        E(f"const i64 t_ = {fetch('1')}; v1 = {edge_ok('t_', '1')}; e1 = v1 ? (u64)t_ : 0;")
+        E(f"rawN = {nbr_list}[e1];")
+        E.level -= 1
+        E("}")
+        E(f"if (maxlen > 2) rawE = {fetch('2')};")
+        E("for (int it = 0; it < maxlen; ++it) {")
+        E.level += 1
+        E("const u64 cur_e = e0; const bool cur_rv = v0; (void)cur_e; (void)cur_rv;")
+        E("oeq_wait_vm();")
+        E("oeq_sync();")
+        readback(E)
+        E("oeq_wait_lds();")
+        E("oeq_sync();")
+        if flush:
+            E("if (it > 0) {")
+            E.level += 1
+            flush(E)
+            E.level -= 1
+            E("}")
+        # indices requested during the previous iteration
+        E(f"v1 = v1 && {nbr_ok('rawN')}; n1 = v1 ? (u64)rawN : 0;")
+        E(f"v2 = {edge_ok('rawE', 'it + 2')}; e2 = v2 ? (u64)rawE : 0;")
+        E("if (it + 1 < maxlen) {")
+        E.level += 1
+        dma(E, "e1", "n1")
+        E.level -= 1
+        E("}")
+        E(f"if (it + 2 < maxlen) rawN = {nbr_list}[e2];")
+        E(f"if (it + 3 < maxlen) rawE = {fetch('it + 3')};")
+        compute(E, 0)
+        E("e0 = e1; v0 = v1; e1 = e2; v1 = v2;")
+        E.level -= 1
+        E("}")
+        if flush:
+            E("if (maxlen > 0) {")
+            E.level += 1
+            flush(E)
+            E.level -= 1
+            E("}")
+
     # ================================================================ backward
     def conv_det_backward_body(self) -> str:
         E = Emitter()
@@ -318,11 +435,17 @@ class UVUDetGenerator(UVUDirectGenerator):
                     E(f"const T g{k} = G{oi}_{k};")
 
                 def sink(E, p, v, expr):
-                    E(f"  if ({self.act(p.a)}) {self.st('Wgr', self.widx(p, 'u', v), expr)}")
+                    if self.lds_backward:          # stored at the top of the next iteration (flush)
+                        E(f"  pw_{p.t}_{v} = {expr};")
+                    else:
+                        E(f"  if ({self.act(p.a)}) {self.st('Wgr', self.widx(p, 'u', v), expr)}")
                 self.emit_backward_block(E, o, "Wr", sink)
                 E.level -= 1
                 E("}")
             self.emit_dy_sum(E)
+            if self.lds_backward:
+                E(" ".join(f"pdy{f} = dy{f};" for f in self.used_y) + " pe = e; pv = rv;")
+                return
             writer = "ul == 0" if self.P < 64 else "lane == 63"
             E(f"if (rv && {writer}) {{")
             if self.NCH > 1:
@@ -332,7 +455,10 @@ class UVUDetGenerator(UVUDirectGenerator):
             for f in range(self.D2):
                 E(f"    Ygr[{f}] = " + (f"dy{f};" if f in self.used_y else "(T)0;"))
             E("}")
-        self.emit_pingpong_loop(E, names, load_idx, load, compute, prefetch_first=self.prefetch_backward)
+        if self.lds_backward:
+            self._emit_staged_backward(E, compute)
+        else:
+            self.emit_pingpong_loop(E, names, load_idx, load, compute, prefetch_first=self.prefetch_backward)
         E("rv = nv;")
         for a in self.in1:
             if a.dim == 0:
@@ -345,6 +471,137 @@ class UVUDetGenerator(UVUDirectGenerator):
             else:
                 self.emit_record_store(E, ["(T)0"] * a.D, dst, self.store_act(a))
         return E.text()
+
+    def _forward_slabs(self):
+        """(slabs, words) of the forward stage: X records of the sender, path weights, Y."""
+        slabs, off = [], 0
+        for i in self.used_in1:
+            for k0, w in self.dma_pieces(self.in1[i].D):
+                slabs.append(("X", i, k0, w, off))
+                off += WAVE * self.dma_stride(w)
+        for p in self.paths:
+            for v in range(p.mv):
+                slabs.append(("W", (p, v), 0, 1, off))
+                off += WAVE
+        return slabs, off + WAVE
+
+    def _emit_staged_forward(self, E: Emitter, compute) -> None:
+        nt = 2 if self.nontemporal else 0
+        slabs, words = self._forward_slabs()
+        y_off = words - WAVE
+        E(f"__shared__ __attribute__((aligned(16))) T stage[{words}];")
+
+        def dma(E, e, n):
+            E("{")
+            E.level += 1
+            E(f"const u64 e = {e}, sndc = {n};")
+            E(f"const T* __restrict__ Wr = W + e * {self.WN};")
+            E(f"OEQ_DMA(4, {nt}, Y + e * {self.D2} + min(ul, {self.D2 - 1}), stage + {y_off});")
+            for kind, key, k0, w, so in slabs:
+                if kind == "W":
+                    p, v = key
+                    E(f"OEQ_DMA(4, {nt}, Wr + {self.widx(p, self.uclamp(p.a, 0), v)}, stage + {so});")
+            for kind, key, k0, w, so in slabs:
+                if kind == "X":
+                    a = self.in1[key]
+                    E(f"OEQ_DMA({4 * w}, 0, X + sndc * {self.D1} + {a.off} + {self.uclamp(a, 0)} * {a.D} + {k0}, stage + {so});")
+            E.level -= 1
+            E("}")
+
+        def readback(E):
+            E("const bool rv = cur_rv;")
+            for f in self.used_y:
+                E(f"const T y{f} = stage[{y_off} + sub * {self.P} + {f}];")
+            for kind, key, k0, w, so in slabs:
+                if kind == "W":
+                    p, v = key
+                    E(f"const T We_{p.t}_{v} = stage[{so} + lane];")
+            for i in self.used_in1:
+                a = self.in1[i]
+                parts = []
+                for kind, key, k0, w, so in slabs:
+                    if kind == "X" and key == i:
+                        parts += [f"stage[{so} + lane * {self.dma_stride(w)} + {r}]" for r in range(w)]
+                # everything an edge adds is proportional to x: zero it for idle lanes
+                E(f"const bool a{i}_ = {self.act(a)};")
+                E("const T " + ", ".join(f"x{i}_{m} = a{i}_ ? {parts[m]} : (T)0" for m in range(a.D)) + ";")
+        self.emit_staged_loop(E, self.edge_pos, "eperm" if self.forward_perm else None, "cols", dma, readback, compute)
+
+    def _emit_staged_backward(self, E: Emitter, compute) -> None:
+        """Stage layout (words): per transfer a [64 lanes x lane stride] slab in lane order - the dZ records
+        of every output block, one word per path weight, and one slab whose lane (sub, f) holds Y[e_sub][f]."""
+        nt = 2 if self.nontemporal else 0          # cache policy bit "nt" for the streamed operands
+        slabs, off = [], 0                         # (kind, key, first word, words, slab offset)
+        for oi in self.used_out:
+            for k0, w in self.dma_pieces(self.out[oi].D):
+                slabs.append(("G", oi, k0, w, off))
+                off += WAVE * self.dma_stride(w)
+        for p in self.paths:
+            for v in range(p.mv):
+                slabs.append(("W", (p, v), 0, 1, off))
+                off += WAVE
+        y_off = off
+        off += WAVE
+        assert off == self.stage_words
+        E(f"__shared__ __attribute__((aligned(16))) T stage[{off}];")
+
+        def dma(E, e, n):
+            E("{")
+            E.level += 1
+            E(f"const u64 e = {e}, rcvc = {n};")
+            E(f"const T* __restrict__ Wr = W + e * {self.WN};")
+            E(f"OEQ_DMA(4, {nt}, Y + e * {self.D2} + min(ul, {self.D2 - 1}), stage + {y_off});")
+            for kind, key, k0, w, so in slabs:
+                if kind == "W":
+                    p, v = key
+                    E(f"OEQ_DMA(4, {nt}, Wr + {self.widx(p, self.uclamp(p.a, 0), v)}, stage + {so});")
+            for kind, key, k0, w, so in slabs:
+                if kind == "G":
+                    o = self.out[key]
+                    E(f"OEQ_DMA({4 * w}, 0, G + rcvc * {self.D3} + {o.off} + {self.uclamp(o, 0)} * {o.D} + {k0}, stage + {so});")
+            E.level -= 1
+            E("}")
+
+        def readback(E):
+            E("rv = cur_rv;")
+            for f in self.used_y:
+                E(f"const T y{f} = stage[{y_off} + sub * {self.P} + {f}];")
+            for kind, key, k0, w, so in slabs:
+                if kind == "W":
+                    p, v = key
+                    E(f"const T We_{p.t}_{v} = stage[{so} + lane];")
+            for oi in self.used_out:
+                o = self.out[oi]
+                parts = []
+                for kind, key, k0, w, so in slabs:
+                    if kind == "G" and key == oi:
+                        parts += [f"stage[{so} + lane * {self.dma_stride(w)} + {r}]" for r in range(w)]
+                # every gradient of an edge is proportional to dZ: zero it for idle lanes
+                E(f"const bool a{oi}_ = {self.act(o)};")
+                E("const T " + ", ".join(f"G{oi}_{k} = a{oi}_ ? {parts[k]} : (T)0" for k in range(o.D)) + ";")
+        def flush(E):
+            """Per-edge results of the edge computed last (dW row, dY row)."""
+            E("{")
+            E.level += 1
+            E("const u64 e = pe; const bool rv = pv;")
+            E(f"T* __restrict__ Wgr = Wg + e * {self.WN};")
+            for p in self.paths:
+                for v in range(p.mv):
+                    E(f"if ({self.act(p.a)}) {self.st('Wgr', self.widx(p, 'u', v), f'pw_{p.t}_{v}')}")
+            writer = "ul == 0" if self.P < 64 else "lane == 63"
+            E(f"if (rv && {writer}) {{")
+            if self.NCH > 1:
+                E(f"    T* __restrict__ Ygr = (T*)((char*)ws + DYPART_OFF) + ((u64)c * nnz + e) * {self.D2};")
+            else:
+                E(f"    T* __restrict__ Ygr = Yg + e * {self.D2};")
+            for f in range(self.D2):
+                E(f"    Ygr[{f}] = " + (f"pdy{f};" if f in self.used_y else "(T)0;"))
+            E("}")
+            E.level -= 1
+            E("}")
+        E("T " + ", ".join([f"pw_{p.t}_{v} = (T)0" for p in self.paths for v in range(p.mv)]
+                           + [f"pdy{f} = (T)0" for f in self.used_y]) + "; u64 pe = 0; bool pv = false;")
+        self.emit_staged_loop(E, self.edge_pos, "tperm", "rows", dma, readback, compute, flush)
 
     def emit_dy_sum(self, E: Emitter) -> None:
         """Sum dy* over the lanes of a row in a fixed order.  A full wavefront per row uses the

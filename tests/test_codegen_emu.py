@@ -81,6 +81,28 @@ def test_conv(variant):
         assert rel_err(got, ref) < TOL
 
 
+@pytest.mark.parametrize("staged", [True, False])
+def test_conv_det_long_edge_lists(staged, monkeypatch):
+    """Edge lists of about 13 edges per node (6-7 iterations of two sub-lists) reach the steady state of
+    the edge pipeline, with the next edge's operands staged through LDS and with register prefetch; the
+    last node has no edges."""
+    monkeypatch.setenv("OEQ_AMD_DET_LDS", "1" if staged else "0")
+    prob, oprob = common.channelwise(common.NEQUIP)
+    g = UVUDetGenerator(prob)
+    assert g.lds_backward == staged and g.lds_forward == staged
+    nodes, nnz = 4, 40
+    rows, cols = common.random_graph(nodes - 1, nnz, 11)          # node 3 has no edges
+    rows, cols, tperm, _ = otp.coord_graph(rows, cols)
+    X, Y, W, G = common.conv_inputs(prob, nodes, nnz, 12)
+    fwd, bwd, ws = g.plan()
+    out = emu.run_conv(g, fwd, X, Y, W, rows, cols, tperm=tperm, ws_bytes=ws(nnz, nodes))
+    assert rel_err(out["Z"], otp.conv_forward(oprob, X, Y, W, rows, cols)) < TOL
+    assert not out["Z"][3].any()
+    out = emu.run_conv(g, bwd, X, Y, W, rows, cols, G=G, tperm=tperm, ws_bytes=ws(nnz, nodes))
+    for got, ref in zip((out["Xg"], out["Yg"], out["Wg"]), otp.conv_backward(oprob, X, Y, W, G, rows, cols)):
+        assert rel_err(got, ref) < TOL
+
+
 def test_conv_det_chunked_ragged():
     irreps = ("5x0e+3x1o+70x2e", "1x0e+1x1o+1x2e", "5x0e+3x1o+70x2e+7x3o")
     prob, oprob = common.channelwise(irreps)

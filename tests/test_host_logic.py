@@ -84,3 +84,35 @@ def test_spherical_harmonics_inputs():
     np.testing.assert_allclose(Y[:, 1:4], np.sqrt(3) * n, atol=1e-13)
     for l in range(4):
         np.testing.assert_allclose((Y[:, l * l:(l + 1) ** 2] ** 2).sum(1), 2 * l + 1, atol=1e-12)
+
+
+def test_lds_dma_transfer_plan():
+    """Records are moved global -> LDS in transfers of 4, 3 or 1 words per lane, as few as possible, and
+    a 3-word transfer occupies a 4-word lane stride in LDS."""
+    from openequivariance_amd.codegen.uvu_det import UVUDetGenerator as G
+    assert G.dma_pieces(1) == [(0, 1)]
+    assert G.dma_pieces(3) == [(0, 3)]
+    assert G.dma_pieces(5) in ([(0, 4), (4, 1)], [(0, 1), (1, 4)])
+    assert sorted(w for _, w in G.dma_pieces(7)) == [3, 4]
+    assert sorted(w for _, w in G.dma_pieces(6)) == [3, 3]
+    for D in range(1, 12):
+        pieces = G.dma_pieces(D)
+        assert [k for k, _ in pieces] == [sum(w for _, w in pieces[:i]) for i in range(len(pieces))]
+        assert sum(w for _, w in pieces) == D
+    assert [G.dma_stride(w) for w in (1, 3, 4)] == [1, 4, 4]
+
+
+def test_staged_conv_selection(monkeypatch):
+    """The LDS-staged edge pipeline is used for fp32 problems whose multiplicity fits one chunk and
+    whose stage leaves room for three wavefronts per SIMD; other problems keep the register pipeline."""
+    from openequivariance_amd.codegen.uvu_det import UVUDetGenerator
+    from openequivariance_amd.problem import ChannelwiseTPP
+    monkeypatch.delenv("OEQ_AMD_DET_LDS", raising=False)
+    small = UVUDetGenerator(ChannelwiseTPP("32x0e+32x1o+32x2e", "1x0e+1x1o+1x2e", "32x0e+32x1o+32x2e"))
+    assert small.lds_forward and small.lds_backward and 12 * small.stage_words * 4 <= 160 * 1024
+    large = UVUDetGenerator(ChannelwiseTPP("256x0e+256x1o+256x2e", "1x0e+1x1o+1x2e+1x3o", "256x0e+256x1o+256x2e"))
+    assert not large.lds_forward and not large.lds_backward
+    import numpy as np
+    dbl = UVUDetGenerator(ChannelwiseTPP("32x0e+32x1o+32x2e", "1x0e+1x1o+1x2e", "32x0e+32x1o+32x2e",
+                                         irrep_dtype=np.float64, weight_dtype=np.float64))
+    assert not dbl.lds_forward and not dbl.lds_backward
