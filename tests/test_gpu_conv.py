@@ -68,6 +68,30 @@ def test_ragged_conv(cuda, deterministic):
     _run(prob, oprob, 50, 333, 34, deterministic)
 
 
+STAGED_SHAPES = {
+    "mul16_four_sublists": ("16x0e+16x1o", "1x0e+1x1o+1x2e", "16x0e+16x1o+16x2e"),
+    "mul8_eight_sublists": ("8x0e+8x1o", "1x0e+1x1o", "8x0e+8x1o"),
+    "mul64_one_list": ("64x0e+64x1o", "1x0e+1x1o", "64x0e+64x1o"),
+    "ragged_multiplicities": ("20x0e+9x1o+3x2e", "1x0e+1x1o+1x2e", "20x0e+9x1o+3x2e"),
+    "l3_seven_word_records": ("16x0e+16x3o", "1x0e+1x1o+1x2e+1x3o", "16x0e+16x1o+16x3o"),
+}
+
+
+@pytest.mark.parametrize("shape", sorted(STAGED_SHAPES))
+@pytest.mark.parametrize("deterministic", [False, True])
+def test_lds_staged_edge_loop_shapes(cuda, shape, deterministic):
+    """Single-chunk fp32 problems run the edge loop that stages operands through LDS (deterministic:
+    forward and backward; unsorted: forward): every sub-list count, ragged multiplicities, and records of
+    1, 3, 5 and 7 words (one, one, two and two LDS-DMA transfers), with long and empty edge lists."""
+    from openequivariance_amd.conv import select_conv_generator
+    prob, oprob = common.channelwise(STAGED_SHAPES[shape])
+    gen = select_conv_generator(prob, deterministic)
+    staged = gen if deterministic else gen.fwd
+    assert staged.lds_forward and (staged.lds_backward or not deterministic)
+    _run(prob, oprob, 23, 700, 40, deterministic)        # about 30 edges per node
+    _run(prob, oprob, 200, 150, 41, deterministic)       # most nodes have no edge or a single one
+
+
 def test_conv_fp64(cuda):
     prob, oprob = common.channelwise(common.NEQUIP, dtype=np.float64)
     _run(prob, oprob, 64, 900, 35, True, dtype=np.float64, sh_lmax=2)
