@@ -32,11 +32,23 @@ class UVUDetGenerator(UVUDirectGenerator):
     _allow_det = True
 
     def __init__(self, problem: TPProblem, prefetch_backward=None, vector_stores: bool = True,
-                 forward_perm: bool = False):
+                 forward_perm: bool = False, backward_perm: bool = False):
         super().__init__(problem, "conv_det", vector_stores=vector_stores)
         # True: the forward walks the receiver-grouped edge order listed in the workspace (built on
         # the fly from an unsorted edge list) instead of the edge list itself
         self.forward_perm = forward_perm
+        # True: the backward likewise walks a sender-grouped order built in the workspace
+        # (pointers | cursors | position list | dY partials) instead of the caller's transpose permutation
+        # (receiver pointers | sender pointers | dY partials)
+        self.backward_perm = backward_perm
+        if backward_perm:
+            self.bwd_ptr_off = "0"
+            self.bwd_list = "((const i64*)ws + 2 * (node_count + 1))"
+            self.dypart_off = "(2 * (node_count + 1) + nnz) * sizeof(i64)"
+        else:
+            self.bwd_ptr_off = "(node_count + 1)"
+            self.bwd_list = "tperm"
+            self.dypart_off = "2 * (node_count + 1) * sizeof(i64)"
         # fetch the next edge's operands while the current edge is being computed; pays when the
         # per-edge register footprint is small enough to keep several wavefronts per SIMD
         words = sum(self.out[i].D for i in self.used_out) + len(self.paths) + len(self.used_y)
@@ -373,7 +385,8 @@ class UVUDetGenerator(UVUDirectGenerator):
     def conv_det_backward_body(self) -> str:
         E = Emitter()
         self.emit_lane_direct(E, lds=False)
-        self._node_setup(E, "(node_count + 1)")
+        self._node_setup(E, self.bwd_ptr_off)
+        E(f"const i64* __restrict__ elist = {self.bwd_list};     // edge ids in (sender, ...) order")
         self._cur_c = "e"
         # this node's own X chunk (fixed over the edge loop)
         E("bool rv = nv;")
@@ -393,7 +406,7 @@ class UVUDetGenerator(UVUDirectGenerator):
             E.level += 1
             E(f"const bool ev = {self.edge_pos(it)} < len;")
             E(f"const u64 j = ev ? (u64)(beg + {self.edge_pos(it)}) : (u64)(nnz - 1);")
-            E("const i64 e0 = tperm[j];")
+            E("const i64 e0 = elist[j];")
             E("const bool ok_e = ev && e0 >= 0 && e0 < (i64)nnz;")
             E("const u64 e = ok_e ? (u64)e0 : 0;")
             E("const i64 rcv = rows[e];")
@@ -601,7 +614,7 @@ class UVUDetGenerator(UVUDirectGenerator):
             E("}")
         E("T " + ", ".join([f"pw_{p.t}_{v} = (T)0" for p in self.paths for v in range(p.mv)]
                            + [f"pdy{f} = (T)0" for f in self.used_y]) + "; u64 pe = 0; bool pv = false;")
-        self.emit_staged_loop(E, self.edge_pos, "tperm", "rows", dma, readback, compute, flush)
+        self.emit_staged_loop(E, self.edge_pos, "elist", "rows", dma, readback, compute, flush)
 
     def emit_dy_sum(self, E: Emitter) -> None:
         """Sum dy* over the lanes of a row in a fixed order.  A full wavefront per row uses the

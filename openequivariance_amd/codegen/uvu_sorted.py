@@ -10,13 +10,18 @@ edges inside a node's group depends on the order in which the integer atomics la
 floating-point sums may differ in the last bits between runs, like the atomic kernel they replace
 (reference: templates/loop_unroll_conv_atomic.cuh:25-141 scatters with atomicAdd).
 
-The backward keeps the register-direct kernel with coalesced atomics: it scatters only d1 values
-per edge (dX) while dW and dY are per-edge outputs.
+The backward scatters only d1 values per edge (dX), dW and dY being per-edge outputs.  While d1 is
+small it keeps the register-direct kernel with coalesced atomics; from ATOMIC_BACKWARD_MAX_D1
+values per edge on, the atomics retire slower than the row gathers of the segmented backward, and
+the backward groups the edges by sender in the same way and runs the deterministic variant's
+backward over that order.
 
 Workspace: (node_count + 1) group pointers, (node_count + 1) fill cursors and nnz edge positions,
-all int64, rebuilt on every forward call.
+all int64 (then the per-chunk dY partial sums of the grouped backward), rebuilt on every call.
 """
 from __future__ import annotations
+
+import os
 
 from ..problem import TPProblem
 from .common import jinja_env
@@ -28,16 +33,29 @@ class UVUSortedGenerator:
     kind = "conv_atomic"
     SCAN_THREADS = 1024
 
-    def __init__(self, problem: TPProblem, vector_stores: bool = True):
+    # dX values per edge from which the grouped backward is used (measured: 288 per edge - atomic 202 us,
+    # grouped 209 us; 2304 per edge - atomic 9.1 ms, grouped 7.7 ms)
+    ATOMIC_BACKWARD_MAX_D1 = 1024
+
+    def __init__(self, problem: TPProblem, vector_stores: bool = True, grouped_backward=None):
         self.problem = problem
         self.fwd = UVUDetGenerator(problem, forward_perm=True, vector_stores=vector_stores)
-        self.bwd = UVUDirectGenerator(problem, "conv_atomic", vector_stores=vector_stores)
+        if grouped_backward is None:
+            env = os.environ.get("OEQ_AMD_CONV_BACKWARD")            # "grouped" / "atomic": A/B runs
+            grouped_backward = (env == "grouped") if env in ("grouped", "atomic") \
+                else self.fwd.D1 >= self.ATOMIC_BACKWARD_MAX_D1
+        self.grouped_backward = grouped_backward
+        if grouped_backward:
+            self.bwd = UVUDetGenerator(problem, backward_perm=True, vector_stores=vector_stores)
+        else:
+            self.bwd = UVUDirectGenerator(problem, "conv_atomic", vector_stores=vector_stores)
         self.T = self.fwd.T
         self.D1, self.D2, self.D3, self.WN = self.fwd.D1, self.fwd.D2, self.fwd.D3, self.fwd.WN
         self.NCH = self.fwd.NCH
 
     def describe(self) -> str:
-        return "sorted forward: " + self.fwd.describe() + " | atomic backward: " + self.bwd.describe()
+        return ("sorted forward: " + self.fwd.describe()
+                + (" | grouped backward: " if self.grouped_backward else " | atomic backward: ") + self.bwd.describe())
 
     def render(self, prelude: str = None) -> str:
         env = jinja_env()
@@ -53,8 +71,22 @@ class UVUSortedGenerator:
                dict(kernel="group_scan", num_threads=self.SCAN_THREADS, grid_kind=FIXED, num_blocks=1),
                dict(kernel="group_fill", num_threads=256, grid_kind=ROW, work_per_block=256),
                dict(kernel="forward", num_threads=64, grid_kind=NODE, work_per_block=1, grid_y=f.NCH)]
-        _, bwd, _ = self.bwd.plan()
+        if not self.grouped_backward:
+            _, bwd, _ = self.bwd.plan()
+
+            def ws(nnz=0, nodes=0):
+                return (2 * (nodes + 1) + nnz) * 8
+            return fwd, bwd, ws
+        b = self.bwd
+        bwd = [dict(kernel="group_clear_backward", num_threads=256, grid_kind=NODE, work_per_block=256),
+               dict(kernel="group_count_backward", num_threads=256, grid_kind=ROW, work_per_block=256),
+               dict(kernel="group_scan_backward", num_threads=self.SCAN_THREADS, grid_kind=FIXED, num_blocks=1),
+               dict(kernel="group_fill_backward", num_threads=256, grid_kind=ROW, work_per_block=256),
+               dict(kernel="backward", num_threads=64, grid_kind=NODE, work_per_block=1, grid_y=b.NCH)]
+        if b.NCH > 1:
+            bwd.append(dict(kernel="backward_dy_reduce", num_threads=256, grid_kind=ROW,
+                            work_per_block=b.dy_rows_per_block))
 
         def ws(nnz=0, nodes=0):
-            return (2 * (nodes + 1) + nnz) * 8
+            return (2 * (nodes + 1) + nnz) * 8 + (b.NCH * nnz * b.D2 * b.itemsize if b.NCH > 1 else 0)
         return fwd, bwd, ws

@@ -125,6 +125,8 @@ class TensorProductConv:
         self.generator = select_conv_generator(config, deterministic)
         # True: the forward writes every row of Z itself; False: it accumulates into a zeroed Z
         self.forward_overwrites = not isinstance(self.generator, UVUDirectGenerator) or deterministic
+        # likewise for dX in the backward (the per-edge backward accumulates with atomics)
+        self.backward_overwrites = deterministic or getattr(self.generator, "grouped_backward", False)
         self.jit_kernel = self.generator.render()
         code = rt.compile_source(self.jit_kernel)
         fwd, bwd, self._ws_bytes = self.generator.plan()
@@ -230,7 +232,7 @@ class TensorProductConv:
             tperm = tperm.contiguous() if tperm is not None else None
             self._check(x, y, w, rows, cols, tperm)
             E, N = rows.shape[0], x.shape[0]
-            xg = (torch.empty_like if det else torch.zeros_like)(x)
+            xg = (torch.empty_like if self.backward_overwrites else torch.zeros_like)(x)
             yg, wg = torch.empty_like(y), torch.empty_like(w)
             self.backward_rawptrs(x.data_ptr(), xg.data_ptr(), y.data_ptr(), yg.data_ptr(), w.data_ptr(),
                                   wg.data_ptr(), g.data_ptr(), rows.data_ptr(), cols.data_ptr(), E, N,
@@ -461,7 +463,7 @@ class TensorProductConv:
             nbytes = self._ws_bytes(graph.nnz, graph.node_count)
             ws = rt.DeviceBuffer(nbytes) if nbytes else None
             ptrs = [b.data_ptr() for b in bufs]
-            zero = (lambda: None) if self.deterministic else (lambda: bufs[1].zero())
+            zero = (lambda: None) if self.backward_overwrites else (lambda: bufs[1].zero())
             times = self._timed(num_warmup, num_iter, lambda: self.internal.backward_rawptrs(
                 *ptrs, graph.nnz, graph.node_count, ws.data_ptr() if ws else 0, tp.data_ptr() if tp else 0, 0), zero)
         ops, data, _ = flops_data_per_tp(self.config, "backward")

@@ -180,8 +180,8 @@ class Workload:
                 op.exec_conv_rawptrs(p["X"], p["Y"], p["W"], p["Z"], p["rows"], p["cols"], E, N, ws, tp_ptr, stream)
 
             def bwd():
-                if not det:
-                    t["Xg"].zero_()
+                if not op.backward_overwrites:
+                    t["Xg"].zero_()             # likewise for the backward that scatters dX with atomics
                 op.backward_rawptrs(p["X"], p["Xg"], p["Y"], p["Yg"], p["W"], p["Wg"], p["G"], p["rows"], p["cols"],
                                     E, N, ws, tp_ptr, stream)
         return Case(op, t, fwd, bwd, h)

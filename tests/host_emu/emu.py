@@ -204,6 +204,12 @@ CONV_EXTRA_SORTED = r"""
         else if (k == "group_scan") FWD_CALL(group_scan);
         else if (k == "group_fill") FWD_CALL(group_fill);
 """
+CONV_EXTRA_GROUPED_BWD = r"""
+        else if (k == "group_clear_backward") BWD_CALL(group_clear_backward);
+        else if (k == "group_count_backward") BWD_CALL(group_count_backward);
+        else if (k == "group_scan_backward") BWD_CALL(group_scan_backward);
+        else if (k == "group_fill_backward") BWD_CALL(group_fill_backward);
+"""
 CONV_EXTRA_DYRED = r"""
         else if (k == "backward_dy_reduce") BWD_CALL(backward_dy_reduce);
 """
@@ -284,6 +290,10 @@ def run_conv(gen, steps: Sequence[Dict], X, Y, W, rows, cols, G=None, tperm=None
             extra += CONV_EXTRA_DYRED
     elif hasattr(gen, "fwd"):
         extra += CONV_EXTRA_SORTED
+        if gen.grouped_backward:
+            extra += CONV_EXTRA_GROUPED_BWD
+            if gen.bwd.NCH > 1:
+                extra += CONV_EXTRA_DYRED
     exe = build(gen.render(prelude=emu_prelude(gen.T)), CONV_MAIN.replace("@EXTRA@", extra))
     nodes, nnz = X.shape[0], rows.shape[0]
     with tempfile.TemporaryDirectory() as d:

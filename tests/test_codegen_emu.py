@@ -58,11 +58,12 @@ def test_generic_tp_shared_weights():
         assert rel_err(got, ref) < TOL
 
 
-@pytest.mark.parametrize("variant", ["atomic", "det", "sorted"])
+@pytest.mark.parametrize("variant", ["atomic", "det", "sorted", "sorted_grouped_backward"])
 def test_conv(variant):
     prob, oprob = common.channelwise(common.NEQUIP)
     det = variant == "det"
-    g = {"det": UVUDetGenerator, "sorted": UVUSortedGenerator,
+    g = {"det": UVUDetGenerator, "sorted": lambda p: UVUSortedGenerator(p, grouped_backward=False),
+         "sorted_grouped_backward": lambda p: UVUSortedGenerator(p, grouped_backward=True),
          "atomic": lambda p: UVUDirectGenerator(p, "conv_atomic")}[variant](prob)
     nodes, nnz = 7, 19
     rows, cols = common.random_graph(nodes, nnz, 5)
@@ -73,10 +74,12 @@ def test_conv(variant):
     fwd, bwd, ws = g.plan()
     # (a transpose permutation makes the emulator start from a junk-filled Z: the deterministic and
     # the sorted forward must write every row themselves; the sorted kernels never read it)
-    out = emu.run_conv(g, fwd, X, Y, W, rows, cols, tperm=np.arange(nnz) if variant == "sorted" else tperm,
+    junk = np.arange(nnz)
+    out = emu.run_conv(g, fwd, X, Y, W, rows, cols, tperm=junk if variant.startswith("sorted") else tperm,
                        ws_bytes=ws(nnz, nodes))
     assert rel_err(out["Z"], otp.conv_forward(oprob, X, Y, W, rows, cols)) < TOL
-    out = emu.run_conv(g, bwd, X, Y, W, rows, cols, G=G, tperm=tperm, ws_bytes=ws(nnz, nodes))
+    out = emu.run_conv(g, bwd, X, Y, W, rows, cols, G=G, tperm=junk if variant == "sorted_grouped_backward" else tperm,
+                       ws_bytes=ws(nnz, nodes))
     for got, ref in zip((out["Xg"], out["Yg"], out["Wg"]), otp.conv_backward(oprob, X, Y, W, G, rows, cols)):
         assert rel_err(got, ref) < TOL
 

@@ -116,3 +116,26 @@ def test_staged_conv_selection(monkeypatch):
     dbl = UVUDetGenerator(ChannelwiseTPP("32x0e+32x1o+32x2e", "1x0e+1x1o+1x2e", "32x0e+32x1o+32x2e",
                                          irrep_dtype=np.float64, weight_dtype=np.float64))
     assert not dbl.lds_forward and not dbl.lds_backward
+
+
+def test_unsorted_conv_backward_selection(monkeypatch):
+    """Unsorted edge lists: the backward scatters dX with atomics while a row of X is short, and groups
+    the edges by sender (four more grouping launches, the segmented backward, larger workspace) from
+    1024 values per edge on."""
+    from openequivariance_amd.codegen.uvu_sorted import UVUSortedGenerator
+    from openequivariance_amd.problem import ChannelwiseTPP
+    monkeypatch.delenv("OEQ_AMD_CONV_BACKWARD", raising=False)
+    small = UVUSortedGenerator(ChannelwiseTPP("32x0e+32x1o+32x2e", "1x0e+1x1o+1x2e", "32x0e+32x1o+32x2e"))
+    large = UVUSortedGenerator(ChannelwiseTPP("256x0e+256x1o+256x2e", "1x0e+1x1o+1x2e+1x3o", "256x0e+256x1o+256x2e"))
+    assert not small.grouped_backward and large.grouped_backward
+    _, bwd, ws = small.plan()
+    assert [s["kernel"] for s in bwd] == ["backward"]
+    assert ws(1000, 10) == (2 * 11 + 1000) * 8
+    _, bwd, ws = large.plan()
+    assert [s["kernel"] for s in bwd] == ["group_clear_backward", "group_count_backward", "group_scan_backward",
+                                          "group_fill_backward", "backward", "backward_dy_reduce"]
+    assert bwd[4]["grid_y"] == 4 and bwd[4]["work_per_block"] == 1
+    assert ws(1000, 10) == (2 * 11 + 1000) * 8 + 4 * 1000 * 16 * 4
+    src = large.render()
+    for name in ("group_fill_backward", "backward_dy_reduce", "void backward("):
+        assert name in src
