@@ -536,8 +536,10 @@ class UVUDetGenerator(UVUDirectGenerator):
                     if kind == "X" and key == i:
                         parts += [f"stage[{so} + lane * {self.dma_stride(w)} + {r}]" for r in range(w)]
                 # everything an edge adds is proportional to x: zero it for idle lanes
+                # (read unconditionally, then masked: a conditional expression would put a branch around every LDS read)
                 E(f"const bool a{i}_ = {self.act(a)};")
-                E("const T " + ", ".join(f"x{i}_{m} = a{i}_ ? {parts[m]} : (T)0" for m in range(a.D)) + ";")
+                E("const T " + ", ".join(f"xr{i}_{m} = {parts[m]}" for m in range(a.D)) + ";")
+                E("const T " + ", ".join(f"x{i}_{m} = a{i}_ ? xr{i}_{m} : (T)0" for m in range(a.D)) + ";")
         self.emit_staged_loop(E, self.edge_pos, "eperm" if self.forward_perm else None, "cols", dma, readback, compute)
 
     def _emit_staged_backward(self, E: Emitter, compute) -> None:
@@ -590,8 +592,10 @@ class UVUDetGenerator(UVUDirectGenerator):
                     if kind == "G" and key == oi:
                         parts += [f"stage[{so} + lane * {self.dma_stride(w)} + {r}]" for r in range(w)]
                 # every gradient of an edge is proportional to dZ: zero it for idle lanes
+                # (read unconditionally, then masked: a conditional expression would put a branch around every LDS read)
                 E(f"const bool a{oi}_ = {self.act(o)};")
-                E("const T " + ", ".join(f"G{oi}_{k} = a{oi}_ ? {parts[k]} : (T)0" for k in range(o.D)) + ";")
+                E("const T " + ", ".join(f"Gr{oi}_{k} = {parts[k]}" for k in range(o.D)) + ";")
+                E("const T " + ", ".join(f"G{oi}_{k} = a{oi}_ ? Gr{oi}_{k} : (T)0" for k in range(o.D)) + ";")
         def flush(E):
             """Per-edge results of the edge computed last (dW row, dY row)."""
             E("{")

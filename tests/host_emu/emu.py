@@ -59,7 +59,7 @@ static inline int oeq_shfl_i32(int v, int src) { g_xi[threadIdx.x] = v; oeq_sync
 static inline int oeq_shfl_xor_i32(int v, int mask) { g_xi[threadIdx.x] = v; oeq_sync(); int r = g_xi[threadIdx.x ^ mask]; oeq_sync(); return r; }
 #define __builtin_amdgcn_readfirstlane(x) oeq_shfl_i32((x), 0)
 struct VT { T v[16 / sizeof(T)]; T& operator[](int i) { return v[i]; } const T& operator[](int i) const { return v[i]; } };
-#define OEQ_DMA(BYTES, POLICY, g, lds_base) memcpy((char*)(lds_base) + ((BYTES) == 12 ? 16 : (BYTES)) * threadIdx.x, (g), (BYTES))
+#define OEQ_DMA(BYTES, POLICY, g, lds_base) memcpy((char*)(lds_base) + ((BYTES) == 12 ? 16 : (BYTES)) * (threadIdx.x & 63), (g), (BYTES))
 static inline void oeq_wait_vm() {}
 static inline void oeq_wait_lds() {}
 static inline T oeq_wave_sum63(T v) { g_xT[threadIdx.x] = v; oeq_sync(); T t = 0; for (int i = 0; i < 64; ++i) t += g_xT[(threadIdx.x & ~63) + i]; oeq_sync(); return t; }
