@@ -163,6 +163,41 @@ def test_full_size_properties(cuda):
     assert rel_err(z.detach()[sl].cpu().numpy(), otp.forward(oprob, X[sl], Y[sl], W[sl])) <= FP32_TOL
 
 
+def test_tensors_beyond_two_giga_elements(cuda):
+    """A batch whose weight tensor has more than 2^31 elements (1.8 M rows of the MACE problem: W and dW
+    9.2 GB each): row offsets must be 64-bit everywhere.  Rows at the start, around element 2^31 and at
+    the end are compared with the oracle on the same inputs (each row depends on that row only)."""
+    import torch
+    import openequivariance_amd as oeq
+    from openequivariance_amd.sh import random_unit_vectors, spherical_harmonics
+    prob, oprob = common.channelwise(common.MACE)
+    n = 1_800_000
+    d1, d3, wn = prob.irreps_in1.dim, prob.irreps_out.dim, prob.weight_numel
+    assert n * wn > 2 ** 31 and n * d3 > 2 ** 31
+    gen = torch.Generator(device=cuda)
+    gen.manual_seed(99)
+    x = torch.randn(n, d1, device=cuda, generator=gen, requires_grad=True)
+    w = torch.randn(n, wn, device=cuda, generator=gen, requires_grad=True)
+    g = torch.randn(n, d3, device=cuda, generator=gen)
+    Y = spherical_harmonics(3, random_unit_vectors(n, np.random.default_rng(99))).astype(np.float32)
+    y = torch.tensor(Y, device=cuda, requires_grad=True)
+    tp = oeq.TensorProduct(prob, torch_op=True)
+    z = tp(x, y, w)
+    z.backward(g)
+    torch.cuda.synchronize()
+    mid = 2 ** 31 // wn
+    rows = np.r_[0:40, mid - 20:mid + 20, n - 40:n]
+    t = torch.from_numpy(rows).to(cuda)
+    Xs, Ws, Gs = (a.detach()[t].cpu().numpy() for a in (x, w, g))
+    Zr = otp.forward(oprob, Xs, Y[rows], Ws)
+    dXr, dYr, dWr = otp.backward(oprob, Xs, Y[rows], Ws, Gs)
+    errs = dict(Z=rel_err(z.detach()[t].cpu().numpy(), Zr), dX=rel_err(x.grad[t].cpu().numpy(), dXr),
+                dY=rel_err(y.grad[t].cpu().numpy(), dYr), dW=rel_err(w.grad[t].cpu().numpy(), dWr))
+    print(f"n={n} rows sampled={rows.size} {errs}", flush=True)
+    for k, v in errs.items():
+        assert v <= FP32_TOL, f"{k}: relative error {v:.3e}"
+
+
 def _misaligned(a, dev):
     """Contiguous device copy of ``a`` whose storage starts 4 bytes past a 16-byte boundary."""
     import torch

@@ -84,6 +84,49 @@ def test_dw_bit_reproducible_and_full_batch(cuda):
     assert rel_err(z.detach()[sl].cpu().numpy(), otp.forward(oprob, X[sl], Y[sl], We_)) <= FP32_TOL
 
 
+def test_uvw_tensors_beyond_two_giga_elements(cuda):
+    """3.8 M rows of the config-4 problem: X, Z and their gradients have more than 2^31 elements each.
+    Sampled rows (start, around element 2^31, end) of Z, dX, dY against the oracle; dW, which sums over
+    all rows, against the sum of the dW of the two halves of the batch (each below 2^31 elements)."""
+    import torch
+    import openequivariance_amd as oeq
+    from openequivariance_amd.sh import random_unit_vectors, spherical_harmonics
+    prob, oprob = common.fully_connected(common.DENSE, shared=True)
+    n = 3_800_000
+    d1, d3, wn = prob.irreps_in1.dim, prob.irreps_out.dim, prob.weight_numel
+    assert n * d1 > 2 ** 31 and n * d3 > 2 ** 31
+    gen = torch.Generator(device=cuda)
+    gen.manual_seed(98)
+    x = torch.randn(n, d1, device=cuda, generator=gen, requires_grad=True)
+    g = torch.randn(n, d3, device=cuda, generator=gen)
+    w = (0.125 * torch.randn(wn, device=cuda, generator=gen)).requires_grad_(True)
+    Y = spherical_harmonics(2, random_unit_vectors(n, np.random.default_rng(98))).astype(np.float32)
+    y = torch.tensor(Y, device=cuda, requires_grad=True)
+    tp = oeq.TensorProduct(prob, torch_op=True)
+    z = tp(x, y, w)
+    z.backward(g)
+    torch.cuda.synchronize()
+    mid = 2 ** 31 // d1
+    rows = np.r_[0:20, mid - 10:mid + 10, n - 20:n]
+    t = torch.from_numpy(rows).to(cuda)
+    We = ow.oeq_to_e3nn(oprob, w.detach().cpu().numpy())
+    Xs, Gs = x.detach()[t].cpu().numpy(), g[t].cpu().numpy()
+    Zr = otp.forward(oprob, Xs, Y[rows], We)
+    dXr, dYr, _ = otp.backward(oprob, Xs, Y[rows], We, Gs)
+    errs = dict(Z=rel_err(z.detach()[t].cpu().numpy(), Zr), dX=rel_err(x.grad[t].cpu().numpy(), dXr),
+                dY=rel_err(y.grad[t].cpu().numpy(), dYr))
+    half = n // 2
+    parts = []
+    for sl in (slice(0, half), slice(half, n)):
+        wh = w.detach().clone().requires_grad_(True)
+        tp(x.detach()[sl], y.detach()[sl], wh).backward(g[sl])
+        parts.append(wh.grad.double())
+    errs["dW"] = float(((parts[0] + parts[1]) - w.grad.double()).abs().max() / w.grad.double().abs().max())
+    print(f"n={n} rows sampled={rows.size} {errs}", flush=True)
+    for k, v in errs.items():
+        assert v <= FP32_TOL, f"{k}: relative error {v:.3e}"
+
+
 def test_uvw_unsupported_cases_raise(cuda):
     import openequivariance_amd as oeq
     for shared in (True, False):
