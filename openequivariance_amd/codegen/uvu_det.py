@@ -23,6 +23,8 @@ kernel reads both at the unpermuted position: templates/loop_unroll_conv_det.cuh
 """
 from __future__ import annotations
 
+import os
+
 from ..problem import TPProblem
 from .common import Emitter, WAVE
 from .uvu_direct import UVUDirectGenerator
@@ -41,18 +43,24 @@ class UVUDetGenerator(UVUDirectGenerator):
         # (pointers | cursors | position list | dY partials) instead of the caller's transpose permutation
         # (receiver pointers | sender pointers | dY partials)
         self.backward_perm = backward_perm
+        # the backward launches the nodes in descending order of their edge count (order_backward writes
+        # the node list behind the pointers): with two launch rounds of wavefronts the long nodes then
+        # run first and the short ones fill the tail
+        self.ordered_backward = os.environ.get("OEQ_AMD_DET_ORDER", "1") != "0"
+        extra = " + node_count" if self.ordered_backward else ""
         if backward_perm:
             self.bwd_ptr_off = "0"
             self.bwd_list = "((const i64*)ws + 2 * (node_count + 1))"
-            self.dypart_off = "(2 * (node_count + 1) + nnz) * sizeof(i64)"
+            self.bwd_order = "((const i64*)ws + 2 * (node_count + 1) + nnz)"
+            self.dypart_off = f"(2 * (node_count + 1) + nnz{extra}) * sizeof(i64)"
         else:
             self.bwd_ptr_off = "(node_count + 1)"
             self.bwd_list = "tperm"
-            self.dypart_off = "2 * (node_count + 1) * sizeof(i64)"
+            self.bwd_order = "((const i64*)ws + 2 * (node_count + 1))"
+            self.dypart_off = f"(2 * (node_count + 1){extra}) * sizeof(i64)"
         # fetch the next edge's operands while the current edge is being computed; pays when the
         # per-edge register footprint is small enough to keep several wavefronts per SIMD
         words = sum(self.out[i].D for i in self.used_out) + len(self.paths) + len(self.used_y)
-        import os
         env = os.environ.get("OEQ_AMD_DET_PREFETCH")          # "0" / "1": tuning override for A/B runs
         if prefetch_backward is None and env in ("0", "1"):
             prefetch_backward = (env == "1")
@@ -86,14 +94,18 @@ class UVUDetGenerator(UVUDirectGenerator):
         return "u"
 
     # ------------------------------------------------------------------ common
-    def _node_setup(self, E: Emitter, ptr_off: str) -> None:
+    def _node_setup(self, E: Emitter, ptr_off: str, order: str = None) -> None:
         """One node per wavefront.  With multiplicity <= 32 the wavefront's R = 64/P lane groups walk
         interleaved sub-lists of the node's edges (edge beg + it*R + sub) and their partial sums are
         combined in a fixed order at the end, which shortens the serial edge loop R-fold."""
         R = self.R
         E("const int c = blockIdx.y; (void)c;")
         E(f"const int u = c * {self.P} + ul;")
-        E("const u64 node = blockIdx.x;")
+        if order:
+            E(f"const i64 nd_ = blockIdx.x < node_count ? {order}[blockIdx.x] : -1;")
+            E("const u64 node = nd_ >= 0 ? (u64)nd_ : node_count;")
+        else:
+            E("const u64 node = blockIdx.x;")
         E("const bool nv = node < node_count;")
         E(f"const i64* __restrict__ ptr = (const i64*)ws + {ptr_off};")
         E("i64 beg = 0, end = 0;")
@@ -126,11 +138,26 @@ class UVUDetGenerator(UVUDirectGenerator):
         base = "nv" if self.R == 1 else "(nv && sub == 0)"
         return base if self.full(blk) else f"({base} && u < {blk.mul})"
 
+    ORDER_THREADS = 1024
+    ORDER_BINS = 256
+
+    def order_step(self) -> dict:
+        return dict(kernel="order_backward", num_threads=self.ORDER_THREADS, grid_kind=0, num_blocks=1)
+
+    def order_bytes(self, nodes: int) -> int:
+        return nodes * 8 if self.ordered_backward else 0
+
     def plan(self):
-        fwd, bwd, ws = super().plan()
+        fwd, bwd, ws0 = super().plan()
         for s in fwd + bwd:
             if s["kernel"] in ("forward", "backward"):
                 s["work_per_block"] = 1
+        if self.ordered_backward:
+            at = [s["kernel"] for s in bwd].index("backward")
+            bwd.insert(at, self.order_step())
+
+        def ws(nnz=0, nodes=0):
+            return ws0(nnz, nodes) + self.order_bytes(nodes)
         return fwd, bwd, ws
 
     # ================================================================= forward
@@ -385,7 +412,7 @@ class UVUDetGenerator(UVUDirectGenerator):
     def conv_det_backward_body(self) -> str:
         E = Emitter()
         self.emit_lane_direct(E, lds=False)
-        self._node_setup(E, self.bwd_ptr_off)
+        self._node_setup(E, self.bwd_ptr_off, self.bwd_order if self.ordered_backward else None)
         E(f"const i64* __restrict__ elist = {self.bwd_list};     // edge ids in (sender, ...) order")
         self._cur_c = "e"
         # this node's own X chunk (fixed over the edge loop)

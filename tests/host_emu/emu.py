@@ -70,6 +70,7 @@ static inline void oeq_block_sync() { pthread_barrier_wait(&g_bar); }
 static inline void oeq_sched_fence() {}
 static inline void __syncthreads() { pthread_barrier_wait(&g_bar); }
 #define __HIP_MEMORY_SCOPE_AGENT 0
+#define __HIP_MEMORY_SCOPE_WORKGROUP 0
 template <class V> static inline V __hip_atomic_fetch_add(V* p, V v, int, int) { std::lock_guard<std::mutex> g(g_atomic_mutex); V o = *p; *p += v; return o; }
 // matrix-core step of one wavefront, emulated collectively by its 64 threads
 struct V4 { T v[4]; T& operator[](int i) { return v[i]; } const T& operator[](int i) const { return v[i]; } };
@@ -198,6 +199,9 @@ CONV_EXTRA_DET = r"""
         else if (k == "prep_forward") FWD_CALL(prep_forward);
         else if (k == "prep_backward") BWD_CALL(prep_backward);
 """
+CONV_EXTRA_ORDER = r"""
+        else if (k == "order_backward") BWD_CALL(order_backward);
+"""
 CONV_EXTRA_SORTED = r"""
         else if (k == "group_clear") FWD_CALL(group_clear);
         else if (k == "group_count") FWD_CALL(group_count);
@@ -286,12 +290,16 @@ def run_conv(gen, steps: Sequence[Dict], X, Y, W, rows, cols, G=None, tperm=None
     extra = ""
     if gen.kind == "conv_det":
         extra += CONV_EXTRA_DET
+        if gen.ordered_backward:
+            extra += CONV_EXTRA_ORDER
         if gen.NCH > 1:
             extra += CONV_EXTRA_DYRED
     elif hasattr(gen, "fwd"):
         extra += CONV_EXTRA_SORTED
         if gen.grouped_backward:
             extra += CONV_EXTRA_GROUPED_BWD
+            if gen.bwd.ordered_backward:
+                extra += CONV_EXTRA_ORDER
             if gen.bwd.NCH > 1:
                 extra += CONV_EXTRA_DYRED
     exe = build(gen.render(prelude=emu_prelude(gen.T)), CONV_MAIN.replace("@EXTRA@", extra))

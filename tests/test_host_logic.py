@@ -43,8 +43,9 @@ def test_launch_plans():
     g = UVUDetGenerator(prob)
     fwd, bwd, ws = g.plan()
     assert [s["kernel"] for s in fwd] == ["prep_forward", "forward"] and fwd[1]["grid_y"] == 4
-    assert [s["kernel"] for s in bwd] == ["prep_backward", "backward", "backward_dy_reduce"]
-    assert ws(1000, 10) == 2 * 11 * 8 + 4 * 1000 * 16 * 4
+    assert [s["kernel"] for s in bwd] == ["prep_backward", "order_backward", "backward", "backward_dy_reduce"]
+    assert bwd[1]["num_blocks"] == 1
+    assert ws(1000, 10) == 2 * 11 * 8 + 10 * 8 + 4 * 1000 * 16 * 4       # pointers | node order | dY partials
     prob, _ = common.fully_connected(common.DENSE)
     fwd, bwd, ws = UVWGenerator(prob).plan()
     assert [s["kernel"] for s in bwd] == ["prep_backward", "backward", "backward_dw", "backward_reduce"]
@@ -133,9 +134,9 @@ def test_unsorted_conv_backward_selection(monkeypatch):
     assert ws(1000, 10) == (2 * 11 + 1000) * 8
     _, bwd, ws = large.plan()
     assert [s["kernel"] for s in bwd] == ["group_clear_backward", "group_count_backward", "group_scan_backward",
-                                          "group_fill_backward", "backward", "backward_dy_reduce"]
-    assert bwd[4]["grid_y"] == 4 and bwd[4]["work_per_block"] == 1
-    assert ws(1000, 10) == (2 * 11 + 1000) * 8 + 4 * 1000 * 16 * 4
+                                          "group_fill_backward", "order_backward", "backward", "backward_dy_reduce"]
+    assert bwd[5]["grid_y"] == 4 and bwd[5]["work_per_block"] == 1
+    assert ws(1000, 10) == (2 * 11 + 1000 + 10) * 8 + 4 * 1000 * 16 * 4
     src = large.render()
     for name in ("group_fill_backward", "backward_dy_reduce", "void backward("):
         assert name in src
