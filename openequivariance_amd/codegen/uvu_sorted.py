@@ -34,7 +34,7 @@ class UVUSortedGenerator:
     SCAN_THREADS = 1024
 
     # dX values per edge from which the grouped backward is used (measured: 288 per edge - atomic 202 us,
-    # grouped 209 us; 2304 per edge - atomic 9.1 ms, grouped 7.7 ms)
+    # grouped 200 us, a tie; 2304 per edge - atomic 9.1 ms, grouped 7.7 ms)
     ATOMIC_BACKWARD_MAX_D1 = 1024
 
     def __init__(self, problem: TPProblem, vector_stores: bool = True, grouped_backward=None):
