@@ -40,8 +40,8 @@ class UVUDetGenerator(UVUDirectGenerator):
         # the fly from an unsorted edge list) instead of the edge list itself
         self.forward_perm = forward_perm
         # True: the backward likewise walks a sender-grouped order built in the workspace
-        # (pointers | cursors | position list | dY partials) instead of the caller's transpose permutation
-        # (receiver pointers | sender pointers | dY partials)
+        # (pointers | cursors | position list | node order | dY partials) instead of the caller's transpose
+        # permutation (receiver pointers | sender pointers | node order | dY partials)
         self.backward_perm = backward_perm
         # the backward launches the nodes in descending order of their edge count (order_backward writes
         # the node list behind the pointers): with two launch rounds of wavefronts the long nodes then
