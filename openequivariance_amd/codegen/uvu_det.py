@@ -23,6 +23,7 @@ kernel reads both at the unpermuted position: templates/loop_unroll_conv_det.cuh
 """
 from __future__ import annotations
 
+import contextlib
 import os
 
 from ..problem import TPProblem
@@ -32,6 +33,7 @@ from .uvu_direct import UVUDirectGenerator
 
 class UVUDetGenerator(UVUDirectGenerator):
     _allow_det = True
+    SPLIT_WORDS = 80
 
     def __init__(self, problem: TPProblem, prefetch_backward=None, vector_stores: bool = True,
                  forward_perm: bool = False, backward_perm: bool = False):
@@ -58,9 +60,29 @@ class UVUDetGenerator(UVUDirectGenerator):
             self.bwd_list = "tperm"
             self.bwd_order = "((const i64*)ws + 2 * (node_count + 1))"
             self.dypart_off = f"(2 * (node_count + 1){extra}) * sizeof(i64)"
+        # Backward: registers per edge = dZ records + weights + Y ("words").  Above SPLIT_WORDS the
+        # kernel would not fit two wavefronts per SIMD even without prefetch, so the output blocks of a
+        # chunk are split into H groups, one backward launch per group (each launch reads only its blocks of
+        # dZ and W; launch 0 writes dX, the later ones add to it; dY goes through per-(chunk, group) partials).
+        def words_of(outs):
+            ps = [p for p in self.paths if p.o.idx in outs]
+            return (sum(self.out[i].D for i in outs) + sum(p.mv for p in ps)
+                    + len({p.b.off + v * p.b.D + j for p in ps for v in range(p.mv) for (_, j) in p.pairs}))
+        words = words_of(self.used_out)
+        H = 1
+        split_env = os.environ.get("OEQ_AMD_DET_SPLIT", "")           # "0": never; a number: threshold for A/B runs
+        limit = int(split_env) if split_env.isdigit() and split_env != "0" else self.SPLIT_WORDS
+        if words > limit and split_env != "0":
+            H = min(len(self.used_out), -(-words // 64))
+        self.out_groups = [[] for _ in range(H)]
+        for oi in sorted(self.used_out, key=lambda i: -(self.out[i].D + len(self.paths_into(i)))):
+            min(self.out_groups, key=words_of).append(oi)
+        self.out_groups = [sorted(g_) for g_ in self.out_groups]
+        self.H = H
+        self.dy_slots = self.NCH * H               # dY partial rows per edge (summed by backward_dy_reduce)
+        words = max(words_of(g_) for g_ in self.out_groups)
         # fetch the next edge's operands while the current edge is being computed; pays when the
         # per-edge register footprint is small enough to keep several wavefronts per SIMD
-        words = sum(self.out[i].D for i in self.used_out) + len(self.paths) + len(self.used_y)
         env = os.environ.get("OEQ_AMD_DET_PREFETCH")          # "0" / "1": tuning override for A/B runs
         if prefetch_backward is None and env in ("0", "1"):
             prefetch_backward = (env == "1")
@@ -71,11 +93,11 @@ class UVUDetGenerator(UVUDirectGenerator):
         self.stage_words = WAVE * (sum(self.dma_stride(w) for i in self.used_out for _, w in self.dma_pieces(self.out[i].D))
                                    + sum(p.mv for p in self.paths) + 1)
         env = os.environ.get("OEQ_AMD_DET_LDS")
-        fits = (self.T == "float" and self.P >= self.D2 and self.prefetch_backward
-                and 12 * self.stage_words * 4 <= 160 * 1024)
+        stage_waves = (160 * 1024) // (4 * self.stage_words * 4)        # wavefronts per SIMD the stage leaves room for
+        fits = self.T == "float" and self.P >= self.D2 and self.NCH == 1 and H == 1 and stage_waves >= 2
         self.lds_backward = fits and env != "0"
         if self.lds_backward:
-            self.waves_per_eu = 3
+            self.waves_per_eu = min(3, stage_waves)
         # the forward likewise when the multiplicity fits one chunk: few wavefronts per node, so the
         # registers saved buy a fifth wavefront per SIMD (with several chunks per node it measured 1 % slower)
         fwd_words = self._forward_slabs()[1]
@@ -83,6 +105,24 @@ class UVUDetGenerator(UVUDirectGenerator):
                             and 16 * (fwd_words + self.lds_elems) * 4 <= 160 * 1024)
         self.uniform_rows = False          # validity is per lane (edge lists differ between sub-rows)
         self.chunk_in_grid = True
+
+    @contextlib.contextmanager
+    def _group(self, h: int):
+        """Restricts the generator to the paths into the output blocks of group h (backward launches)."""
+        saved = (self.paths, self.used_out, self.used_in1, self.used_y)
+        outs = self.out_groups[h]
+        self.paths = [p for p in saved[0] if p.o.idx in outs]
+        self.used_out = list(outs)
+        self.used_in1 = sorted({p.a.idx for p in self.paths})
+        self.used_y = sorted({p.b.off + v * p.b.D + j for p in self.paths for v in range(p.mv) for (_, j) in p.pairs})
+        try:
+            yield
+        finally:
+            self.paths, self.used_out, self.used_in1, self.used_y = saved
+
+    def backward_kernels(self):
+        """(kernel name, group) of the backward launches, in launch order."""
+        return [("backward" if h == 0 else f"backward_g{h}", h) for h in range(self.H)]
 
     def act(self, blk):
         return "rv" if self.full(blk) else f"(rv && u < {blk.mul})"
@@ -147,17 +187,28 @@ class UVUDetGenerator(UVUDirectGenerator):
     def order_bytes(self, nodes: int) -> int:
         return nodes * 8 if self.ordered_backward else 0
 
+    def backward_steps(self):
+        """Launches of the segmented backward behind the pointer / position-list preparation."""
+        steps = [self.order_step()] if self.ordered_backward else []
+        steps += [dict(kernel=name, num_threads=64, grid_kind=2, work_per_block=1, grid_y=self.NCH)
+                  for name, _ in self.backward_kernels()]
+        if self.dy_slots > 1:
+            steps.append(dict(kernel="backward_dy_reduce", num_threads=256, grid_kind=1,
+                              work_per_block=self.dy_rows_per_block))
+        return steps
+
+    def dy_partial_bytes(self, nnz: int) -> int:
+        return self.dy_slots * nnz * self.D2 * self.itemsize if self.dy_slots > 1 else 0
+
     def plan(self):
-        fwd, bwd, ws0 = super().plan()
-        for s in fwd + bwd:
-            if s["kernel"] in ("forward", "backward"):
+        fwd, bwd, _ = super().plan()
+        for s in fwd:
+            if s["kernel"] == "forward":
                 s["work_per_block"] = 1
-        if self.ordered_backward:
-            at = [s["kernel"] for s in bwd].index("backward")
-            bwd.insert(at, self.order_step())
+        bwd = [s for s in bwd if s["kernel"] == "prep_backward"] + self.backward_steps()
 
         def ws(nnz=0, nodes=0):
-            return ws0(nnz, nodes) + self.order_bytes(nodes)
+            return 2 * (nodes + 1) * 8 + self.order_bytes(nodes) + self.dy_partial_bytes(nnz)
         return fwd, bwd, ws
 
     # ================================================================= forward
@@ -409,7 +460,11 @@ class UVUDetGenerator(UVUDirectGenerator):
             E("}")
 
     # ================================================================ backward
-    def conv_det_backward_body(self) -> str:
+    def conv_det_backward_body(self, grp: int = 0) -> str:
+        with self._group(grp):
+            return self._backward_body(grp)
+
+    def _backward_body(self, grp: int) -> str:
         E = Emitter()
         self.emit_lane_direct(E, lds=False)
         self._node_setup(E, self.bwd_ptr_off, self.bwd_order if self.ordered_backward else None)
@@ -488,15 +543,15 @@ class UVUDetGenerator(UVUDirectGenerator):
                 return
             writer = "ul == 0" if self.P < 64 else "lane == 63"
             E(f"if (rv && {writer}) {{")
-            if self.NCH > 1:
-                E(f"    T* __restrict__ Ygr = (T*)((char*)ws + DYPART_OFF) + ((u64)c * nnz + e) * {self.D2};")
+            if self.dy_slots > 1:
+                E(f"    T* __restrict__ Ygr = (T*)((char*)ws + DYPART_OFF) + ((u64)(c * {self.H} + {grp}) * nnz + e) * {self.D2};")
             else:
                 E(f"    T* __restrict__ Ygr = Yg + e * {self.D2};")
             for f in range(self.D2):
                 E(f"    Ygr[{f}] = " + (f"dy{f};" if f in self.used_y else "(T)0;"))
             E("}")
         if self.lds_backward:
-            self._emit_staged_backward(E, compute)
+            self._emit_staged_backward(E, compute, grp)
         else:
             self.emit_pingpong_loop(E, names, load_idx, load, compute, prefetch_first=self.prefetch_backward)
         E("rv = nv;")
@@ -507,8 +562,11 @@ class UVUDetGenerator(UVUDirectGenerator):
             if a.idx in self.used_in1:
                 dxs = [f"dx{a.idx}_{m}" for m in range(a.D)]
                 self.emit_sub_sum(E, dxs)
+                if grp > 0:            # the launches of the earlier groups have written this row: add to it
+                    E(f"if ({self.store_act(a)}) {{ const T* __restrict__ q_ = {dst}; "
+                      + " ".join(f"dx{a.idx}_{m} += q_[{m}];" for m in range(a.D)) + " }")
                 self.emit_record_store(E, dxs, dst, self.store_act(a))
-            else:
+            elif grp == 0:
                 self.emit_record_store(E, ["(T)0"] * a.D, dst, self.store_act(a))
         return E.text()
 
@@ -569,7 +627,7 @@ class UVUDetGenerator(UVUDirectGenerator):
                 E("const T " + ", ".join(f"x{i}_{m} = a{i}_ ? xr{i}_{m} : (T)0" for m in range(a.D)) + ";")
         self.emit_staged_loop(E, self.edge_pos, "eperm" if self.forward_perm else None, "cols", dma, readback, compute)
 
-    def _emit_staged_backward(self, E: Emitter, compute) -> None:
+    def _emit_staged_backward(self, E: Emitter, compute, grp: int = 0) -> None:
         """Stage layout (words): per transfer a [64 lanes x lane stride] slab in lane order - the dZ records
         of every output block, one word per path weight, and one slab whose lane (sub, f) holds Y[e_sub][f]."""
         nt = 2 if self.nontemporal else 0          # cache policy bit "nt" for the streamed operands
@@ -634,8 +692,8 @@ class UVUDetGenerator(UVUDirectGenerator):
                     E(f"if ({self.act(p.a)}) {self.st('Wgr', self.widx(p, 'u', v), f'pw_{p.t}_{v}')}")
             writer = "ul == 0" if self.P < 64 else "lane == 63"
             E(f"if (rv && {writer}) {{")
-            if self.NCH > 1:
-                E(f"    T* __restrict__ Ygr = (T*)((char*)ws + DYPART_OFF) + ((u64)c * nnz + e) * {self.D2};")
+            if self.dy_slots > 1:
+                E(f"    T* __restrict__ Ygr = (T*)((char*)ws + DYPART_OFF) + ((u64)(c * {self.H} + {grp}) * nnz + e) * {self.D2};")
             else:
                 E(f"    T* __restrict__ Ygr = Yg + e * {self.D2};")
             for f in range(self.D2):

@@ -82,14 +82,8 @@ class UVUSortedGenerator:
                dict(kernel="group_count_backward", num_threads=256, grid_kind=ROW, work_per_block=256),
                dict(kernel="group_scan_backward", num_threads=self.SCAN_THREADS, grid_kind=FIXED, num_blocks=1),
                dict(kernel="group_fill_backward", num_threads=256, grid_kind=ROW, work_per_block=256)]
-        if b.ordered_backward:
-            bwd.append(b.order_step())
-        bwd.append(dict(kernel="backward", num_threads=64, grid_kind=NODE, work_per_block=1, grid_y=b.NCH))
-        if b.NCH > 1:
-            bwd.append(dict(kernel="backward_dy_reduce", num_threads=256, grid_kind=ROW,
-                            work_per_block=b.dy_rows_per_block))
+        bwd += b.backward_steps()
 
         def ws(nnz=0, nodes=0):
-            return ((2 * (nodes + 1) + nnz) * 8 + b.order_bytes(nodes)
-                    + (b.NCH * nnz * b.D2 * b.itemsize if b.NCH > 1 else 0))
+            return (2 * (nodes + 1) + nnz) * 8 + b.order_bytes(nodes) + b.dy_partial_bytes(nnz)
         return fwd, bwd, ws

@@ -24,6 +24,8 @@ MACE = ("128x0e+128x1o+128x2e", "1x0e+1x1o+1x2e+1x3o", "128x0e+128x1o+128x2e+128
 # the same inputs with every triangle-allowed output kept, also the unnatural parities 1e, 2o, 3e
 MACE_ALL = ("128x0e+128x1o+128x2e", "1x0e+1x1o+1x2e+1x3o", "128x0e+128x1o+128x1e+128x2e+128x2o+128x3o+128x3e")
 NEQUIP = ("32x0e+32x1o+32x2e", "1x0e+1x1o+1x2e", "32x0e+32x1o+32x2e")
+NEQUIP_ALL = ("32x0e+32x1o+32x2e", "1x0e+1x1o+1x2e", "32x0e+32x1o+32x1e+32x2e+32x2o")
+LARGE_ALL = ("256x0e+256x1o+256x2e", "1x0e+1x1o+1x2e+1x3o", "256x0e+256x1o+256x1e+256x2e+256x2o")
 LARGE = ("256x0e+256x1o+256x2e", "1x0e+1x1o+1x2e+1x3o", "256x0e+256x1o+256x2e")
 DENSE = ("64x0e+64x1o+64x2e", "1x0e+1x1o+1x2e", "64x0e+64x1o+64x2e")
 
@@ -231,6 +233,24 @@ def get(name: str) -> Workload:
                         + ("deterministic" if det else "atomic"),
                         "conv", LARGE, 800000, "edges/s", "hbm", "f32", 12349,
                         {"nodes": 20000, "paths": 13, "deterministic": det}, nodes=20000, deterministic=det, sh_lmax=3)
+    if name in ("mace_conv_det", "mace_conv_atomic"):
+        det = name.endswith("det")
+        return Workload(name, "MACE-style fused uvu conv (the problem of the tensor-product benchmark as a convolution), "
+                        "128x0e+128x1o+128x2e (x) SH(lmax 3) -> l3<=3, 17 paths, 10000 nodes, 300000 edges, fp32, "
+                        "forward+backward, " + ("deterministic (receiver-sorted)" if det else "unsorted"),
+                        "conv", MACE, 300000, "edges/s", "hbm", "f32", 12350,
+                        {"nodes": 10000, "paths": 17, "deterministic": det}, nodes=10000, deterministic=det, sh_lmax=3)
+    if name == "nequip_conv_det_all_parities":
+        return Workload(name, "fused uvu conv, 32x0e+32x1o+32x2e (x) SH(lmax 2) -> every triangle-allowed l3<=2 of either "
+                        "parity, 15 paths, 5000 nodes, 150000 edges, fp32, forward+backward, deterministic (receiver-sorted)",
+                        "conv", NEQUIP_ALL, 150000, "edges/s", "hbm", "f32", 12347,
+                        {"nodes": 5000, "paths": 15, "deterministic": True}, nodes=5000, deterministic=True, sh_lmax=2)
+    if name == "large_conv_det_all_parities":
+        return Workload(name, "large fused uvu conv, 256x0e+256x1o+256x2e (x) SH(lmax 3) -> every triangle-allowed l3<=2 of "
+                        "either parity, 18 paths, 20000 nodes, Poisson(40) in-degree (~800000 edges), fp32, "
+                        "forward+backward, deterministic",
+                        "conv", LARGE_ALL, 800000, "edges/s", "hbm", "f32", 12349,
+                        {"nodes": 20000, "paths": 18, "deterministic": True}, nodes=20000, deterministic=True, sh_lmax=3)
     if name in ("dense_uvw_f32", "dense_uvw_f64"):
         dt = "f32" if name.endswith("f32") else "f64"
         w = Workload(name, "dense uvw TP with shared weights, 64x0e+64x1o+64x2e (x) SH(lmax 2) -> 64x0e+64x1o+64x2e, "

@@ -288,20 +288,22 @@ def run_tp(gen, steps: Sequence[Dict], X, Y, W, G=None, ws_bytes: int = 0):
 def run_conv(gen, steps: Sequence[Dict], X, Y, W, rows, cols, G=None, tperm=None, ws_bytes: int = 0):
     dt = np.float32 if gen.T == "float" else np.float64
     extra = ""
+    det = None
     if gen.kind == "conv_det":
         extra += CONV_EXTRA_DET
-        if gen.ordered_backward:
-            extra += CONV_EXTRA_ORDER
-        if gen.NCH > 1:
-            extra += CONV_EXTRA_DYRED
+        det = gen
     elif hasattr(gen, "fwd"):
         extra += CONV_EXTRA_SORTED
         if gen.grouped_backward:
             extra += CONV_EXTRA_GROUPED_BWD
-            if gen.bwd.ordered_backward:
-                extra += CONV_EXTRA_ORDER
-            if gen.bwd.NCH > 1:
-                extra += CONV_EXTRA_DYRED
+            det = gen.bwd
+    if det is not None:
+        if det.ordered_backward:
+            extra += CONV_EXTRA_ORDER
+        for name, h in det.backward_kernels()[1:]:
+            extra += f'        else if (k == "{name}") BWD_CALL({name});\n'
+        if det.dy_slots > 1:
+            extra += CONV_EXTRA_DYRED
     exe = build(gen.render(prelude=emu_prelude(gen.T)), CONV_MAIN.replace("@EXTRA@", extra))
     nodes, nnz = X.shape[0], rows.shape[0]
     with tempfile.TemporaryDirectory() as d:

@@ -68,6 +68,32 @@ def test_ragged_conv(cuda, deterministic):
     _run(prob, oprob, 50, 333, 34, deterministic)
 
 
+@pytest.mark.parametrize("deterministic", [False, True])
+@pytest.mark.parametrize("which", ["nequip", "large"])
+def test_conv_outputs_of_either_parity(cuda, which, deterministic):
+    """The literal reading of the benchmark configurations 3 and 5: every triangle-allowed l3 <= 2 with the
+    output parity p1 * p2, which adds the 1e and 2o outputs (15 and 18 paths)."""
+    from openequivariance_amd import workloads
+    irreps = workloads.NEQUIP_ALL if which == "nequip" else workloads.LARGE_ALL
+    prob, oprob = common.channelwise(irreps)
+    assert len(prob.instructions) == (15 if which == "nequip" else 18)
+    if which == "nequip":
+        _run(prob, oprob, 200, 5000, 37, deterministic, sh_lmax=2)
+    else:
+        _run(prob, oprob, 30, 400, 38, deterministic, sh_lmax=3)
+
+
+@pytest.mark.parametrize("deterministic", [False, True])
+def test_mace_conv_backward_split_over_output_blocks(cuda, deterministic):
+    """The MACE problem as a convolution: 104 registers of operands per edge, so the backward runs as two
+    launches over two groups of output blocks (the second adds to dX; dY through per-group partials)."""
+    from openequivariance_amd.conv import select_conv_generator
+    prob, oprob = common.channelwise(common.MACE)
+    gen = select_conv_generator(prob, True)
+    assert gen.H == 2 and sorted(sum(gen.out_groups, [])) == gen.used_out
+    _run(prob, oprob, 60, 900, 39, deterministic, sh_lmax=3)
+
+
 STAGED_SHAPES = {
     "mul16_four_sublists": ("16x0e+16x1o", "1x0e+1x1o+1x2e", "16x0e+16x1o+16x2e"),
     "mul8_eight_sublists": ("8x0e+8x1o", "1x0e+1x1o", "8x0e+8x1o"),

@@ -140,3 +140,23 @@ def test_unsorted_conv_backward_selection(monkeypatch):
     src = large.render()
     for name in ("group_fill_backward", "backward_dy_reduce", "void backward("):
         assert name in src
+
+
+def test_backward_split_over_output_block_groups():
+    """Problems whose per-edge operands exceed 80 registers run the segmented backward as one launch per
+    group of output blocks; the groups partition the output blocks and balance their operand counts."""
+    from openequivariance_amd.codegen.uvu_det import UVUDetGenerator
+    from openequivariance_amd.problem import ChannelwiseTPP
+    large = UVUDetGenerator(ChannelwiseTPP("256x0e+256x1o+256x2e", "1x0e+1x1o+1x2e+1x3o", "256x0e+256x1o+256x2e"))
+    assert large.H == 1 and [k for k, _ in large.backward_kernels()] == ["backward"] and large.dy_slots == 4
+    mace = UVUDetGenerator(ChannelwiseTPP("128x0e+128x1o+128x2e", "1x0e+1x1o+1x2e+1x3o", "128x0e+128x1o+128x2e+128x3o"))
+    assert mace.H == 2 and mace.dy_slots == 4 and mace.prefetch_backward
+    assert sorted(sum(mace.out_groups, [])) == mace.used_out and all(mace.out_groups)
+    _, bwd, ws = mace.plan()
+    assert [s["kernel"] for s in bwd] == ["prep_backward", "order_backward", "backward", "backward_g1", "backward_dy_reduce"]
+    assert ws(1000, 10) == (2 * 11 + 10) * 8 + 4 * 1000 * 16 * 4
+    src = mace.render()
+    assert "void backward_g1(" in src and "c * 2 + 1" in src
+    with mace._group(1):
+        assert {p.o.idx for p in mace.paths} == set(mace.out_groups[1])
+    assert len(mace.paths) == 17                         # restored after the group context
