@@ -15,6 +15,9 @@ computed, either into a second register set (emit_pingpong_loop) or, for fp32 pr
 multiplicity fits one chunk, through LDS by LDS-DMA (emit_staged_loop), which needs one register set
 and so keeps more wavefronts resident.
 
+The backward launches its nodes longest first (order_backward), and when one edge's operands would not
+leave room for two wavefronts per SIMD it runs as one launch per group of output blocks (out_groups).
+
 All loads are unconditional from clamped, range-checked indices (see uvu_direct.py); an edge
 that is out of range for its lane, or names a node that does not exist, contributes zero.  The
 CSR pointers come from the prep kernels of the template (workspace).  The backward reads sender
