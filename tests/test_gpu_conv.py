@@ -140,6 +140,29 @@ def test_isolated_nodes_and_asymmetric_graph(cuda):
         assert float(x.grad[:25].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("deterministic", [False, True])
+def test_star_graph_with_self_loops(cuda, deterministic):
+    """Half of the edges start or end at node 0 (about 750 edges each way: far more than the 255 the
+    launch-order bins distinguish, and hundreds of iterations of the edge pipeline), with self loops and
+    repeated edges."""
+    rng = np.random.default_rng(42)
+    nodes, nnz = 50, 3000
+    rows = rng.integers(0, nodes, nnz)
+    cols = rng.integers(0, nodes, nnz)
+    rows[: nnz // 4] = 0
+    cols[nnz // 4: nnz // 2] = 0
+    cols[-20:] = rows[-20:]                       # self loops
+    rows[-40:-20], cols[-40:-20] = rows[-60:-40], cols[-60:-40]      # repeated edges
+    rows, cols = rows.astype(np.int64), cols.astype(np.int64)
+    tperm = None
+    if deterministic:
+        rows, cols, tperm, _ = otp.coord_graph(rows, cols)
+    prob, oprob = common.channelwise(common.NEQUIP)
+    _run(prob, oprob, nodes, nnz, 43, deterministic, sh_lmax=2, graph=(rows, cols, tperm))
+    prob, oprob = common.channelwise(common.LARGE)
+    _run(prob, oprob, nodes, nnz, 44, deterministic, sh_lmax=3, graph=(rows, cols, tperm))
+
+
 def test_no_edges(cuda):
     import torch
     import openequivariance_amd as oeq
