@@ -141,7 +141,9 @@ class UVUGenerator:
         self.used_out = sorted({p.o.idx for p in self.paths})
         self.used_y = sorted({p.b.off + v * p.b.D + j for p in self.paths for v in range(p.mv) for (_, j) in p.pairs})
 
-        max_mul = max(self.in1[i].mul for i in self.used_in1)
+        # lanes <-> channels over the widest block of X or Z: blocks that no path touches are zero-filled
+        # through the same mapping, so it has to cover them too
+        max_mul = max([b.mul for b in self.in1 if b.dim > 0] + [o.mul for o in self.out if o.dim > 0])
         if max_mul <= 32:
             self.P = next_pow2(max_mul)
             self.R = WAVE // self.P

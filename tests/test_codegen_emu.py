@@ -106,6 +106,25 @@ def test_conv_det_long_edge_lists(staged, monkeypatch):
         assert rel_err(got, ref) < TOL
 
 
+def test_conv_blocks_no_path_touches_are_zero_filled():
+    """in1 holds a 16-channel l = 3 block that no path reads while the blocks in use have one channel: its
+    dX columns must come out as zeros (the emulator starts the deterministic outputs from junk)."""
+    irreps = ("1x0e+1x1o+16x3o", "1x0e+1x1o", "16x0e+16x0o+16x1e+16x1o")
+    prob, oprob = common.channelwise(irreps)
+    g = UVUDetGenerator(prob)
+    assert g.used_in1 == [0, 1] and g.P == 16
+    nodes, nnz = 21, 265
+    rows, cols, tperm, _ = otp.coord_graph(*common.random_graph(nodes, nnz, 2038, self_loops=True))
+    X, Y, W, G = common.conv_inputs(prob, nodes, nnz, 2038)
+    fwd, bwd, ws = g.plan()
+    out = emu.run_conv(g, fwd, X, Y, W, rows, cols, tperm=tperm, ws_bytes=ws(nnz, nodes))
+    assert rel_err(out["Z"], otp.conv_forward(oprob, X, Y, W, rows, cols)) < TOL
+    out = emu.run_conv(g, bwd, X, Y, W, rows, cols, G=G, tperm=tperm, ws_bytes=ws(nnz, nodes))
+    assert not out["Xg"][:, 4:].any()
+    for got, ref in zip((out["Xg"], out["Yg"], out["Wg"]), otp.conv_backward(oprob, X, Y, W, G, rows, cols)):
+        assert rel_err(got, ref) < TOL
+
+
 def test_conv_det_chunked_ragged():
     irreps = ("5x0e+3x1o+70x2e", "1x0e+1x1o+1x2e", "5x0e+3x1o+70x2e+7x3o")
     prob, oprob = common.channelwise(irreps)

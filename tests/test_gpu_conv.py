@@ -95,6 +95,10 @@ def test_mace_conv_backward_split_over_output_blocks(cuda, deterministic):
 
 
 STAGED_SHAPES = {
+    # one full 64-channel list, a single path, D = 1 output: every staged Y read has a constant LDS address,
+    # which the compiler once moved behind the next transfer into the same slab
+    "mul64_single_path_l1": ("64x1o", "1x0e+1x1o+1x2e+1x3o", "64x0e"),
+    "mul64_single_path_l2": ("64x2e", "1x0e+1x1o+1x2e", "64x0e"),
     "mul16_four_sublists": ("16x0e+16x1o", "1x0e+1x1o+1x2e", "16x0e+16x1o+16x2e"),
     "mul8_eight_sublists": ("8x0e+8x1o", "1x0e+1x1o", "8x0e+8x1o"),
     "mul64_one_list": ("64x0e+64x1o", "1x0e+1x1o", "64x0e+64x1o"),
@@ -161,6 +165,15 @@ def test_star_graph_with_self_loops(cuda, deterministic):
     _run(prob, oprob, nodes, nnz, 43, deterministic, sh_lmax=2, graph=(rows, cols, tperm))
     prob, oprob = common.channelwise(common.LARGE)
     _run(prob, oprob, nodes, nnz, 44, deterministic, sh_lmax=3, graph=(rows, cols, tperm))
+
+
+@pytest.mark.parametrize("deterministic", [False, True])
+def test_blocks_no_path_touches(cuda, deterministic):
+    """A wide in1 block that no path reads (and narrow blocks in use): its dX columns are zeros."""
+    irreps = ("1x0e+1x1o+16x3o", "1x0e+1x1o", "16x0e+16x0o+16x1e+16x1o")
+    prob, oprob = common.channelwise(irreps)
+    _, (x, *_rest) = _run(prob, oprob, 21, 265, 2038, deterministic)
+    assert not x.grad[:, 4:].any()
 
 
 def test_no_edges(cuda):

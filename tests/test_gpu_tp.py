@@ -130,6 +130,13 @@ def test_shared_weights_uvu(cuda):
     assert torch.equal(w.grad, w2.grad), "shared-weight dW must be bit-reproducible"
 
 
+def test_blocks_no_path_touches(cuda):
+    """A wide in1 block that no path reads (and narrow blocks in use): its dX columns are zeros."""
+    irreps = ("1x0e+1x1o+16x3o", "1x0e+1x1o", "16x0e+16x0o+16x1e+16x1o")
+    prob, oprob = common.channelwise(irreps)
+    _run(prob, oprob, 300, 51, np.float32)
+
+
 def test_empty_batch(cuda):
     import torch
     import openequivariance_amd as oeq
