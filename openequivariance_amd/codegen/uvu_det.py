@@ -93,11 +93,16 @@ class UVUDetGenerator(UVUDirectGenerator):
         self.nontemporal = os.environ.get("OEQ_AMD_DET_NT", "1") == "1"   # streaming hint on W / Y / dW / dY
         # backward operands of the next edge travel global -> LDS without passing through registers
         # (LDS-DMA), which leaves room for a third wavefront per SIMD; see emit_staged_loop
-        self.stage_words = WAVE * (sum(self.dma_stride(w) for i in self.used_out for _, w in self.dma_pieces(self.out[i].D))
-                                   + sum(p.mv for p in self.paths) + 1)
+        def stage_words_of(outs):
+            return WAVE * (sum(self.dma_stride(w) for i in outs for _, w in self.dma_pieces(self.out[i].D))
+                           + sum(p.mv for p in self.paths if p.o.idx in outs) + 1)
+        self.stage_words = max(stage_words_of(g_) for g_ in self.out_groups)      # of the largest group
         env = os.environ.get("OEQ_AMD_DET_LDS")
         stage_waves = (160 * 1024) // (4 * self.stage_words * 4)        # wavefronts per SIMD the stage leaves room for
-        fits = self.T == "float" and self.P >= self.D2 and self.NCH == 1 and H == 1 and stage_waves >= 2
+        # one chunk per node: also at two wavefronts per SIMD (the register pipeline then has one); chunked
+        # problems only when three fit (config 5, two: 1 % slower than the register pipeline)
+        small = self.NCH == 1 and H == 1
+        fits = self.T == "float" and self.P >= self.D2 and (stage_waves >= 3 or (small and stage_waves >= 2))
         self.lds_backward = fits and env != "0"
         if self.lds_backward:
             self.waves_per_eu = min(3, stage_waves)
@@ -645,7 +650,7 @@ class UVUDetGenerator(UVUDirectGenerator):
                 off += WAVE
         y_off = off
         off += WAVE
-        assert off == self.stage_words
+        assert off <= self.stage_words
         E(f"__shared__ __attribute__((aligned(16))) T stage[{off}];")
 
         def dma(E, e, n):
