@@ -264,5 +264,6 @@ def get(name: str) -> Workload:
     raise KeyError(f"unknown workload {name!r}")
 
 
-ALL = ("readme_uvu", "mace_uvu", "mace_uvu_all_parities", "nequip_conv_atomic", "nequip_conv_det", "dense_uvw_f32", "dense_uvw_f64",
-       "large_conv_det")
+ALL = ("readme_uvu", "mace_uvu", "mace_uvu_all_parities", "nequip_conv_atomic", "nequip_conv_det", "nequip_conv_det_all_parities",
+       "large_conv_det", "large_conv_atomic", "large_conv_det_all_parities", "mace_conv_det", "mace_conv_atomic",
+       "dense_uvw_f32", "dense_uvw_f64")
