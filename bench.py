@@ -6,7 +6,10 @@ A step is one forward and one backward pass of the hot path over one batch of sy
 seeded inputs that already live in HBM.  Prints ONE JSON line.  Besides the whole-job
 throughput (edges/s) it reports, for the dominant kernel, the achieved algorithmic bandwidth
 measured with HIP events around every launch of the timed region, and a CPU baseline (the
-e3nn-equivalent torch implementation on the host cores, on a bounded sample).
+e3nn-equivalent torch implementation on the host cores, on a bounded sample).  Without
+``--workload`` the headline fields are those of ``mace_uvu`` and the key ``workloads`` holds the
+same measurements for every other benchmark configuration (fused convolutions, dense uvw, the
+single-path example), each timed with the same protocol in the same process.
 """
 from __future__ import annotations
 
@@ -30,7 +33,10 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="mace_uvu")
+    ap.add_argument("--workload", default=None,
+                    help="time this workload only (default: mace_uvu as the headline and every other benchmark "
+                         "configuration under the key 'workloads')")
+    ap.add_argument("--headline-only", action="store_true", help="mace_uvu only, without the other configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-cold", action="store_true", help="skip the flushed-cache timing leg")
     ap.add_argument("--cpu-sample", type=int, default=0, help="edges in the CPU sample (0 = automatic)")
@@ -80,7 +86,7 @@ def load_traffic(key):
     return None
 
 
-def cpu_baseline(wl, case, sample):
+def cpu_baseline(wl, case, sample, seconds=10.0):
     """e3nn-equivalent torch implementation on the host cores, forward+backward, fp32, on a
     bounded sample of the same seeded inputs (the op is independent per row/edge, so the rate of
     the sample is the rate of the workload).  This is the only place where the oracle package is
@@ -99,15 +105,15 @@ def cpu_baseline(wl, case, sample):
         W = h["W"] if h["W"].ndim == 1 else h["W"][:n]
         args_ = (h["X"][:n], h["Y"][:n], W, h["G"][:n])
         sec = torch_cpu.time_forward_backward(oprob, *args_, threads=cores, repeats=1)
-        reps = max(1, min(20, int(10.0 / max(sec, 1e-3))))
+        reps = max(1, min(20, int(seconds / max(sec, 1e-3))))
         sec = torch_cpu.time_forward_backward(oprob, *args_, threads=cores, repeats=reps)
         what = f"first {n} rows of the same seeded batch, {reps} repeats"
     else:
-        n = sample or min(wl.units, 5000)
+        n = min(sample or min(wl.units, 5000), h["W"].shape[0])
         rows, cols = h["rows"][:n], h["cols"][:n]
         args_ = (h["X"], h["Y"][:n], h["W"][:n], h["G"])
         sec = torch_cpu.time_forward_backward(oprob, *args_, threads=cores, repeats=1, rows=rows, cols=cols)
-        reps = max(1, min(20, int(10.0 / max(sec, 1e-3))))
+        reps = max(1, min(20, int(seconds / max(sec, 1e-3))))
         sec = torch_cpu.time_forward_backward(oprob, *args_, threads=cores, repeats=reps, rows=rows, cols=cols)
         what = f"first {n} edges of the same seeded graph (all nodes), {reps} repeats"
     return {"value": round(n / sec, 1), "unit": wl.unit, "cores": cores, "kind": "port",
@@ -123,47 +129,94 @@ extern "C" __global__ __launch_bounds__(256) void oeq_copy_calibration(const flo
 """
 
 STREAM_SRC = r"""
-// Streaming probe with a fixed read:write mix: every thread reads NR 16-byte vectors (one from each
-// of NR input streams) and writes NW (one to each of NW output streams), nothing else.
-typedef float v4 __attribute__((ext_vector_type(4)));
-extern "C" __global__ __launch_bounds__(256) void oeq_stream_probe(const v4* __restrict__ in, v4* __restrict__ out, unsigned long long n) {
-    v4 keep = {0.f, 0.f, 0.f, 0.f};
+// Streaming probe with a fixed read:write mix: every thread reads NR vectors (one from each of NR
+// input streams) and writes NW (one to each of NW output streams), nothing else.  VEC = floats per
+// access (2 or 4), NT = 1 for non-temporal accesses; the grid is what the host launches (one element
+// per thread when oversubscribed, a grid-stride loop over few workgroups when persistent).
+typedef float vN __attribute__((ext_vector_type(VEC)));
+static __device__ __forceinline__ vN ld(const vN* p) { return NT ? __builtin_nontemporal_load(p) : *p; }
+static __device__ __forceinline__ void st(vN* p, vN v) { if (NT) __builtin_nontemporal_store(v, p); else *p = v; }
+extern "C" __global__ __launch_bounds__(256) void oeq_stream_probe(const vN* __restrict__ in, vN* __restrict__ out, unsigned long long n) {
+    vN keep = (vN)(0.f);
     for (unsigned long long i = (unsigned long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (unsigned long long)gridDim.x * 256) {
-        v4 acc = {1.f, 2.f, 3.f, 4.f};
+        vN acc = (vN)(1.f);
 #pragma unroll
-        for (int r = 0; r < NR; ++r) acc += __builtin_nontemporal_load(in + r * n + i);
+        for (int r = 0; r < NR; ++r) acc += ld(in + r * n + i);
 #pragma unroll
-        for (int w = 0; w < NW; ++w) __builtin_nontemporal_store(acc, out + w * n + i);
+        for (int w = 0; w < NW; ++w) st(out + w * n + i, acc);
         keep += acc;
     }
     if (NW == 0 && keep.x == 12345.678f) out[0] = keep;       // keeps the loads alive; never true for zero inputs
 }
 """
 
+# (label, non-temporal, floats per access, workgroups: 0 = one element per thread, k = k per compute unit)
+PROBE_VARIANTS = [(f"{'nt' if nt else 'plain'}/{4 * vec}B/{'1 elem per thread' if k == 0 else f'{k} workgroups per CU'}", nt, vec, k)
+                  for nt in (1, 0) for vec in (4, 2) for k in (0, 4, 8, 16)]
 
-def stream_probe(nr, nw, total_bytes=3 << 30, reps=5):
-    """GB/s of a plain streaming kernel that reads ``nr`` and writes ``nw`` 16-byte vectors per
-    thread (best of ``reps`` launches, 3 GiB per launch so that the 256 MiB Infinity Cache does not
-    help): what HBM sustains for this read:write mix, the practical ceiling of a kernel with it."""
+
+def stream_probe(nr, nw, total_bytes=3 << 30, reps=5, variants=None):
+    """Best GB/s over a sweep of plain streaming kernels that read ``nr`` and write ``nw`` vectors per
+    thread (3 GiB per launch, so that the 256 MiB Infinity Cache does not help; best of ``reps``
+    launches per variant): what the memory system sustains for this read:write mix, the practical
+    ceiling of a kernel with it.  The sweep covers temporal / non-temporal accesses, 8- and 16-byte
+    accesses, and oversubscribed / persistent grids; returns (best GB/s, label of the best variant,
+    {label: GB/s})."""
     import ctypes as C
     import torch
     from openequivariance_amd import runtime as rt
-    n = total_bytes // 16 // (nr + nw)
-    src = torch.zeros(max(nr, 1) * n * 4, dtype=torch.float32, device="cuda")
-    dst = torch.empty(max(nw, 1) * n * 4, dtype=torch.float32, device="cuda")
-    mod = rt.Module(rt.compile_source(STREAM_SRC, options=tuple(rt.DEFAULT_OPTIONS) + (f"-DNR={nr}", f"-DNW={nw}")))
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
     stream = torch.cuda.current_stream().cuda_stream
-    args = [C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr()), C.c_uint64(n)]
-    best = float("inf")
-    for r in range(reps + 2):
-        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        a.record()
-        mod.launch("oeq_stream_probe", 32768, 256, args, stream=stream)
-        b.record()
-        b.synchronize()
-        if r >= 2:
-            best = min(best, a.elapsed_time(b))
-    return (nr + nw) * n * 16 / (best * 1e-3) / 1e9
+    n16 = total_bytes // 16 // (nr + nw)
+    src = torch.zeros(max(nr, 1) * n16 * 4, dtype=torch.float32, device="cuda")
+    dst = torch.empty(max(nw, 1) * n16 * 4, dtype=torch.float32, device="cuda")
+    table = {}
+    for label, nt, vec, k in (variants or PROBE_VARIANTS):
+        n = n16 * (4 // vec)
+        grid = (n + 255) // 256 if k == 0 else cus * k
+        if grid >= 2 ** 31:
+            continue
+        opts = tuple(rt.DEFAULT_OPTIONS) + (f"-DNR={nr}", f"-DNW={nw}", f"-DVEC={vec}", f"-DNT={nt}")
+        mod = rt.Module(rt.compile_source(STREAM_SRC, options=opts))
+        args = [C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr()), C.c_uint64(n)]
+        best = float("inf")
+        for r in range(reps + 2):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            mod.launch("oeq_stream_probe", grid, 256, args, stream=stream)
+            b.record()
+            b.synchronize()
+            if r >= 2:
+                best = min(best, a.elapsed_time(b))
+        table[label] = round((nr + nw) * n16 * 16 / (best * 1e-3) / 1e9, 1)
+    top = max(table, key=table.get)
+    return table[top], top, table
+
+
+def torch_stream_reference(total_bytes=3 << 30, reps=5):
+    """The same kind of measurement with torch's own elementwise kernels, as an outside reference:
+    copy_ (1 read : 1 write), add (2 : 1), sum (read only), fill_ (write only)."""
+    import torch
+    out = {}
+
+    def best_ms(fn):
+        best = float("inf")
+        for r in range(reps + 2):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            fn()
+            b.record()
+            b.synchronize()
+            if r >= 2:
+                best = min(best, a.elapsed_time(b))
+        return best
+    n = total_bytes // 4 // 3
+    x, y, z = (torch.zeros(n, dtype=torch.float32, device="cuda") for _ in range(3))
+    out["torch copy_ (1:1)"] = round(2 * n * 4 / (best_ms(lambda: y.copy_(x)) * 1e-3) / 1e9, 1)
+    out["torch add (2:1)"] = round(3 * n * 4 / (best_ms(lambda: torch.add(x, y, out=z)) * 1e-3) / 1e9, 1)
+    out["torch sum (1:0)"] = round(n * 4 / (best_ms(lambda: x.sum()) * 1e-3) / 1e9, 1)
+    out["torch fill_ (0:1)"] = round(n * 4 / (best_ms(lambda: x.fill_(1.0)) * 1e-3) / 1e9, 1)
+    return out
 
 
 def mix_of(read_bytes, write_bytes):
@@ -200,11 +253,118 @@ def copy_calibration(steps):
 
 
 def stream_calibration():
-    """Sustained HBM rate of plain streaming kernels for several read:write mixes."""
-    out = {"workload": "stream_calibration", "unit": "GB/s", "peak": HBM_PEAK_GBS}
-    for nr, nw in ((1, 0), (4, 1), (1, 1), (1, 3), (0, 1)):
-        out[f"read{nr}_write{nw}"] = round(stream_probe(nr, nw), 1)
+    """Sustained rate of plain streaming kernels for several read:write mixes: the whole sweep per
+    mix, its best variant, and torch's own elementwise kernels beside it."""
+    out = {"workload": "stream_calibration", "unit": "GB/s", "peak": HBM_PEAK_GBS, "mixes": {}}
+    for nr, nw in ((1, 0), (4, 1), (3, 1), (2, 1), (1, 1), (1, 3), (0, 1)):
+        best, label, table = stream_probe(nr, nw)
+        out["mixes"][f"read{nr}_write{nw}"] = {"best": best, "best_variant": label, "sweep": table}
+    out["torch"] = torch_stream_reference()
     print(json.dumps(out))
+
+
+def measure(name, steps, warmup, cold=True, cpu=True, cpu_sample=0, ceiling=True, cpu_seconds=10.0):
+    """Build one workload, time ``steps`` forward+backward steps after ``warmup`` untimed ones and
+    return (workload, record): whole-job throughput from the wall clock around the timed region, and
+    the per-direction averages from HIP event pairs recorded around every launch inside it."""
+    import torch
+    from openequivariance_amd import workloads
+    dev = torch.device("cuda:0")
+    wl = workloads.get(name)
+    case = wl.build(dev)                      # operator + device tensors + raw-call closures
+    ev = Events()
+
+    def step(timed):
+        if timed:
+            ev.wrap("forward", case.forward)
+            ev.wrap("backward", case.backward)
+        else:
+            case.forward()
+            case.backward()
+
+    for _ in range(warmup):
+        step(False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step(True)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / steps
+    value = wl.units / (ms_per_step * 1e-3)
+
+    fwd_ms, bwd_ms = ev.mean_ms("forward"), ev.mean_ms("backward")
+    dom = "backward" if bwd_ms >= fwd_ms else "forward"
+    dom_ms = max(fwd_ms, bwd_ms)
+    if wl.bound == "hbm":
+        work, scale = wl.alg_bytes, 1e9
+        peak, unit = HBM_PEAK_GBS, "GB/s"
+    else:
+        work, scale = wl.alg_flops, 1e12
+        peak, unit = (MFMA_FP32_PEAK_TFLOPS if wl.dtype == "f32" else MFMA_FP64_PEAK_TFLOPS), "TFLOP/s"
+    alg = work[dom]
+    achieved = alg / (dom_ms * 1e-3) / scale
+    roofline = {"bound": wl.bound, "kernel": f"{wl.name}:{dom}", "achieved": round(achieved, 2), "peak": peak,
+                "unit": unit, "frac": round(achieved / peak, 4), "traffic": load_traffic(f"{wl.name}:{dom}"),
+                "algorithmic_per_launch": alg, "algorithmic": {"forward": work["forward"], "backward": work["backward"]},
+                "avg_launch_ms": round(dom_ms, 5),
+                "forward_ms": round(fwd_ms, 5), "backward_ms": round(bwd_ms, 5),
+                "fwd_bwd_frac": round((work["forward"] + work["backward"]) / ((fwd_ms + bwd_ms) * 1e-3) / scale / peak, 4),
+                "forward_frac": round(work["forward"] / (fwd_ms * 1e-3) / scale / peak, 4),
+                "backward_frac": round(work["backward"] / (bwd_ms * 1e-3) / scale / peak, 4)}
+
+    if wl.bound == "hbm" and ceiling:
+        # what plain streaming kernels with the dominant kernel's read:write mix sustain on this GPU
+        # (best of a sweep over access width, cache policy and grid shape): the practical ceiling
+        # under the 8 TB/s datasheet peak
+        rd, wr = wl.read_write_split(dom)
+        nr, nw = mix_of(rd, wr)
+        ceil, label, _ = stream_probe(nr, nw)
+        roofline["streaming_ceiling"] = {"mix": f"{nr} reads : {nw} writes", "GB/s": ceil, "variant": label,
+                                         "frac_of_ceiling": round(achieved / ceil, 4)}
+
+    if cold:
+        # second leg, outside the timed region: the same launches with the caches flushed before
+        # each one (a 512 MiB fill, twice the 256 MiB Infinity Cache), the protocol of the reference's
+        # timers (openequivariance/extension/util/backend_hip.hpp:65-99 clears a 100 MB buffer)
+        flush = torch.empty(512 << 20, dtype=torch.uint8, device=dev)
+        for _ in range(min(steps, 30)):
+            flush.fill_(1)
+            ev.wrap("forward_cold", case.forward)
+            flush.fill_(2)
+            ev.wrap("backward_cold", case.backward)
+        torch.cuda.synchronize()
+        del flush
+        fm, fmin = ev.median_min_ms("forward_cold")
+        bm, bmin = ev.median_min_ms("backward_cold")
+        roofline["flushed_caches"] = {
+            "forward_ms_median": round(fm, 5), "forward_ms_min": round(fmin, 5),
+            "backward_ms_median": round(bm, 5), "backward_ms_min": round(bmin, 5),
+            "fwd_bwd_frac": round((work["forward"] + work["backward"]) / ((fm + bm) * 1e-3) / scale / peak, 4)}
+
+    if case.forward_with_prep is not None:
+        # the timed launches reuse the graph preparation left in the workspace, as the layers of a model
+        # do; the same launches including the preparation, for callers that see every graph once
+        for _ in range(min(steps, 10)):
+            ev.wrap("forward_with_prep", case.forward_with_prep)
+            ev.wrap("backward_with_prep", case.backward_with_prep)
+        torch.cuda.synchronize()
+        roofline["with_graph_preparation"] = {"forward_ms": round(ev.mean_ms("forward_with_prep"), 5),
+                                              "backward_ms": round(ev.mean_ms("backward_with_prep"), 5)}
+        case.forward()
+        case.backward()
+
+    rec = {"value": round(value, 1), "unit": wl.unit, "ms_per_step": round(ms_per_step, 5), "dtype": wl.dtype,
+           "data": wl.data_note, "config": {"workload": wl.description, **wl.config}, "roofline": roofline,
+           "cpu_baseline": cpu_baseline(wl, case, cpu_sample, cpu_seconds) if cpu else None}
+    del case
+    torch.cuda.empty_cache()
+    return wl, rec
+
+
+# every BASELINE configuration besides the headline one (config 2 = mace_uvu), and the MACE problem as a convolution
+OTHER_WORKLOADS = ("readme_uvu", "nequip_conv_det", "nequip_conv_atomic", "dense_uvw_f32", "dense_uvw_f64",
+                   "large_conv_det", "large_conv_atomic", "mace_conv_det")
 
 
 def main():
@@ -220,102 +380,43 @@ def main():
               "without communication and is measured on one)", file=sys.stderr)
         sys.exit(2)
 
-    import numpy as np
     import torch
-    import openequivariance_amd as oeq
-    from openequivariance_amd import workloads
-
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
-    dev = torch.device("cuda:0")
-    wl = workloads.get(args.workload)
-    case = wl.build(dev)                      # operator + device tensors + raw-call closures
-    ev = Events()
 
-    def step(timed):
-        if timed:
-            ev.wrap("forward", case.forward)
-            ev.wrap("backward", case.backward)
-        else:
-            case.forward()
-            case.backward()
-
-    for _ in range(args.warmup):
-        step(False)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step(True)
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ms_per_step = wall * 1e3 / args.steps
-    value = wl.units / (ms_per_step * 1e-3)
-
-    fwd_ms, bwd_ms = ev.mean_ms("forward"), ev.mean_ms("backward")
-    dom = "backward" if bwd_ms >= fwd_ms else "forward"
-    dom_ms = max(fwd_ms, bwd_ms)
-    if wl.bound == "hbm":
-        alg = wl.alg_bytes[dom]
-        achieved = alg / (dom_ms * 1e-3) / 1e9
-        peak, unit = HBM_PEAK_GBS, "GB/s"
-    else:
-        alg = wl.alg_flops[dom]
-        achieved = alg / (dom_ms * 1e-3) / 1e12
-        peak, unit = (MFMA_FP32_PEAK_TFLOPS if wl.dtype == "f32" else MFMA_FP64_PEAK_TFLOPS), "TFLOP/s"
-    roofline = {"bound": wl.bound, "kernel": f"{wl.name}:{dom}", "achieved": round(achieved, 2), "peak": peak,
-                "unit": unit, "frac": round(achieved / peak, 4), "traffic": load_traffic(f"{wl.name}:{dom}"),
-                "algorithmic_per_launch": alg, "avg_launch_ms": round(dom_ms, 5),
-                "forward_ms": round(fwd_ms, 5), "backward_ms": round(bwd_ms, 5)}
-    if wl.bound == "hbm":
-        tot = wl.alg_bytes["forward"] + wl.alg_bytes["backward"]
-        roofline["fwd_bwd_frac"] = round(tot / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / peak, 4)
-        roofline["forward_frac"] = round(wl.alg_bytes["forward"] / (fwd_ms * 1e-3) / 1e9 / peak, 4)
-        roofline["backward_frac"] = round(wl.alg_bytes["backward"] / (bwd_ms * 1e-3) / 1e9 / peak, 4)
-    else:
-        tot = wl.alg_flops["forward"] + wl.alg_flops["backward"]
-        roofline["fwd_bwd_frac"] = round(tot / ((fwd_ms + bwd_ms) * 1e-3) / 1e12 / peak, 4)
-
-    if wl.bound == "hbm" and not args.no_cold:
-        # what a plain streaming kernel with the dominant kernel's read:write mix sustains on this
-        # GPU: the practical ceiling under the 8 TB/s datasheet peak
-        rd, wr = wl.read_write_split(dom)
-        nr, nw = mix_of(rd, wr)
-        ceil = stream_probe(nr, nw)
-        roofline["streaming_ceiling"] = {"mix": f"{nr} reads : {nw} writes", "GB/s": round(ceil, 1),
-                                         "frac_of_ceiling": round(achieved / ceil, 4)}
-
-    if not args.no_cold:
-        # second leg, outside the timed region: the same launches with the caches flushed before
-        # each one (a 512 MiB fill, twice the 256 MiB Infinity Cache), the protocol of the reference's
-        # timers (openequivariance/extension/util/backend_hip.hpp:65-99 clears a 100 MB buffer)
-        flush = torch.empty(512 << 20, dtype=torch.uint8, device=dev)
-        for _ in range(min(args.steps, 30)):
-            flush.fill_(1)
-            ev.wrap("forward_cold", case.forward)
-            flush.fill_(2)
-            ev.wrap("backward_cold", case.backward)
-        torch.cuda.synchronize()
-        del flush
-        fm, fmin = ev.median_min_ms("forward_cold")
-        bm, bmin = ev.median_min_ms("backward_cold")
-        work = wl.alg_bytes if wl.bound == "hbm" else wl.alg_flops
-        scale = 1e9 if wl.bound == "hbm" else 1e12
-        roofline["flushed_caches"] = {
-            "forward_ms_median": round(fm, 5), "forward_ms_min": round(fmin, 5),
-            "backward_ms_median": round(bm, 5), "backward_ms_min": round(bmin, 5),
-            "fwd_bwd_frac": round((work["forward"] + work["backward"]) / ((fm + bm) * 1e-3) / scale / peak, 4)}
-
-    cpu = None
-    if not args.no_cpu:
-        cpu = cpu_baseline(wl, case, args.cpu_sample)
-
+    headline = args.workload or "mace_uvu"
+    wl, rec = measure(headline, args.steps, args.warmup, cold=not args.no_cold, cpu=not args.no_cpu,
+                      cpu_sample=args.cpu_sample)
     out = {"metric": "fwd+bwd edges/s and % HBM roofline, MACE-style uvu TP and fused conv",
-           "value": round(value, 1), "unit": wl.unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-           "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak",
-           "vs_baseline": None, "dtype": wl.dtype, "data": "synthetic",
-           "config": {"workload": wl.description, **wl.config},
-           "roofline": roofline, "cpu_baseline": cpu,
+           "value": rec["value"], "unit": rec["unit"], "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+           "ms_per_step": rec["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+           "vs_baseline": None, "dtype": rec["dtype"], "data": rec["data"], "config": rec["config"],
+           "roofline": rec["roofline"], "cpu_baseline": rec["cpu_baseline"],
            "device": torch.cuda.get_device_name(0)}
+    if not args.workload and not args.headline_only:
+        # the other BASELINE configurations, same protocol (same steps and warm-up, HIP events around every
+        # launch), with a shorter CPU leg each
+        others = {}
+        for name in OTHER_WORKLOADS:
+            t0 = time.perf_counter()
+            try:
+                _, r = measure(name, args.steps, args.warmup, cold=not args.no_cold, cpu=not args.no_cpu,
+                               ceiling=False, cpu_seconds=3.0)
+                rf = r["roofline"]
+                others[name] = {"value": r["value"], "unit": r["unit"], "ms_per_step": r["ms_per_step"],
+                                "forward_ms": rf["forward_ms"], "backward_ms": rf["backward_ms"],
+                                "dtype": r["dtype"], "data": r["data"], "config": r["config"], "bound": rf["bound"],
+                                "dominant": rf["kernel"], "frac": rf["frac"], "fwd_bwd_frac": rf["fwd_bwd_frac"],
+                                "forward_frac": rf["forward_frac"], "backward_frac": rf["backward_frac"],
+                                "algorithmic_per_launch": rf["algorithmic"],
+                                "traffic": {"forward": load_traffic(f"{name}:forward"), "backward": load_traffic(f"{name}:backward")},
+                                "flushed_caches": rf.get("flushed_caches"),
+                                "with_graph_preparation": rf.get("with_graph_preparation"), "cpu_baseline": r["cpu_baseline"],
+                                "bench_seconds": None}
+            except Exception as exc:          # one workload failing must not hide the others
+                others[name] = {"error": f"{type(exc).__name__}: {exc}"}
+            others[name]["bench_seconds"] = round(time.perf_counter() - t0, 1)
+        out["workloads"] = others
     print(json.dumps(out))
 
 

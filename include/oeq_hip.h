@@ -62,6 +62,12 @@ int  oeq_hiprtc_version(int* major, int* minor);
 /* One kernel launch of an operator.  Replaces KernelLaunchConfig
  * (extension/util/backend_hip.hpp:123-133) and adds how the grid follows the work size. */
 enum { OEQ_GRID_FIXED = 0, OEQ_GRID_PER_ROW = 1, OEQ_GRID_PER_NODE = 2 };
+/* What a step dereferences and what it is for.  A call whose plan holds a step with
+ * OEQ_STEP_NEEDS_WORKSPACE (OEQ_STEP_NEEDS_TPERM) is rejected, before anything is launched, when the
+ * workspace (transpose permutation) pointer is NULL.  OEQ_STEP_GRAPH_PREP marks the steps that only
+ * derive graph structure (CSR pointers, position lists, node order) from rows / cols /
+ * transpose_perm into the workspace: the *_prepared entry points skip them. */
+enum { OEQ_STEP_NEEDS_WORKSPACE = 1, OEQ_STEP_NEEDS_TPERM = 2, OEQ_STEP_GRAPH_PREP = 4 };
 typedef struct {
     char     kernel[64];        /* extern "C" symbol in the code object */
     uint32_t num_threads;       /* workgroup size */
@@ -71,6 +77,7 @@ typedef struct {
     uint32_t num_blocks;        /* OEQ_GRID_FIXED: the grid; otherwise an upper bound (0 = none) */
     uint32_t grid_y;            /* second grid dimension (0 or 1 = none), e.g. one 64-channel chunk each */
     uint32_t warp_size;         /* informational: 64 */
+    uint32_t flags;             /* OEQ_STEP_* */
 } oeq_step;
 
 /* ------------------------------------------------------ batch tensor product */
@@ -119,6 +126,22 @@ int  oeq_conv_backward(oeq_conv* conv, const void* L1_in, void* L1_grad, const v
                        void* L2_grad, const void* weights, void* weights_grad, const void* L3_grad,
                        const void* rows, const void* cols, uint64_t nnz, uint64_t node_count,
                        void* workspace, const void* transpose_perm, void* stream);
+
+/* The same two calls for a workspace that already holds this graph's preparation: the steps flagged
+ * OEQ_STEP_GRAPH_PREP are skipped.  Valid only if the last oeq_conv_forward (for _forward_prepared) /
+ * oeq_conv_backward (for _backward_prepared) that used this workspace ran with the same rows, cols,
+ * transpose_perm contents, nnz and node_count, and nothing else has written the workspace's
+ * preparation areas since (forward and backward keep theirs in disjoint parts of the workspace).  A
+ * model calls one graph for the forward, the backward and the seven launches of the double backward
+ * of every layer; the reference allocates its workspace once and rebuilds nothing either
+ * (implementations/convolution/ConvolutionBase.py:93-100). */
+int  oeq_conv_forward_prepared(oeq_conv* conv, const void* L1_in, const void* L2_in, const void* weights,
+                               void* L3_out, const void* rows, const void* cols, uint64_t nnz,
+                               uint64_t node_count, void* workspace, const void* transpose_perm, void* stream);
+int  oeq_conv_backward_prepared(oeq_conv* conv, const void* L1_in, void* L1_grad, const void* L2_in,
+                                void* L2_grad, const void* weights, void* weights_grad, const void* L3_grad,
+                                const void* rows, const void* cols, uint64_t nnz, uint64_t node_count,
+                                void* workspace, const void* transpose_perm, void* stream);
 
 /* ------------------------------------------------------------ generic module */
 /* Thin access to a loaded code object, for callers that pack their own arguments

@@ -95,6 +95,8 @@ def _blocks(irreps) -> List[Block]:
 class UVUGenerator:
     """Builds the source text and the launch plan for one uvu problem."""
 
+    idx_ctype = "i64"        # element type of the convolution's index tensors ("int" for int32 callers)
+
     def __init__(self, problem: TPProblem, kind: str = "tp", dw_partials: int = 1024):
         if kind not in ("tp", "conv_atomic", "conv_det"):
             raise ValueError(kind)
@@ -662,9 +664,9 @@ class UVUGenerator:
             fwd = [dict(kernel="forward", num_threads=w, grid_kind=ROW, work_per_block=self.R)]
             bwd = [dict(kernel="backward", num_threads=w, grid_kind=ROW, work_per_block=self.R)]
             return fwd, bwd, (lambda nnz=0, nodes=0: 0)
-        fwd = [dict(kernel="prep_forward", num_threads=256, grid_kind=ROW, work_per_block=256),
+        fwd = [dict(kernel="prep_forward", num_threads=256, grid_kind=ROW, work_per_block=256, prep=True),
                dict(kernel="forward", num_threads=w, grid_kind=NODE, work_per_block=self.R, grid_y=self.NCH)]
-        bwd = [dict(kernel="prep_backward", num_threads=256, grid_kind=ROW, work_per_block=256),
+        bwd = [dict(kernel="prep_backward", num_threads=256, grid_kind=ROW, work_per_block=256, prep=True),
                dict(kernel="backward", num_threads=w, grid_kind=NODE, work_per_block=self.R, grid_y=self.NCH)]
         if self.NCH > 1:
             bwd.append(dict(kernel="backward_dy_reduce", num_threads=256, grid_kind=ROW,

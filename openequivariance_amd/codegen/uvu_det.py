@@ -39,8 +39,9 @@ class UVUDetGenerator(UVUDirectGenerator):
     SPLIT_WORDS = 80
 
     def __init__(self, problem: TPProblem, prefetch_backward=None, vector_stores: bool = True,
-                 forward_perm: bool = False, backward_perm: bool = False):
+                 forward_perm: bool = False, backward_perm: bool = False, idx_ctype: str = "i64"):
         super().__init__(problem, "conv_det", vector_stores=vector_stores)
+        self.idx_ctype = idx_ctype
         # True: the forward walks the receiver-grouped edge order listed in the workspace (built on
         # the fly from an unsorted edge list) instead of the edge list itself
         self.forward_perm = forward_perm
@@ -54,10 +55,13 @@ class UVUDetGenerator(UVUDirectGenerator):
         self.ordered_backward = os.environ.get("OEQ_AMD_DET_ORDER", "1") != "0"
         extra = " + node_count" if self.ordered_backward else ""
         if backward_perm:
-            self.bwd_ptr_off = "0"
-            self.bwd_list = "((const i64*)ws + 2 * (node_count + 1))"
-            self.bwd_order = "((const i64*)ws + 2 * (node_count + 1) + nnz)"
-            self.dypart_off = f"(2 * (node_count + 1) + nnz{extra}) * sizeof(i64)"
+            # behind the forward's grouping (pointers | cursors | position list), so that both stay valid
+            # side by side and a graph prepared once serves forward and backward calls alike
+            base = "(2 * (node_count + 1) + nnz)"
+            self.bwd_ptr_off = base
+            self.bwd_list = f"((const i64*)ws + {base} + 2 * (node_count + 1))"
+            self.bwd_order = f"((const i64*)ws + {base} + 2 * (node_count + 1) + nnz)"
+            self.dypart_off = f"(2 * {base}{extra}) * sizeof(i64)"
         else:
             self.bwd_ptr_off = "(node_count + 1)"
             self.bwd_list = "tperm"
@@ -190,7 +194,7 @@ class UVUDetGenerator(UVUDirectGenerator):
     ORDER_BINS = 256
 
     def order_step(self) -> dict:
-        return dict(kernel="order_backward", num_threads=self.ORDER_THREADS, grid_kind=0, num_blocks=1)
+        return dict(kernel="order_backward", num_threads=self.ORDER_THREADS, grid_kind=0, num_blocks=1, prep=True)
 
     def order_bytes(self, nodes: int) -> int:
         return nodes * 8 if self.ordered_backward else 0
@@ -476,7 +480,8 @@ class UVUDetGenerator(UVUDirectGenerator):
         E = Emitter()
         self.emit_lane_direct(E, lds=False)
         self._node_setup(E, self.bwd_ptr_off, self.bwd_order if self.ordered_backward else None)
-        E(f"const i64* __restrict__ elist = {self.bwd_list};     // edge ids in (sender, ...) order")
+        list_t = "IDX" if self.bwd_list == "tperm" else "i64"
+        E(f"const {list_t}* __restrict__ elist = {self.bwd_list};     // edge ids in (sender, ...) order")
         self._cur_c = "e"
         # this node's own X chunk (fixed over the edge loop)
         E("bool rv = nv;")

@@ -17,7 +17,9 @@ the backward groups the edges by sender in the same way and runs the determinist
 backward over that order.
 
 Workspace: (node_count + 1) group pointers, (node_count + 1) fill cursors and nnz edge positions,
-all int64 (then the per-chunk dY partial sums of the grouped backward), rebuilt on every call.
+all int64, for the forward; behind them the same three arrays of the grouped backward (by sender), its
+node order and its per-chunk dY partial sums.  The two groupings do not overlap, so a workspace
+prepared by one forward and one backward call serves later calls on the same graph unchanged.
 """
 from __future__ import annotations
 
@@ -37,18 +39,19 @@ class UVUSortedGenerator:
     # grouped 200 us, a tie; 2304 per edge - atomic 9.1 ms, grouped 7.7 ms)
     ATOMIC_BACKWARD_MAX_D1 = 1024
 
-    def __init__(self, problem: TPProblem, vector_stores: bool = True, grouped_backward=None):
+    def __init__(self, problem: TPProblem, vector_stores: bool = True, grouped_backward=None, idx_ctype: str = "i64"):
         self.problem = problem
-        self.fwd = UVUDetGenerator(problem, forward_perm=True, vector_stores=vector_stores)
+        self.fwd = UVUDetGenerator(problem, forward_perm=True, vector_stores=vector_stores, idx_ctype=idx_ctype)
         if grouped_backward is None:
             env = os.environ.get("OEQ_AMD_CONV_BACKWARD")            # "grouped" / "atomic": A/B runs
             grouped_backward = (env == "grouped") if env in ("grouped", "atomic") \
                 else self.fwd.D1 >= self.ATOMIC_BACKWARD_MAX_D1
         self.grouped_backward = grouped_backward
         if grouped_backward:
-            self.bwd = UVUDetGenerator(problem, backward_perm=True, vector_stores=vector_stores)
+            self.bwd = UVUDetGenerator(problem, backward_perm=True, vector_stores=vector_stores, idx_ctype=idx_ctype)
         else:
             self.bwd = UVUDirectGenerator(problem, "conv_atomic", vector_stores=vector_stores)
+            self.bwd.idx_ctype = idx_ctype
         self.T = self.fwd.T
         self.D1, self.D2, self.D3, self.WN = self.fwd.D1, self.fwd.D2, self.fwd.D3, self.fwd.WN
         self.NCH = self.fwd.NCH
@@ -66,10 +69,10 @@ class UVUSortedGenerator:
     def plan(self):
         ROW, NODE, FIXED = 1, 2, 0
         f = self.fwd
-        fwd = [dict(kernel="group_clear", num_threads=256, grid_kind=NODE, work_per_block=256),
-               dict(kernel="group_count", num_threads=256, grid_kind=ROW, work_per_block=256),
-               dict(kernel="group_scan", num_threads=self.SCAN_THREADS, grid_kind=FIXED, num_blocks=1),
-               dict(kernel="group_fill", num_threads=256, grid_kind=ROW, work_per_block=256),
+        fwd = [dict(kernel="group_clear", num_threads=256, grid_kind=NODE, work_per_block=256, prep=True),
+               dict(kernel="group_count", num_threads=256, grid_kind=ROW, work_per_block=256, prep=True),
+               dict(kernel="group_scan", num_threads=self.SCAN_THREADS, grid_kind=FIXED, num_blocks=1, prep=True),
+               dict(kernel="group_fill", num_threads=256, grid_kind=ROW, work_per_block=256, prep=True),
                dict(kernel="forward", num_threads=64, grid_kind=NODE, work_per_block=1, grid_y=f.NCH)]
         if not self.grouped_backward:
             _, bwd, _ = self.bwd.plan()
@@ -78,12 +81,12 @@ class UVUSortedGenerator:
                 return (2 * (nodes + 1) + nnz) * 8
             return fwd, bwd, ws
         b = self.bwd
-        bwd = [dict(kernel="group_clear_backward", num_threads=256, grid_kind=NODE, work_per_block=256),
-               dict(kernel="group_count_backward", num_threads=256, grid_kind=ROW, work_per_block=256),
-               dict(kernel="group_scan_backward", num_threads=self.SCAN_THREADS, grid_kind=FIXED, num_blocks=1),
-               dict(kernel="group_fill_backward", num_threads=256, grid_kind=ROW, work_per_block=256)]
+        bwd = [dict(kernel="group_clear_backward", num_threads=256, grid_kind=NODE, work_per_block=256, prep=True),
+               dict(kernel="group_count_backward", num_threads=256, grid_kind=ROW, work_per_block=256, prep=True),
+               dict(kernel="group_scan_backward", num_threads=self.SCAN_THREADS, grid_kind=FIXED, num_blocks=1, prep=True),
+               dict(kernel="group_fill_backward", num_threads=256, grid_kind=ROW, work_per_block=256, prep=True)]
         bwd += b.backward_steps()
 
         def ws(nnz=0, nodes=0):
-            return (2 * (nodes + 1) + nnz) * 8 + b.order_bytes(nodes) + b.dy_partial_bytes(nnz)
+            return 2 * (2 * (nodes + 1) + nnz) * 8 + b.order_bytes(nodes) + b.dy_partial_bytes(nnz)
         return fwd, bwd, ws

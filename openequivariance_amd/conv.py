@@ -15,12 +15,14 @@ assumption about the graph.
 """
 from __future__ import annotations
 
+import os
 import typing
 
 import numpy as np
 import torch
 
 from . import runtime as rt
+from .autograd_glue import double_backward_terms
 from .codegen.uvu_det import UVUDetGenerator
 from .codegen.uvu_direct import UVUDirectGenerator
 from .codegen.uvu_sorted import UVUSortedGenerator
@@ -88,16 +90,30 @@ def sort_by_receiver(rows: "torch.Tensor", cols: "torch.Tensor", node_count: typ
     return rows_s, cols_s, receiver_perm, transpose_perm
 
 
-def select_conv_generator(config: TPProblem, deterministic: bool, vector_stores: bool = True):
+def select_conv_generator(config: TPProblem, deterministic: bool, vector_stores: bool = True, idx_dtype=np.int64):
     """Kernel generator of the fused convolution: one node per wavefront with fixed summation order
     when deterministic; otherwise a forward that groups the edges by receiver on the fly and a
     backward with coalesced atomics."""
+    idx_ctype = "i64" if np.dtype(idx_dtype) == np.dtype(np.int64) else "int"
     if deterministic:
-        return UVUDetGenerator(config, vector_stores=vector_stores)
-    import os
+        return UVUDetGenerator(config, vector_stores=vector_stores, idx_ctype=idx_ctype)
     if os.environ.get("OEQ_AMD_CONV_FORWARD", "sorted") == "atomic":     # A/B measurements only
-        return UVUDirectGenerator(config, "conv_atomic", vector_stores=vector_stores)
-    return UVUSortedGenerator(config, vector_stores=vector_stores)
+        g = UVUDirectGenerator(config, "conv_atomic", vector_stores=vector_stores)
+        g.idx_ctype = idx_ctype
+        return g
+    return UVUSortedGenerator(config, vector_stores=vector_stores, idx_ctype=idx_ctype)
+
+
+class _StreamWorkspace:
+    """Device scratch of one operator on one stream, and which graph its preparation areas
+    (CSR pointers, position lists, node order) currently describe."""
+
+    def __init__(self):
+        self.buffer, self.size = None, 0
+        self.retired = []            # outgrown buffers that a captured HIP graph may still name
+        self.captured = False        # a HIP graph capture has used this workspace
+        self.fwd_key = self.bwd_key = None
+        self.refs = {}               # index tensors of the cached keys, kept alive so that their addresses stay theirs
 
 
 class TensorProductConv:
@@ -110,9 +126,11 @@ class TensorProductConv:
         self.config = config
         self.L1, self.L2, self.L3 = config.irreps_in1, config.irreps_in2, config.irreps_out
         self.torch_op, self.deterministic = torch_op, deterministic
-        if np.dtype(idx_dtype) != np.dtype(np.int64):
-            raise NotImplementedError("index tensors must be int64")
-        self.idx_dtype = np.int64
+        if np.dtype(idx_dtype) not in (np.dtype(np.int64), np.dtype(np.int32)):
+            raise NotImplementedError("index tensors must be int64 or int32")
+        # reference: LoopUnrollConv.py:53,78 (idx_type_map = {np.int32: "int", np.int64: "long"})
+        self.idx_dtype = np.dtype(idx_dtype).type
+        self._torch_idx = torch.int64 if self.idx_dtype == np.int64 else torch.int32
         self.conv_id = TensorProductConv.next_conv_id
         TensorProductConv.next_conv_id += 1
 
@@ -122,17 +140,17 @@ class TensorProductConv:
         if mode != "uvu":
             raise NotImplementedError("TensorProductConv supports uvu problems")
 
-        self.generator = select_conv_generator(config, deterministic)
+        self.generator = select_conv_generator(config, deterministic, idx_dtype=self.idx_dtype)
         # True: the forward writes every row of Z itself; False: it accumulates into a zeroed Z
         self.forward_overwrites = not isinstance(self.generator, UVUDirectGenerator) or deterministic
         # likewise for dX in the backward (the per-edge backward accumulates with atomics)
         self.backward_overwrites = deterministic or getattr(self.generator, "grouped_backward", False)
+        # the deterministic backward walks the caller's transpose permutation
+        self.backward_needs_tperm = deterministic
         self.jit_kernel = self.generator.render()
-        code = rt.compile_source(self.jit_kernel)
-        fwd, bwd, self._ws_bytes = self.generator.plan()
-        self.internal = rt.ConvImpl(code, _make_steps(fwd), _make_steps(bwd))
-        self.workspace_buffer = None
-        self.workspace_size = 0
+        self.internal = self._build(self.generator, self.jit_kernel)
+        self._workspaces: typing.Dict[int, _StreamWorkspace] = {}
+        self.graph_cache = os.environ.get("OEQ_AMD_GRAPH_CACHE", "1") != "0"
         self._internal_unaligned = None
         self._reorder = WeightReorder(config)
         self.reorder_weights_e3nn_to_oeq = self._reorder.e3nn_to_oeq
@@ -140,27 +158,53 @@ class TensorProductConv:
         if torch_op:
             self._setup_torch_module()
 
+    def _build(self, generator, source=None) -> "rt.ConvImpl":
+        fwd, bwd, self._ws_bytes = generator.plan()
+        need_ws = rt.STEP_NEEDS_WORKSPACE if self._ws_bytes(1, 1) > 0 else 0
+        need_tp = rt.STEP_NEEDS_TPERM if self.backward_needs_tperm else 0
+        code = rt.compile_source(source if source is not None else generator.render())
+        return rt.ConvImpl(code, _make_steps(fwd, need_ws), _make_steps(bwd, need_ws | need_tp))
+
     @staticmethod
     def name():
         return "LoopUnrollConv"
 
     # ------------------------------------------------------------------ helpers
-    def workspace_ptr(self, nnz: int, node_count: int) -> int:
-        """Device scratch for the deterministic variant, grown on demand and kept for the
-        lifetime of the object (reference: ConvolutionBase.py:93-100 allocates it once)."""
+    def _workspace_record(self, nnz: int, node_count: int, stream: typing.Optional[int] = None) -> _StreamWorkspace:
+        """The operator's scratch for ``stream`` (torch's current one by default), grown on demand.  Every
+        stream gets its own, so two streams using one operator do not share CSR pointers or position
+        lists.  A buffer that has been outgrown is freed unless a HIP graph capture has used it: a captured
+        graph has the address baked in, so such buffers stay alive as long as the operator (the reference
+        allocates its workspace once at a fixed size: ConvolutionBase.py:93-100)."""
+        sid = self._stream() if stream is None else int(stream)
+        rec = self._workspaces.get(sid)
+        if rec is None:
+            rec = self._workspaces[sid] = _StreamWorkspace()
         need = self._ws_bytes(nnz, node_count)
-        if need == 0:
+        if need > rec.size:
+            if rec.captured and rec.buffer is not None:
+                rec.retired.append(rec.buffer)
+            rec.size = int(need * 1.25) + 256
+            rec.buffer = torch.empty(rec.size, dtype=torch.uint8, device="cuda")
+            rec.fwd_key = rec.bwd_key = None
+            rec.refs.clear()
+        return rec
+
+    def workspace_ptr(self, nnz: int, node_count: int, stream: typing.Optional[int] = None) -> int:
+        """Device scratch for a call with this many edges and nodes on ``stream`` (0 when the
+        kernels use none).  Calling it invalidates nothing, but whoever launches with it outside the
+        operator's own entry points is responsible for the ``prepared`` flag."""
+        if self._ws_bytes(nnz, node_count) == 0:
             return 0
-        if self.workspace_buffer is None or self.workspace_size < need:
-            self.workspace_size = int(need * 1.25) + 256
-            self.workspace_buffer = torch.empty(self.workspace_size, dtype=torch.uint8, device="cuda")
-        return self.workspace_buffer.data_ptr()
+        return self._workspace_record(nnz, node_count, stream).buffer.data_ptr()
 
     @staticmethod
     def _stream() -> int:
         return torch.cuda.current_stream().cuda_stream
 
-    def _check(self, x, y, w, rows, cols, tperm=None):
+    def _check(self, x, y, w, rows, cols, tperm=None, g=None):
+        """Shapes, dtypes and devices, before anything is launched: the kernels dereference every
+        pointer they are handed, so a host tensor or a tensor of another GPU must never reach them."""
         E, N = rows.shape[0], x.shape[0]
         if N >= 2 ** 31:
             raise ValueError("node count must be below 2^31")
@@ -170,41 +214,96 @@ class TensorProductConv:
             raise ValueError(f"L2_in must have shape [{E}, {self.L2.dim}], got {tuple(y.shape)}")
         if tuple(w.shape) != (E, self.config.weight_numel):
             raise ValueError(f"weights must have shape [{E}, {self.config.weight_numel}], got {tuple(w.shape)}")
-        for name, t in (("rows", rows), ("cols", cols)) + ((("transpose_perm", tperm),) if tperm is not None else ()):
-            if t.dtype != torch.int64 or tuple(t.shape) != (E,):
-                raise TypeError(f"{name} must be an int64 tensor of shape [{E}]")
+        if g is not None and tuple(g.shape) != (N, self.L3.dim):
+            raise ValueError(f"L3_grad must have shape [{N}, {self.L3.dim}], got {tuple(g.shape)}")
+        if self.deterministic and tperm is None:
+            raise ValueError("the deterministic convolution needs transpose_perm")
+        index = (("rows", rows), ("cols", cols)) + ((("transpose_perm", tperm),) if tperm is not None else ())
+        for name, t in index:
+            if t.dtype != self._torch_idx or tuple(t.shape) != (E,):
+                raise TypeError(f"{name} must be an {self._torch_idx} tensor of shape [{E}]")
         tdt = {np.float32: torch.float32, np.float64: torch.float64}[self.config.irrep_dtype]
-        if x.dtype != tdt or y.dtype != tdt or w.dtype != tdt:
-            raise TypeError(f"tensors must be {tdt}")
+        data = (("L1_in", x), ("L2_in", y), ("weights", w)) + ((("L3_grad", g),) if g is not None else ())
+        for name, t in data:
+            if t.dtype != tdt:
+                raise TypeError(f"tensors must be {tdt}")
+        for name, t in data + index:
+            if not t.is_cuda:
+                raise ValueError(f"{name} is on {t.device}: every tensor, index tensors included, must be on the GPU "
+                                 "(there is no CPU implementation)")
+            if t.device != x.device:
+                raise ValueError(f"{name} is on {t.device}, L1_in on {x.device}: all tensors must share one device")
 
     def _pick(self, *ptrs):
         """The forward kernels write Z with 16-byte vector stores; a misaligned tensor (rare: a view
         with an odd storage offset) gets a variant without them, compiled on first need."""
         if any(int(p) % 16 for p in ptrs):
             if self._internal_unaligned is None:
-                g = select_conv_generator(self.config, self.deterministic, vector_stores=False)
-                fwd, bwd, _ = g.plan()
-                self._internal_unaligned = rt.ConvImpl(rt.compile_source(g.render()), _make_steps(fwd), _make_steps(bwd))
+                g = select_conv_generator(self.config, self.deterministic, vector_stores=False, idx_dtype=self.idx_dtype)
+                ws_bytes = self._ws_bytes
+                self._internal_unaligned = self._build(g)
+                self._ws_bytes = ws_bytes
             return self._internal_unaligned
         return self.internal
 
     # ---------------------------------------------------------- raw entry points
     def exec_conv_rawptrs(self, L1_in, L2_in, weights, L3_out, rows, cols, nnz, node_count, workspace=0,
-                          transpose_perm=0, stream=None):
-        """reference: extension/convolution.hpp:121-147"""
+                          transpose_perm=0, stream=None, prepared=False):
+        """reference: extension/convolution.hpp:121-147.  Without ``workspace`` the operator's own scratch
+        for the stream is used.  ``prepared=True`` promises that the workspace still holds the forward
+        preparation of exactly this graph (left by an earlier forward call): the preparation kernels are
+        then skipped."""
+        nnz, node_count = int(nnz), int(node_count)
+        if nnz > 0 and not (rows and cols):
+            raise ValueError("rows / cols must be device pointers")
         impl = self._pick(L1_in, L2_in, weights, L3_out)
-        workspace = workspace or self.workspace_ptr(int(nnz), int(node_count))     # the operator owns one
-        impl.exec_conv_rawptrs(L1_in, L2_in, weights, L3_out, rows, cols, int(nnz), int(node_count),
-                               workspace, transpose_perm, self._stream() if stream is None else stream)
+        if not workspace:
+            rec = self._workspace_record(nnz, node_count, stream)
+            rec.fwd_key = None                                  # the caller's graph is unknown to the cache
+            workspace = rec.buffer.data_ptr() if self._ws_bytes(nnz, node_count) else 0
+        impl.exec_conv_rawptrs(L1_in, L2_in, weights, L3_out, rows, cols, nnz, node_count,
+                               workspace, transpose_perm, self._stream() if stream is None else stream, prepared)
 
     def backward_rawptrs(self, L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_grad, rows, cols, nnz,
-                         node_count, workspace=0, transpose_perm=0, stream=None):
-        """reference: extension/convolution.hpp:149-173"""
+                         node_count, workspace=0, transpose_perm=0, stream=None, prepared=False):
+        """reference: extension/convolution.hpp:149-173; ``workspace`` and ``prepared`` as in
+        exec_conv_rawptrs (the backward keeps its own preparation in the workspace)."""
+        nnz, node_count = int(nnz), int(node_count)
+        if nnz > 0 and not (rows and cols):
+            raise ValueError("rows / cols must be device pointers")
+        if self.backward_needs_tperm and nnz > 0 and not transpose_perm:
+            raise ValueError("the deterministic backward needs transpose_perm (a device pointer), got 0")
         impl = self._pick(L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_grad)
-        workspace = workspace or self.workspace_ptr(int(nnz), int(node_count))
+        if not workspace:
+            rec = self._workspace_record(nnz, node_count, stream)
+            rec.bwd_key = None
+            workspace = rec.buffer.data_ptr() if self._ws_bytes(nnz, node_count) else 0
         impl.backward_rawptrs(L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_grad, rows, cols,
-                              int(nnz), int(node_count), workspace, transpose_perm,
-                              self._stream() if stream is None else stream)
+                              nnz, node_count, workspace, transpose_perm,
+                              self._stream() if stream is None else stream, prepared)
+
+    def _cached_call(self, which: str, rows, cols, tperm, E: int, N: int, launch) -> None:
+        """Run ``launch(workspace pointer, prepared)`` for the torch operators.  The graph preparation a
+        call leaves in the stream's workspace is reused by the next call of the same direction when it
+        names the same graph: same index tensors (address and in-place version counter), same sizes.  The
+        tensors are kept referenced while their key is cached, so the addresses cannot be handed to other
+        tensors meanwhile.  Under HIP graph capture, and on a workspace that a capture has used, the
+        preparation always runs: a replay may rewrite the workspace behind the cache's back."""
+        if self._ws_bytes(E, N) == 0:
+            launch(0, False)
+            return
+        rec = self._workspace_record(E, N)
+        if torch.cuda.is_current_stream_capturing():
+            rec.captured = True
+        key = None
+        if self.graph_cache and not rec.captured:
+            key = (E, N) + tuple((t.data_ptr(), t._version) for t in (rows, cols, tperm) if t is not None)
+        attr = which + "_key"
+        prepared = key is not None and getattr(rec, attr) == key
+        setattr(rec, attr, None)
+        launch(rec.buffer.data_ptr(), prepared)
+        setattr(rec, attr, key)
+        rec.refs[which] = (rows, cols, tperm) if key is not None else None
 
     # ------------------------------------------------------------------ torch ops
     def _setup_torch_module(self) -> None:
@@ -221,78 +320,44 @@ class TensorProductConv:
             E, N = rows.shape[0], x.shape[0]
             # the atomic kernels accumulate into Z; the deterministic ones write every row
             out = (torch.empty if self.forward_overwrites else torch.zeros)((N, L3_dim), dtype=x.dtype, device=x.device)
-            self.exec_conv_rawptrs(x.data_ptr(), y.data_ptr(), w.data_ptr(), out.data_ptr(), rows.data_ptr(),
-                                   cols.data_ptr(), E, N, self.workspace_ptr(E, N),
-                                   tperm.data_ptr() if tperm is not None else 0)
+            with torch.cuda.device(x.device):
+                self._cached_call("fwd", rows, cols, tperm, E, N, lambda ws, prepared: self.exec_conv_rawptrs(
+                    x.data_ptr(), y.data_ptr(), w.data_ptr(), out.data_ptr(), rows.data_ptr(), cols.data_ptr(), E, N,
+                    ws, tperm.data_ptr() if tperm is not None else 0, prepared=prepared))
             return out
 
         def bwd_impl(L1_in, L2_in, weights, L3_grad, rows, cols, tperm):
             x, y, w, g = L1_in.contiguous(), L2_in.contiguous(), weights.contiguous(), L3_grad.contiguous()
             rows, cols = rows.contiguous(), cols.contiguous()
             tperm = tperm.contiguous() if tperm is not None else None
-            self._check(x, y, w, rows, cols, tperm)
+            self._check(x, y, w, rows, cols, tperm, g)
             E, N = rows.shape[0], x.shape[0]
             xg = (torch.empty_like if self.backward_overwrites else torch.zeros_like)(x)
             yg, wg = torch.empty_like(y), torch.empty_like(w)
-            self.backward_rawptrs(x.data_ptr(), xg.data_ptr(), y.data_ptr(), yg.data_ptr(), w.data_ptr(),
-                                  wg.data_ptr(), g.data_ptr(), rows.data_ptr(), cols.data_ptr(), E, N,
-                                  self.workspace_ptr(E, N), tperm.data_ptr() if tperm is not None else 0)
+            with torch.cuda.device(x.device):
+                self._cached_call("bwd", rows, cols, tperm, E, N, lambda ws, prepared: self.backward_rawptrs(
+                    x.data_ptr(), xg.data_ptr(), y.data_ptr(), yg.data_ptr(), w.data_ptr(), wg.data_ptr(), g.data_ptr(),
+                    rows.data_ptr(), cols.data_ptr(), E, N, ws, tperm.data_ptr() if tperm is not None else 0,
+                    prepared=prepared))
             return [xg, yg, wg]
 
+        # the two variants differ only in the trailing transpose_perm argument, which torch's operator
+        # schemas need spelled out
         if not det:
             @torch.library.custom_op(f"openequivariance_amd::conv_forward{cid}", mutates_args=(), device_types="cuda")
             def forward(L1_in: torch.Tensor, L2_in: torch.Tensor, weights: torch.Tensor, rows: torch.Tensor,
                         cols: torch.Tensor) -> torch.Tensor:
                 return fwd_impl(L1_in, L2_in, weights, rows, cols, None)
 
-            @forward.register_fake
-            def _(L1_in, L2_in, weights, rows, cols):
-                return L1_in.new_empty(L1_in.shape[0], L3_dim)
-
             @torch.library.custom_op(f"openequivariance_amd::conv_backward{cid}", mutates_args=(), device_types="cuda")
             def backward_helper(L1_in: torch.Tensor, L2_in: torch.Tensor, weights: torch.Tensor, L3_grad: torch.Tensor,
                                 rows: torch.Tensor, cols: torch.Tensor) -> typing.List[torch.Tensor]:
                 return bwd_impl(L1_in, L2_in, weights, L3_grad, rows, cols, None)
-
-            @backward_helper.register_fake
-            def _(L1_in, L2_in, weights, L3_grad, rows, cols):
-                return [L1_in.new_empty(*L1_in.shape), L2_in.new_empty(*L2_in.shape), weights.new_empty(*weights.shape)]
-
-            def setup_context(ctx, inputs, output):
-                ctx.L1_in, ctx.L2_in, ctx.weights, ctx.rows, ctx.cols = inputs
-
-            def backward(ctx, grad_output):
-                r = backward_helper(ctx.L1_in, ctx.L2_in, ctx.weights, grad_output, ctx.rows, ctx.cols)
-                return r[0], r[1], r[2], None, None
-
-            forward.register_autograd(backward, setup_context=setup_context)
-
-            def setup_context_double_backward(ctx, inputs, output):
-                ctx.L1_in, ctx.L2_in, ctx.weights, ctx.L3_grad, ctx.rows, ctx.cols = inputs
-
-            def double_backward(ctx, grad_output):
-                A, B, C, D = ctx.L1_in, ctx.L2_in, ctx.L3_grad, ctx.weights
-                E, F, G = grad_output[0], grad_output[1], grad_output[2]
-                r, c = ctx.rows, ctx.cols
-                op1 = backward_helper(E, F, D, C, r, c)
-                op2 = backward_helper(A, B, G, C, r, c)
-                op3 = forward(E, B, D, r, c)
-                op4 = backward_helper(E, B, D, C, r, c)
-                op5 = backward_helper(A, F, D, C, r, c)
-                op6 = forward(A, F, D, r, c)
-                op7 = forward(A, B, G, r, c)
-                return op1[0] + op2[0], op1[1] + op2[1], (op4[2] + op5[2]), (op3 + op6 + op7), None, None
-
-            backward_helper.register_autograd(double_backward, setup_context=setup_context_double_backward)
         else:
             @torch.library.custom_op(f"openequivariance_amd::conv_forward{cid}", mutates_args=(), device_types="cuda")
             def forward(L1_in: torch.Tensor, L2_in: torch.Tensor, weights: torch.Tensor, rows: torch.Tensor,
                         cols: torch.Tensor, transpose_perm: torch.Tensor) -> torch.Tensor:
                 return fwd_impl(L1_in, L2_in, weights, rows, cols, transpose_perm)
-
-            @forward.register_fake
-            def _(L1_in, L2_in, weights, rows, cols, transpose_perm):
-                return L1_in.new_empty(L1_in.shape[0], L3_dim)
 
             @torch.library.custom_op(f"openequivariance_amd::conv_backward{cid}", mutates_args=(), device_types="cuda")
             def backward_helper(L1_in: torch.Tensor, L2_in: torch.Tensor, weights: torch.Tensor, L3_grad: torch.Tensor,
@@ -300,38 +365,32 @@ class TensorProductConv:
                                 transpose_perm: torch.Tensor) -> typing.List[torch.Tensor]:
                 return bwd_impl(L1_in, L2_in, weights, L3_grad, rows, cols, transpose_perm)
 
-            @backward_helper.register_fake
-            def _(L1_in, L2_in, weights, L3_grad, rows, cols, transpose_perm):
-                return [L1_in.new_empty(*L1_in.shape), L2_in.new_empty(*L2_in.shape), weights.new_empty(*weights.shape)]
+        @forward.register_fake
+        def _(L1_in, L2_in, weights, *index):
+            return L1_in.new_empty(L1_in.shape[0], L3_dim)
 
-            def setup_context(ctx, inputs, output):
-                ctx.L1_in, ctx.L2_in, ctx.weights, ctx.rows, ctx.cols, ctx.transpose_perm = inputs
+        @backward_helper.register_fake
+        def _(L1_in, L2_in, weights, L3_grad, *index):
+            return [L1_in.new_empty(*L1_in.shape), L2_in.new_empty(*L2_in.shape), weights.new_empty(*weights.shape)]
 
-            def backward(ctx, grad_output):
-                r = backward_helper(ctx.L1_in, ctx.L2_in, ctx.weights, grad_output, ctx.rows, ctx.cols,
-                                    ctx.transpose_perm)
-                return r[0], r[1], r[2], None, None, None
+        def setup_context(ctx, inputs, output):
+            ctx.L1_in, ctx.L2_in, ctx.weights, *ctx.index = inputs
 
-            forward.register_autograd(backward, setup_context=setup_context)
+        def backward(ctx, grad_output):
+            r = backward_helper(ctx.L1_in, ctx.L2_in, ctx.weights, grad_output, *ctx.index)
+            return (r[0], r[1], r[2]) + (None,) * len(ctx.index)
 
-            def setup_context_double_backward(ctx, inputs, output):
-                ctx.L1_in, ctx.L2_in, ctx.weights, ctx.L3_grad, ctx.rows, ctx.cols, ctx.transpose_perm = inputs
+        forward.register_autograd(backward, setup_context=setup_context)
 
-            def double_backward(ctx, grad_output):
-                A, B, C, D = ctx.L1_in, ctx.L2_in, ctx.L3_grad, ctx.weights
-                E, F, G = grad_output[0], grad_output[1], grad_output[2]
-                r, c, t = ctx.rows, ctx.cols, ctx.transpose_perm
-                op1 = backward_helper(E, F, D, C, r, c, t)
-                op2 = backward_helper(A, B, G, C, r, c, t)
-                op3 = forward(E, B, D, r, c, t)
-                op4 = backward_helper(E, B, D, C, r, c, t)
-                op5 = backward_helper(A, F, D, C, r, c, t)
-                op6 = forward(A, F, D, r, c, t)
-                op7 = forward(A, B, G, r, c, t)
-                return (op1[0] + op2[0], op1[1] + op2[1], (op4[2] + op5[2]), (op3 + op6 + op7), None, None, None)
+        def setup_context_double_backward(ctx, inputs, output):
+            ctx.L1_in, ctx.L2_in, ctx.weights, ctx.L3_grad, *ctx.index = inputs
 
-            backward_helper.register_autograd(double_backward, setup_context=setup_context_double_backward)
+        def double_backward(ctx, grad_output):
+            terms = double_backward_terms(forward, backward_helper, ctx.L1_in, ctx.L2_in, ctx.weights, ctx.L3_grad,
+                                          grad_output[0], grad_output[1], grad_output[2], tuple(ctx.index))
+            return terms + (None,) * len(ctx.index)
 
+        backward_helper.register_autograd(double_backward, setup_context=setup_context_double_backward)
         self.forward = forward
         self.backward_helper = backward_helper
 

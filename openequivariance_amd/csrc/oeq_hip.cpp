@@ -97,6 +97,17 @@ int launch(const Step& s, uint64_t rows, uint64_t nodes, void** args, void* stre
     return 0;
 }
 
+// Rejects a NULL workspace / transpose permutation that a step of the plan would dereference.
+int check_pointers(const std::vector<Step>& steps, const void* workspace, const void* tperm, const char* what) {
+    for (auto& s : steps) {
+        if ((s.desc.flags & OEQ_STEP_NEEDS_WORKSPACE) && !workspace)
+            return fail("%s: kernel '%s' needs a workspace, but the workspace pointer is NULL", what, s.desc.kernel);
+        if ((s.desc.flags & OEQ_STEP_NEEDS_TPERM) && !tperm)
+            return fail("%s: kernel '%s' reads the transpose permutation, but that pointer is NULL", what, s.desc.kernel);
+    }
+    return 0;
+}
+
 }  // namespace
 
 struct oeq_tp {
@@ -229,6 +240,7 @@ int oeq_tp_forward(oeq_tp* tp, uint64_t n, const void* L1, const void* L2, void*
                    void* workspace, void* stream) {
     if (!tp) return fail("null handle");
     if (tp->fwd.empty()) return fail("this operator was built without a forward plan");
+    if (n > 0 && check_pointers(tp->fwd, workspace, (const void*)1, "forward")) return 1;
     void* args[] = {&n, &L1, &L2, &L3, &W, &workspace};
     for (auto& s : tp->fwd)
         if (launch(s, n, 0, args, stream)) return 1;
@@ -239,6 +251,7 @@ int oeq_tp_backward(oeq_tp* tp, uint64_t n, const void* L1, void* L1g, const voi
                     const void* W, void* Wg, const void* L3g, void* workspace, void* stream) {
     if (!tp) return fail("null handle");
     if (tp->bwd.empty()) return fail("this operator was built without a backward plan");
+    if (n > 0 && check_pointers(tp->bwd, workspace, (const void*)1, "backward")) return 1;
     void* args[] = {&n, &L1, &L1g, &L2, &L2g, &W, &Wg, &L3g, &workspace};
     for (auto& s : tp->bwd)
         if (launch(s, n, 0, args, stream)) return 1;
@@ -261,28 +274,60 @@ int oeq_conv_create(const void* code, size_t code_size, const oeq_step* fs, int 
 
 void oeq_conv_destroy(oeq_conv* c) { delete c; }
 
-int oeq_conv_forward(oeq_conv* c, const void* L1, const void* L2, const void* W, void* L3,
-                     const void* rows, const void* cols, uint64_t nnz, uint64_t node_count,
-                     void* workspace, const void* tperm, void* stream) {
+static int conv_forward(oeq_conv* c, const void* L1, const void* L2, const void* W, void* L3,
+                        const void* rows, const void* cols, uint64_t nnz, uint64_t node_count,
+                        void* workspace, const void* tperm, void* stream, bool prepared) {
     if (!c) return fail("null handle");
     if (c->fwd.empty()) return fail("this operator was built without a forward plan");
     if (nnz > 0 && node_count == 0) return fail("convolution called with %llu edges but no nodes", (unsigned long long)nnz);
+    if (nnz > 0 && (!rows || !cols)) return fail("forward: rows / cols are NULL");
+    if ((nnz > 0 || node_count > 0) && check_pointers(c->fwd, workspace, tperm, "forward")) return 1;
     void* args[] = {&L1, &L2, &W, &L3, &rows, &cols, &nnz, &node_count, &workspace, &tperm};
-    for (auto& s : c->fwd)
+    for (auto& s : c->fwd) {
+        if (prepared && (s.desc.flags & OEQ_STEP_GRAPH_PREP)) continue;
         if (launch(s, nnz, node_count, args, stream)) return 1;
+    }
     return 0;
+}
+
+static int conv_backward(oeq_conv* c, const void* L1, void* L1g, const void* L2, void* L2g, const void* W,
+                         void* Wg, const void* L3g, const void* rows, const void* cols, uint64_t nnz,
+                         uint64_t node_count, void* workspace, const void* tperm, void* stream, bool prepared) {
+    if (!c) return fail("null handle");
+    if (c->bwd.empty()) return fail("this operator was built without a backward plan");
+    if (nnz > 0 && node_count == 0) return fail("convolution called with %llu edges but no nodes", (unsigned long long)nnz);
+    if (nnz > 0 && (!rows || !cols)) return fail("backward: rows / cols are NULL");
+    if ((nnz > 0 || node_count > 0) && check_pointers(c->bwd, workspace, tperm, "backward")) return 1;
+    void* args[] = {&L1, &L1g, &L2, &L2g, &W, &Wg, &L3g, &rows, &cols, &nnz, &node_count, &workspace, &tperm};
+    for (auto& s : c->bwd) {
+        if (prepared && (s.desc.flags & OEQ_STEP_GRAPH_PREP)) continue;
+        if (launch(s, nnz, node_count, args, stream)) return 1;
+    }
+    return 0;
+}
+
+int oeq_conv_forward(oeq_conv* c, const void* L1, const void* L2, const void* W, void* L3,
+                     const void* rows, const void* cols, uint64_t nnz, uint64_t node_count,
+                     void* workspace, const void* tperm, void* stream) {
+    return conv_forward(c, L1, L2, W, L3, rows, cols, nnz, node_count, workspace, tperm, stream, false);
+}
+
+int oeq_conv_forward_prepared(oeq_conv* c, const void* L1, const void* L2, const void* W, void* L3,
+                              const void* rows, const void* cols, uint64_t nnz, uint64_t node_count,
+                              void* workspace, const void* tperm, void* stream) {
+    return conv_forward(c, L1, L2, W, L3, rows, cols, nnz, node_count, workspace, tperm, stream, true);
 }
 
 int oeq_conv_backward(oeq_conv* c, const void* L1, void* L1g, const void* L2, void* L2g, const void* W,
                       void* Wg, const void* L3g, const void* rows, const void* cols, uint64_t nnz,
                       uint64_t node_count, void* workspace, const void* tperm, void* stream) {
-    if (!c) return fail("null handle");
-    if (c->bwd.empty()) return fail("this operator was built without a backward plan");
-    if (nnz > 0 && node_count == 0) return fail("convolution called with %llu edges but no nodes", (unsigned long long)nnz);
-    void* args[] = {&L1, &L1g, &L2, &L2g, &W, &Wg, &L3g, &rows, &cols, &nnz, &node_count, &workspace, &tperm};
-    for (auto& s : c->bwd)
-        if (launch(s, nnz, node_count, args, stream)) return 1;
-    return 0;
+    return conv_backward(c, L1, L1g, L2, L2g, W, Wg, L3g, rows, cols, nnz, node_count, workspace, tperm, stream, false);
+}
+
+int oeq_conv_backward_prepared(oeq_conv* c, const void* L1, void* L1g, const void* L2, void* L2g, const void* W,
+                               void* Wg, const void* L3g, const void* rows, const void* cols, uint64_t nnz,
+                               uint64_t node_count, void* workspace, const void* tperm, void* stream) {
+    return conv_backward(c, L1, L1g, L2, L2g, W, Wg, L3g, rows, cols, nnz, node_count, workspace, tperm, stream, true);
 }
 
 // ---------------------------------------------------------- generic module

@@ -25,7 +25,7 @@ def benchmark_generators():
             ("mace/tp", select_generator(ChannelwiseTPP(*MACE))),
             ("mace-all-parities/tp", select_generator(ChannelwiseTPP(*MACE_ALL))),
             ("nequip/tp", select_generator(ChannelwiseTPP(*NEQUIP)))]
-    for label, irreps in (("nequip", NEQUIP), ("large", LARGE)):
+    for label, irreps in (("nequip", NEQUIP), ("large", LARGE), ("mace", MACE)):
         for det in (False, True):
             gens.append((f"{label}/conv_{'det' if det else 'atomic'}", select_conv_generator(ChannelwiseTPP(*irreps), det)))
     for dt in (np.float32, np.float64):
@@ -34,9 +34,10 @@ def benchmark_generators():
     return gens
 
 
-def compile_benchmark_kernels(verbose: bool = False) -> None:
+def compile_benchmark_kernels(verbose: bool = False, refresh: bool = False) -> None:
+    """``refresh``: compile every kernel set again even where the cache already holds its code object."""
     for name, g in benchmark_generators():
         t = time.time()
-        code = rt.compile_source(g.render())
+        code = rt.compile_source(g.render(), refresh=refresh)
         if verbose:
             print(f"hipRTC gfx950 {name}: {len(code) // 1024} KiB ({time.time() - t:.1f}s)", flush=True)

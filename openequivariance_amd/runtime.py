@@ -20,6 +20,7 @@ CACHE_DIR = pathlib.Path(os.environ.get("OEQ_AMD_CACHE", PKG_DIR / "_kcache"))
 TARGET_ARCH = "gfx950"
 
 GRID_FIXED, GRID_PER_ROW, GRID_PER_NODE = 0, 1, 2
+STEP_NEEDS_WORKSPACE, STEP_NEEDS_TPERM, STEP_GRAPH_PREP = 1, 2, 4
 
 
 class DeviceProp(C.Structure):
@@ -35,15 +36,16 @@ class Step(C.Structure):
     """Mirror of ``oeq_step``: one kernel launch of an operator."""
     _fields_ = [("kernel", C.c_char * 64), ("num_threads", C.c_uint32), ("smem", C.c_uint32),
                 ("grid_kind", C.c_uint32), ("work_per_block", C.c_uint32), ("num_blocks", C.c_uint32),
-                ("grid_y", C.c_uint32), ("warp_size", C.c_uint32)]
+                ("grid_y", C.c_uint32), ("warp_size", C.c_uint32), ("flags", C.c_uint32)]
 
     @classmethod
     def make(cls, kernel: str, num_threads: int, smem: int = 0, grid_kind: int = GRID_PER_ROW,
-             work_per_block: int = 1, num_blocks: int = 0, grid_y: int = 1) -> "Step":
+             work_per_block: int = 1, num_blocks: int = 0, grid_y: int = 1, flags: int = 0) -> "Step":
         s = cls()
         s.kernel = kernel.encode()
         s.num_threads, s.smem, s.grid_kind = num_threads, smem, grid_kind
         s.work_per_block, s.num_blocks, s.grid_y, s.warp_size = work_per_block, num_blocks, grid_y, 64
+        s.flags = flags
         return s
 
 
@@ -86,6 +88,8 @@ def lib() -> C.CDLL:
             "oeq_conv_destroy": (None, [vp]),
             "oeq_conv_forward": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, u64, u64, vp, vp, vp]),
             "oeq_conv_backward": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, u64, u64, vp, vp, vp]),
+            "oeq_conv_forward_prepared": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, u64, u64, vp, vp, vp]),
+            "oeq_conv_backward_prepared": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, u64, u64, vp, vp, vp]),
             "oeq_module_load": (C.c_int, [vp, sz, C.POINTER(vp)]),
             "oeq_module_unload": (None, [vp]),
             "oeq_module_launch": (C.c_int, [vp, C.c_char_p, C.c_uint32, C.c_uint32, C.c_uint32, vp, C.POINTER(vp)]),
@@ -112,6 +116,7 @@ EXPORTED_SYMBOLS = [
     "oeq_last_error", "oeq_device_props", "oeq_device_count", "oeq_compile", "oeq_free", "oeq_hiprtc_version",
     "oeq_tp_create", "oeq_tp_destroy", "oeq_tp_forward", "oeq_tp_backward",
     "oeq_conv_create", "oeq_conv_destroy", "oeq_conv_forward", "oeq_conv_backward",
+    "oeq_conv_forward_prepared", "oeq_conv_backward_prepared",
     "oeq_module_load", "oeq_module_unload", "oeq_module_launch",
     "oeq_timer_create", "oeq_timer_destroy", "oeq_timer_start", "oeq_timer_stop", "oeq_timer_clear_cache",
     "oeq_buffer_alloc", "oeq_buffer_free", "oeq_buffer_h2d", "oeq_buffer_d2h", "oeq_buffer_zero",
@@ -149,12 +154,13 @@ def hiprtc_version() -> str:
 
 
 def compile_source(source: str, arch: str = TARGET_ARCH, options: Sequence[str] = DEFAULT_OPTIONS,
-                   use_cache: bool = True) -> bytes:
+                   use_cache: bool = True, refresh: bool = False) -> bytes:
     """hipRTC-compile ``source`` for ``arch``; code objects are cached on disk keyed by
-    (source, arch, options, hipRTC version)."""
+    (source, arch, options, hipRTC version).  ``refresh`` compiles even when the cache holds the
+    code object and replaces it."""
     key = hashlib.sha256("\0".join([source, arch, *options, hiprtc_version()]).encode()).hexdigest()[:32]
     path = CACHE_DIR / f"{key}.hsaco"
-    if use_cache and path.exists():
+    if use_cache and not refresh and path.exists():
         return path.read_bytes()
     opts = (C.c_char_p * len(options))(*[o.encode() for o in options])
     code, size = C.c_void_p(), C.c_size_t()
@@ -214,13 +220,17 @@ class ConvImpl:
         ba, nb = _steps(backward_steps)
         _check(lib().oeq_conv_create(code, len(code), fa, nf, ba, nb, C.byref(self._h)))
 
-    def exec_conv_rawptrs(self, L1, L2, W, L3, rows, cols, nnz, node_count, workspace=0, tperm=0, stream=0):
-        _check(lib().oeq_conv_forward(self._h, L1, L2, W, L3, rows, cols, nnz, node_count, workspace, tperm, stream))
+    def exec_conv_rawptrs(self, L1, L2, W, L3, rows, cols, nnz, node_count, workspace=0, tperm=0, stream=0,
+                          prepared=False):
+        """``prepared``: the workspace still holds this graph's forward preparation (see
+        oeq_conv_forward_prepared); the preparation kernels are then not launched."""
+        fn = lib().oeq_conv_forward_prepared if prepared else lib().oeq_conv_forward
+        _check(fn(self._h, L1, L2, W, L3, rows, cols, nnz, node_count, workspace, tperm, stream))
 
     def backward_rawptrs(self, L1, L1g, L2, L2g, W, Wg, L3g, rows, cols, nnz, node_count,
-                         workspace=0, tperm=0, stream=0):
-        _check(lib().oeq_conv_backward(self._h, L1, L1g, L2, L2g, W, Wg, L3g, rows, cols, nnz, node_count,
-                                       workspace, tperm, stream))
+                         workspace=0, tperm=0, stream=0, prepared=False):
+        fn = lib().oeq_conv_backward_prepared if prepared else lib().oeq_conv_backward
+        _check(fn(self._h, L1, L1g, L2, L2g, W, Wg, L3g, rows, cols, nnz, node_count, workspace, tperm, stream))
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None

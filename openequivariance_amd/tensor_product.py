@@ -16,6 +16,7 @@ import numpy as np
 import torch
 
 from . import runtime as rt
+from .autograd_glue import double_backward_terms
 from .codegen.uvu import UVUGenerator
 from .codegen.uvu_direct import UVUDirectGenerator
 from .problem import TPProblem
@@ -23,9 +24,12 @@ from .weight_order import WeightReorder, is_identity
 from .wigner import wigner_3j
 
 
-def _make_steps(descs):
+def _make_steps(descs, flags: int = 0):
+    """Plan dictionaries of a generator -> ``runtime.Step`` records.  ``flags`` (STEP_NEEDS_*) apply to
+    every step of the plan; a step's own ``prep=True`` marks it as graph preparation."""
     return [rt.Step.make(d["kernel"], d["num_threads"], d.get("smem", 0), d.get("grid_kind", rt.GRID_PER_ROW),
-                         d.get("work_per_block", 1), d.get("num_blocks", 0), d.get("grid_y", 1)) for d in descs]
+                         d.get("work_per_block", 1), d.get("num_blocks", 0), d.get("grid_y", 1),
+                         flags | (rt.STEP_GRAPH_PREP if d.get("prep") else 0)) for d in descs]
 
 
 def select_generator(config: TPProblem):
@@ -89,8 +93,9 @@ class TensorProduct(TensorProductBase):
         code = rt.compile_source(self.jit_kernel)
         fwd, bwd, ws = self.generator.plan()
         self.workspace_bytes = ws()
-        self.internal = rt.TPImpl(code, _make_steps(fwd), _make_steps(bwd))
-        self._workspace = None
+        self._step_flags = rt.STEP_NEEDS_WORKSPACE if self.workspace_bytes else 0
+        self.internal = rt.TPImpl(code, _make_steps(fwd, self._step_flags), _make_steps(bwd, self._step_flags))
+        self._workspaces = {}                 # stream -> scratch tensor (fixed size, never regrown)
         self._internal_unaligned = None       # kernels without 16-byte vector stores, compiled on first need
 
         self._reorder = WeightReorder(config)
@@ -108,12 +113,16 @@ class TensorProduct(TensorProductBase):
         return "LoopUnrollTP"
 
     # ----------------------------------------------------------- raw entry points
-    def _workspace_ptr(self) -> int:
+    def _workspace_ptr(self, stream=None) -> int:
+        """Scratch of this operator for ``stream`` (packed weights, dW partial sums): one buffer per
+        stream, so that two streams using one operator do not overwrite each other's partial sums."""
         if self.workspace_bytes == 0:
             return 0
-        if self._workspace is None:
-            self._workspace = torch.empty(self.workspace_bytes, dtype=torch.uint8, device="cuda")
-        return self._workspace.data_ptr()
+        sid = self._stream() if stream is None else int(stream)
+        buf = self._workspaces.get(sid)
+        if buf is None:
+            buf = self._workspaces[sid] = torch.empty(self.workspace_bytes, dtype=torch.uint8, device="cuda")
+        return buf.data_ptr()
 
     @staticmethod
     def _stream() -> int:
@@ -126,14 +135,15 @@ class TensorProduct(TensorProductBase):
             if self._internal_unaligned is None:
                 g = UVUDirectGenerator(self.config, "tp", vector_stores=False)
                 fwd, bwd, _ = g.plan()
-                self._internal_unaligned = rt.TPImpl(rt.compile_source(g.render()), _make_steps(fwd), _make_steps(bwd))
+                self._internal_unaligned = rt.TPImpl(rt.compile_source(g.render()), _make_steps(fwd, self._step_flags),
+                                                     _make_steps(bwd, self._step_flags))
             return self._internal_unaligned
         return self.internal
 
     def forward_raw(self, batch, L1_in, L2_in, L3_out, weights, stream=None) -> None:
         """Device pointers as integers (reference: TensorProductBase.py:41-49)."""
         impl = self._pick(L1_in, L2_in, L3_out, weights)
-        impl.exec_tensor_product(int(batch), L1_in, L2_in, L3_out, weights, self._workspace_ptr(),
+        impl.exec_tensor_product(int(batch), L1_in, L2_in, L3_out, weights, self._workspace_ptr(stream),
                                  self._stream() if stream is None else stream)
 
     def backward_raw(self, batch_size, L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_grad,
@@ -141,7 +151,7 @@ class TensorProduct(TensorProductBase):
         """reference: TensorProductBase.py:51-61."""
         impl = self._pick(L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_grad)
         impl.backward(int(batch_size), L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_grad,
-                      self._workspace_ptr(), self._stream() if stream is None else stream)
+                      self._workspace_ptr(stream), self._stream() if stream is None else stream)
 
     # ------------------------------------------------- numpy entry points (tests)
     def forward_cpu(self, L1_in, L2_in, L3_out, weights) -> None:
@@ -183,7 +193,8 @@ class TensorProduct(TensorProductBase):
             x, y, w = L1_in.contiguous(), L2_in.contiguous(), weights.contiguous()
             self._check_inputs(x, y, w)
             out = torch.empty((x.shape[0], L3_dim), dtype=x.dtype, device=x.device)
-            self.forward_raw(x.shape[0], x.data_ptr(), y.data_ptr(), out.data_ptr(), w.data_ptr())
+            with torch.cuda.device(x.device):
+                self.forward_raw(x.shape[0], x.data_ptr(), y.data_ptr(), out.data_ptr(), w.data_ptr())
             return out
 
         @forward.register_fake
@@ -196,10 +207,11 @@ class TensorProduct(TensorProductBase):
         def backward_helper(L1_in: torch.Tensor, L2_in: torch.Tensor, weights: torch.Tensor,
                             L3_grad: torch.Tensor) -> typing.List[torch.Tensor]:
             x, y, w, g = L1_in.contiguous(), L2_in.contiguous(), weights.contiguous(), L3_grad.contiguous()
-            self._check_inputs(x, y, w)
+            self._check_inputs(x, y, w, g)
             xg, yg, wg = torch.empty_like(x), torch.empty_like(y), torch.empty_like(w)
-            self.backward_raw(x.shape[0], x.data_ptr(), xg.data_ptr(), y.data_ptr(), yg.data_ptr(),
-                              w.data_ptr(), wg.data_ptr(), g.data_ptr())
+            with torch.cuda.device(x.device):
+                self.backward_raw(x.shape[0], x.data_ptr(), xg.data_ptr(), y.data_ptr(), yg.data_ptr(),
+                                  w.data_ptr(), wg.data_ptr(), g.data_ptr())
             return [xg, yg, wg]
 
         @backward_helper.register_fake
@@ -221,20 +233,14 @@ class TensorProduct(TensorProductBase):
             ctx.L1_in, ctx.L2_in, ctx.weights, ctx.L3_grad = inputs
 
         def double_backward(ctx, grad_output):
-            A, B, C, D = ctx.L1_in, ctx.L2_in, ctx.L3_grad, ctx.weights
-            E, F, G = grad_output[0], grad_output[1], grad_output[2]
-            op1 = backward_helper(E, F, D, C)
-            op2 = backward_helper(A, B, G, C)
-            op3 = forward(E, B, D)
-            op4 = backward_helper(E, B, D, C)
-            op5 = backward_helper(A, F, D, C)
-            op6 = forward(A, F, D)
-            op7 = forward(A, B, G)
-            return op1[0] + op2[0], op1[1] + op2[1], (op4[2] + op5[2]), (op3 + op6 + op7)
+            return double_backward_terms(forward, backward_helper, ctx.L1_in, ctx.L2_in, ctx.weights, ctx.L3_grad,
+                                         grad_output[0], grad_output[1], grad_output[2])
 
         backward_helper.register_autograd(double_backward, setup_context=setup_context_double_backward)
 
-    def _check_inputs(self, x, y, w) -> None:
+    def _check_inputs(self, x, y, w, g=None) -> None:
+        """Shapes, dtypes and devices, before anything is launched (the kernels dereference every
+        pointer they are handed)."""
         B = x.shape[0]
         if x.ndim != 2 or x.shape[1] != self.L1.dim:
             raise ValueError(f"L1_in must have shape [batch, {self.L1.dim}], got {tuple(x.shape)}")
@@ -243,9 +249,17 @@ class TensorProduct(TensorProductBase):
         want = (self.config.weight_numel,) if self.config.shared_weights else (B, self.config.weight_numel)
         if tuple(w.shape) != want:
             raise ValueError(f"weights must have shape {want}, got {tuple(w.shape)}")
+        if g is not None and tuple(g.shape) != (B, self.L3.dim):
+            raise ValueError(f"L3_grad must have shape [{B}, {self.L3.dim}], got {tuple(g.shape)}")
         tdt = {np.float32: torch.float32, np.float64: torch.float64}[self.irrep_dtype]
-        if x.dtype != tdt or y.dtype != tdt or w.dtype != tdt:
-            raise TypeError(f"tensors must be {tdt}")
+        data = (("L1_in", x), ("L2_in", y), ("weights", w)) + ((("L3_grad", g),) if g is not None else ())
+        for name, t in data:
+            if t.dtype != tdt:
+                raise TypeError(f"tensors must be {tdt}")
+            if not t.is_cuda:
+                raise ValueError(f"{name} is on {t.device}: all tensors must be on the GPU (there is no CPU implementation)")
+            if t.device != x.device:
+                raise ValueError(f"{name} is on {t.device}, L1_in on {x.device}: all tensors must share one device")
 
     # ------------------------------------------------------------------ timing
     def benchmark_forward(self, num_warmup: int, num_iter: int, L1_in, L2_in, L3_buffer, weights) -> np.ndarray:

@@ -49,6 +49,10 @@ class Case:
     forward: Callable[[], None]
     backward: Callable[[], None]
     host: Dict[str, np.ndarray] = field(default_factory=dict)
+    # convolutions: the same launches including the graph preparation (CSR pointers, position lists,
+    # node order), which ``forward`` / ``backward`` reuse from the workspace
+    forward_with_prep: Optional[Callable[[], None]] = None
+    backward_with_prep: Optional[Callable[[], None]] = None
 
 
 @dataclass
@@ -70,6 +74,14 @@ class Workload:
     w_scale: float = 1.0
     alg_bytes: Dict[str, int] = field(default_factory=dict)
     alg_flops: Dict[str, int] = field(default_factory=dict)
+    # True: X, W and G are drawn on the GPU with torch's generator (the large workload's weights
+    # are 10.6 GB; drawing them on the host takes minutes); the graph and Y still come from numpy
+    device_inputs: bool = False
+
+    @property
+    def data_note(self) -> str:
+        return ("synthetic (graph and Y seeded on the host, X / W / dZ drawn on the GPU)" if self.device_inputs
+                else "synthetic")
 
     def read_write_split(self, direction: str):
         """(bytes read, bytes written) of the algorithmic traffic of one launch."""
@@ -138,10 +150,12 @@ class Workload:
             h["rows"], h["cols"] = rows, cols
             if tperm is not None:
                 h["tperm"] = tperm
-            h["X"] = _normal(rng, (self.nodes, d1), dt)
+            if not self.device_inputs:
+                h["X"] = _normal(rng, (self.nodes, d1), dt)
             h["Y"] = spherical_harmonics(self.sh_lmax, random_unit_vectors(E, rng)).astype(dt)
-            h["W"] = _normal(rng, (E, wn), dt)
-            h["G"] = _normal(rng, (self.nodes, d3), dt)
+            if not self.device_inputs:
+                h["W"] = _normal(rng, (E, wn), dt)
+                h["G"] = _normal(rng, (self.nodes, d3), dt)
         return prob, h
 
     # -------------------------------------------------------------------- build
@@ -149,6 +163,17 @@ class Workload:
         import torch
         prob, h = self.host_inputs()
         t = {k: torch.from_numpy(v).to(device) for k, v in h.items()}
+        if self.device_inputs:
+            gen = torch.Generator(device=device)
+            gen.manual_seed(self.seed)
+            tdt = torch.float32 if self.dtype == "f32" else torch.float64
+            E = h["rows"].size
+            t["X"] = torch.randn(self.nodes, prob.irreps_in1.dim, device=device, dtype=tdt, generator=gen)
+            t["W"] = torch.randn(E, prob.weight_numel, device=device, dtype=tdt, generator=gen)
+            t["G"] = torch.randn(self.nodes, prob.irreps_out.dim, device=device, dtype=tdt, generator=gen)
+            # the host copies the CPU baseline needs: node tensors whole, per-edge ones for a sample
+            h["X"], h["G"] = t["X"].cpu().numpy(), t["G"].cpu().numpy()
+            h["W"] = t["W"][:8192].cpu().numpy()
         stream = torch.cuda.current_stream().cuda_stream
         if self.kind == "tp":
             op = TensorProduct(prob, torch_op=True)
@@ -176,16 +201,22 @@ class Workload:
             ws = op.workspace_ptr(E, N)
             det = self.deterministic
 
-            def fwd():
+            def fwd(prepared=True):
                 if not op.forward_overwrites:
                     t["Z"].zero_()              # atomic kernels accumulate: part of the operator's work
-                op.exec_conv_rawptrs(p["X"], p["Y"], p["W"], p["Z"], p["rows"], p["cols"], E, N, ws, tp_ptr, stream)
+                op.exec_conv_rawptrs(p["X"], p["Y"], p["W"], p["Z"], p["rows"], p["cols"], E, N, ws, tp_ptr, stream,
+                                     prepared=prepared)
 
-            def bwd():
+            def bwd(prepared=True):
                 if not op.backward_overwrites:
                     t["Xg"].zero_()             # likewise for the backward that scatters dX with atomics
                 op.backward_rawptrs(p["X"], p["Xg"], p["Y"], p["Yg"], p["W"], p["Wg"], p["G"], p["rows"], p["cols"],
-                                    E, N, ws, tp_ptr, stream)
+                                    E, N, ws, tp_ptr, stream, prepared=prepared)
+            # a model calls one graph many times (forward, backward and double backward of every layer):
+            # the graph is prepared once, here, and the timed launches reuse the workspace
+            fwd(False)
+            bwd(False)
+            return Case(op, t, fwd, bwd, h, lambda: fwd(False), lambda: bwd(False))
         return Case(op, t, fwd, bwd, h)
 
     def _fill_conv_bytes(self, prob, E, N):
@@ -232,7 +263,8 @@ def get(name: str) -> Workload:
                         "Poisson(40) in-degree (~800000 edges), fp32, forward+backward, "
                         + ("deterministic" if det else "atomic"),
                         "conv", LARGE, 800000, "edges/s", "hbm", "f32", 12349,
-                        {"nodes": 20000, "paths": 13, "deterministic": det}, nodes=20000, deterministic=det, sh_lmax=3)
+                        {"nodes": 20000, "paths": 13, "deterministic": det}, nodes=20000, deterministic=det, sh_lmax=3,
+                        device_inputs=True)
     if name in ("mace_conv_det", "mace_conv_atomic"):
         det = name.endswith("det")
         return Workload(name, "MACE-style fused uvu conv (the problem of the tensor-product benchmark as a convolution), "
@@ -250,7 +282,8 @@ def get(name: str) -> Workload:
                         "either parity, 18 paths, 20000 nodes, Poisson(40) in-degree (~800000 edges), fp32, "
                         "forward+backward, deterministic",
                         "conv", LARGE_ALL, 800000, "edges/s", "hbm", "f32", 12349,
-                        {"nodes": 20000, "paths": 18, "deterministic": True}, nodes=20000, deterministic=True, sh_lmax=3)
+                        {"nodes": 20000, "paths": 18, "deterministic": True}, nodes=20000, deterministic=True, sh_lmax=3,
+                        device_inputs=True)
     if name in ("dense_uvw_f32", "dense_uvw_f64"):
         dt = "f32" if name.endswith("f32") else "f64"
         w = Workload(name, "dense uvw TP with shared weights, 64x0e+64x1o+64x2e (x) SH(lmax 2) -> 64x0e+64x1o+64x2e, "

@@ -21,7 +21,7 @@ import sys
 
 import numpy as np
 
-LMAX = 4
+LMAX = 7
 
 SH2, SH3 = "1x0e+1x1o+1x2e", "1x0e+1x1o+1x2e+1x3o"
 

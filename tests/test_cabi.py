@@ -33,9 +33,12 @@ def test_every_declared_symbol_is_exported():
 
 def test_step_struct_matches_header():
     fields = re.search(r"typedef struct \{(.*?)\} oeq_step;", HEADER, flags=re.S).group(1)
-    order = re.findall(r"\b(kernel|num_threads|smem|grid_kind|work_per_block|num_blocks|grid_y|warp_size)\b[\[;]", fields)
+    order = re.findall(r"\b(kernel|num_threads|smem|grid_kind|work_per_block|num_blocks|grid_y|warp_size|flags)\b[\[;]", fields)
     assert order == [f[0] for f in rt.Step._fields_]
-    assert ctypes.sizeof(rt.Step) == 64 + 7 * 4
+    assert ctypes.sizeof(rt.Step) == 64 + 8 * 4
+    for name in ("OEQ_STEP_NEEDS_WORKSPACE", "OEQ_STEP_NEEDS_TPERM", "OEQ_STEP_GRAPH_PREP"):
+        value = int(re.search(name + r"\s*=\s*(\d+)", HEADER).group(1))
+        assert value == getattr(rt, name[4:])
 
 
 def test_hiprtc_compiles_for_gfx950_without_a_gpu_and_reports_errors():
@@ -49,5 +52,8 @@ def test_error_reporting_without_device():
     L = rt.lib()
     assert L.oeq_tp_forward(None, 1, None, None, None, None, None, None) != 0
     assert b"null handle" in L.oeq_last_error()
+    for fn in (L.oeq_conv_forward, L.oeq_conv_forward_prepared):
+        assert fn(None, None, None, None, None, None, None, 0, 0, None, None, None) != 0
+        assert b"null handle" in L.oeq_last_error()
     n = ctypes.c_int(-1)
     assert L.oeq_device_count(ctypes.byref(n)) == 0 and n.value >= 0

@@ -55,6 +55,61 @@ def test_convolution_rejects_bad_inputs(cuda, deterministic):
         assert torch.isfinite(z).all()
 
 
+@pytest.mark.parametrize("deterministic", [False, True])
+def test_pointers_that_kernels_would_dereference_are_checked_first(cuda, deterministic):
+    """Host tensors among GPU tensors, a missing transpose permutation and a NULL workspace are
+    rejected on the host, in Python and again behind the C ABI; no kernel is launched with them."""
+    import torch
+    import openequivariance_amd as oeq
+    from openequivariance_amd import runtime as rt
+    prob, _ = common.channelwise(common.NEQUIP)
+    conv = oeq.TensorProductConv(prob, torch_op=True, deterministic=deterministic)
+    x, y, w = torch.randn(6, 288, device=cuda), torch.randn(12, 9, device=cuda), torch.randn(12, 352, device=cuda)
+    rows = torch.arange(12, device=cuda) // 2
+    cols = (rows + 1) % 6
+    extra = [torch.argsort(cols * 6 + rows, stable=True)] if deterministic else []
+    with pytest.raises(ValueError, match="must be on the GPU"):
+        conv.forward(x, y, w, rows.cpu(), cols, *extra)
+    with pytest.raises(ValueError, match="must be on the GPU"):
+        conv.forward(x, y.cpu(), w, rows, cols, *extra)
+    if deterministic:
+        with pytest.raises(ValueError, match="must be on the GPU"):
+            conv.forward(x, y, w, rows, cols, extra[0].cpu())
+        z, xg, yg, wg = torch.empty(6, 1120, device=cuda), torch.empty_like(x), torch.empty_like(y), torch.empty_like(w)
+        with pytest.raises(ValueError, match="transpose_perm"):
+            conv.backward_rawptrs(x.data_ptr(), xg.data_ptr(), y.data_ptr(), yg.data_ptr(), w.data_ptr(), wg.data_ptr(),
+                                  z.data_ptr(), rows.data_ptr(), cols.data_ptr(), 12, 6)
+        with pytest.raises(RuntimeError, match="transpose permutation"):      # the library checks again
+            conv.internal.backward_rawptrs(x.data_ptr(), xg.data_ptr(), y.data_ptr(), yg.data_ptr(), w.data_ptr(),
+                                           wg.data_ptr(), z.data_ptr(), rows.data_ptr(), cols.data_ptr(), 12, 6,
+                                           conv.workspace_ptr(12, 6), 0, 0)
+    z = torch.empty(6, 1120, device=cuda)
+    with pytest.raises(RuntimeError, match="needs a workspace"):
+        conv.internal.exec_conv_rawptrs(x.data_ptr(), y.data_ptr(), w.data_ptr(), z.data_ptr(), rows.data_ptr(),
+                                        cols.data_ptr(), 12, 6, 0, extra[0].data_ptr() if extra else 0, 0)
+    with pytest.raises(RuntimeError, match="rows / cols"):
+        conv.internal.exec_conv_rawptrs(x.data_ptr(), y.data_ptr(), w.data_ptr(), z.data_ptr(), 0, 0, 12, 6,
+                                        conv.workspace_ptr(12, 6), 0, 0)
+    torch.cuda.synchronize()
+
+
+def test_tensor_product_rejects_host_tensors_among_gpu_tensors(cuda):
+    import torch
+    import openequivariance_amd as oeq
+    prob, _ = common.channelwise(common.NEQUIP)
+    tp = oeq.TensorProduct(prob, torch_op=True)
+    x, y, w = (torch.randn(10, d, device=cuda) for d in (288, 9, 352))
+    with pytest.raises(ValueError, match="must be on the GPU"):
+        tp(x, y.cpu(), w)
+    shared = oeq.TensorProduct(oeq.FullyConnectedTPProblem("4x0e", "1x0e", "4x0e", shared_weights=True,
+                                                           internal_weights=False), torch_op=True)
+    xs, ys, ws_ = torch.randn(5, 4, device=cuda), torch.randn(5, 1, device=cuda), torch.randn(16, device=cuda)
+    zs = torch.empty(5, 4, device=cuda)
+    with pytest.raises(RuntimeError, match="needs a workspace"):     # behind the C ABI as well
+        shared.internal.exec_tensor_product(5, xs.data_ptr(), ys.data_ptr(), zs.data_ptr(), ws_.data_ptr(), 0, 0)
+    torch.cuda.synchronize()
+
+
 def test_unsupported_problems_raise():
     import openequivariance_amd as oeq
     with pytest.raises(NotImplementedError):      # uvw needs multiplicity 1 on the second operand

@@ -34,10 +34,11 @@ def test_random_convolution(cuda, seed):
     import torch
     import openequivariance_amd as oeq
     rng = np.random.default_rng(seed)
-    irreps = _channelwise(rng, [1, 3, 8, 16, 20, 32, 48, 64, 100, 128])
-    prob, oprob = common.channelwise(irreps)
-    if not prob.instructions:
-        pytest.skip("no path is allowed for these irreps")
+    while True:                                   # drawn again until at least one path is allowed
+        irreps = _channelwise(rng, [1, 3, 8, 16, 20, 32, 48, 64, 100, 128])
+        prob, oprob = common.channelwise(irreps)
+        if prob.instructions:
+            break
     nodes, nnz = int(rng.integers(1, 80)), int(rng.integers(0, 2000))
     for deterministic in (True, False):
         rows, cols = common.random_graph(nodes, nnz, seed, self_loops=True)
@@ -66,18 +67,19 @@ def test_random_tensor_product(cuda, seed):
     dtype = np.float64 if rng.random() < 0.25 else np.float32
     tol = FP32_TOL if dtype == np.float32 else FP64_TOL
     n = int(rng.choice([1, 5, 17, 64, 300, 1111]))
-    if kind == "uvu":
-        irreps = _channelwise(rng, [1, 3, 8, 16, 20, 32, 48, 64, 100, 128, 200])
-        prob, oprob = common.channelwise(irreps, dtype=dtype)
-    else:
-        ls = sorted(rng.choice(4, size=rng.integers(1, 4), replace=False))
-        mul = lambda: int(rng.choice([1, 4, 16, 20, 32, 48, 64, 96]))
-        irreps = ("+".join(f"{mul()}x{l}{_par(l)}" for l in ls),
-                  "+".join(f"1x{l}{_par(l)}" for l in range(int(rng.integers(0, 4)) + 1)),
-                  "+".join(f"{mul()}x{l}{_par(l)}" for l in range(int(rng.integers(0, 4)) + 1)))
-        prob, oprob = common.fully_connected(irreps, shared=(kind == "uvw_shared"), dtype=dtype)
-    if not prob.instructions:
-        pytest.skip("no path is allowed for these irreps")
+    while True:                                   # drawn again until at least one path is allowed
+        if kind == "uvu":
+            irreps = _channelwise(rng, [1, 3, 8, 16, 20, 32, 48, 64, 100, 128, 200])
+            prob, oprob = common.channelwise(irreps, dtype=dtype)
+        else:
+            ls = sorted(rng.choice(4, size=rng.integers(1, 4), replace=False))
+            mul = lambda: int(rng.choice([1, 4, 16, 20, 32, 48, 64, 96]))
+            irreps = ("+".join(f"{mul()}x{l}{_par(l)}" for l in ls),
+                      "+".join(f"1x{l}{_par(l)}" for l in range(int(rng.integers(0, 4)) + 1)),
+                      "+".join(f"{mul()}x{l}{_par(l)}" for l in range(int(rng.integers(0, 4)) + 1)))
+            prob, oprob = common.fully_connected(irreps, shared=(kind == "uvw_shared"), dtype=dtype)
+        if prob.instructions:
+            break
     print(f"seed={seed} {kind} {dtype.__name__} {irreps} paths={len(prob.instructions)} n={n}", flush=True)
     tp = oeq.TensorProduct(prob, torch_op=True)
     X, Y, We, G = common.tp_inputs(prob, n, seed, dtype, w_scale=0.3)

@@ -136,7 +136,9 @@ def test_unsorted_conv_backward_selection(monkeypatch):
     assert [s["kernel"] for s in bwd] == ["group_clear_backward", "group_count_backward", "group_scan_backward",
                                           "group_fill_backward", "order_backward", "backward", "backward_dy_reduce"]
     assert bwd[5]["grid_y"] == 4 and bwd[5]["work_per_block"] == 1
-    assert ws(1000, 10) == (2 * 11 + 1000 + 10) * 8 + 4 * 1000 * 16 * 4
+    # the forward's grouping and the backward's lie side by side (a prepared workspace serves both)
+    assert ws(1000, 10) == (2 * (2 * 11 + 1000) + 10) * 8 + 4 * 1000 * 16 * 4
+    assert all(s.get("prep") for s in bwd[:5]) and not any(s.get("prep") for s in bwd[5:])
     src = large.render()
     for name in ("group_fill_backward", "backward_dy_reduce", "void backward("):
         assert name in src

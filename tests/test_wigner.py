@@ -14,8 +14,9 @@ TRIPLES = [tuple(map(int, k.split("_"))) for k in GOLDEN.files]
 
 @pytest.mark.parametrize("impl", [w3j_oracle, w3j_product], ids=["oracle", "product"])
 def test_matches_reference_golden_vectors(impl):
-    """65 tensors (l <= 4) written from the reference's own wigner_3j: fixes the sign convention."""
-    assert len(TRIPLES) == 65
+    """260 tensors (l1, l2, l3 <= 7: everything the problem families of the benchmarks use) written from
+    the reference's own wigner_3j: fixes the sign convention."""
+    assert len(TRIPLES) == 260 and max(max(t) for t in TRIPLES) == 7
     for (l1, l2, l3) in TRIPLES:
         np.testing.assert_allclose(impl(l1, l2, l3), GOLDEN[f"{l1}_{l2}_{l3}"], atol=1e-13, rtol=0)
 
