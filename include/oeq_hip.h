@@ -143,6 +143,19 @@ int  oeq_conv_backward_prepared(oeq_conv* conv, const void* L1_in, void* L1_grad
                                 const void* rows, const void* cols, uint64_t nnz, uint64_t node_count,
                                 void* workspace, const void* transpose_perm, void* stream);
 
+/* oeq_conv_forward for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * The workspace is a static device array of OEQ_NOALLOC_SCRATCH_BYTES inside the library (one copy
+ * per GPU, held until the process ends); the call allocates and frees nothing.  The forward kernels
+ * use 8 * (2 * (node_count + 1) + nnz) bytes of it; larger graphs are rejected with an error.  All
+ * calls on one GPU share the array: calls that overlap in time on one GPU (different streams or
+ * threads) race on it, and a captured graph holding such a call must not replay concurrently with
+ * another.  Inputs and outputs are the caller's, as in oeq_conv_forward. */
+#define OEQ_NOALLOC_SCRATCH_BYTES (16u << 20)
+int  oeq_conv_forward_noalloc(oeq_conv* conv, const void* L1_in, const void* L2_in, const void* weights,
+                              void* L3_out, const void* rows, const void* cols, uint64_t nnz,
+                              uint64_t node_count, const void* transpose_perm, void* stream);
+
 /* ------------------------------------------------------------ generic module */
 /* Thin access to a loaded code object, for callers that pack their own arguments
  * (HIPJITKernel::execute, extension/util/backend_hip.hpp:266-283). */

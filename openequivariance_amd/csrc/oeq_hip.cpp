@@ -14,8 +14,14 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <vector>
+
+// Scratch of oeq_conv_forward_noalloc: device memory that exists from the moment the library is
+// loaded, one copy per GPU.  Host code never uses this name as an address; it asks the runtime for
+// the array's device address once per device (noalloc_scratch) and passes that to the kernels.
+static __device__ __align__(256) unsigned char oeq_noalloc_scratch[OEQ_NOALLOC_SCRATCH_BYTES];
 
 namespace {
 
@@ -328,6 +334,42 @@ int oeq_conv_backward_prepared(oeq_conv* c, const void* L1, void* L1g, const voi
                                void* Wg, const void* L3g, const void* rows, const void* cols, uint64_t nnz,
                                uint64_t node_count, void* workspace, const void* tperm, void* stream) {
     return conv_backward(c, L1, L1g, L2, L2g, W, Wg, L3g, rows, cols, nnz, node_count, workspace, tperm, stream, true);
+}
+
+// Device address of this GPU's copy of oeq_noalloc_scratch, looked up on first use per device.
+static int noalloc_scratch(void** out) {
+    enum { MAX_DEVICES = 64 };
+    static void* ptrs[MAX_DEVICES] = {nullptr};
+    static std::mutex mu;
+    int dev = -1;
+    OEQ_HIP_CHECK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MAX_DEVICES) return fail("device ordinal %d is out of range", dev);
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptrs[dev]) {
+        void* p = nullptr;
+        OEQ_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(oeq_noalloc_scratch)));
+        if (!p) return fail("hipGetSymbolAddress returned a null address for the static scratch");
+        ptrs[dev] = p;
+    }
+    *out = ptrs[dev];
+    return 0;
+}
+
+int oeq_conv_forward_noalloc(oeq_conv* c, const void* L1, const void* L2, const void* W, void* L3,
+                             const void* rows, const void* cols, uint64_t nnz, uint64_t node_count,
+                             const void* tperm, void* stream) {
+    if (!c) return fail("null handle");
+    // bytes the forward kernels of any plan use: two pointer arrays and one position list, int64
+    if (nnz > (1ull << 40) || node_count > (1ull << 40)) return fail("graph too large");
+    const uint64_t need = 8ull * (2ull * (node_count + 1ull) + nnz);
+    if (need > (uint64_t)OEQ_NOALLOC_SCRATCH_BYTES)
+        return fail("oeq_conv_forward_noalloc: %llu edges and %llu nodes need %llu bytes of scratch, the static "
+                    "scratch holds %llu (use oeq_conv_forward with a caller-owned workspace)",
+                    (unsigned long long)nnz, (unsigned long long)node_count, (unsigned long long)need,
+                    (unsigned long long)OEQ_NOALLOC_SCRATCH_BYTES);
+    void* scratch = nullptr;
+    if (noalloc_scratch(&scratch)) return 1;
+    return conv_forward(c, L1, L2, W, L3, rows, cols, nnz, node_count, scratch, tperm, stream, false);
 }
 
 // ---------------------------------------------------------- generic module

@@ -21,6 +21,7 @@ TARGET_ARCH = "gfx950"
 
 GRID_FIXED, GRID_PER_ROW, GRID_PER_NODE = 0, 1, 2
 STEP_NEEDS_WORKSPACE, STEP_NEEDS_TPERM, STEP_GRAPH_PREP = 1, 2, 4
+NOALLOC_SCRATCH_BYTES = 16 << 20        # OEQ_NOALLOC_SCRATCH_BYTES
 
 
 class DeviceProp(C.Structure):
@@ -90,6 +91,7 @@ def lib() -> C.CDLL:
             "oeq_conv_backward": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, u64, u64, vp, vp, vp]),
             "oeq_conv_forward_prepared": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, u64, u64, vp, vp, vp]),
             "oeq_conv_backward_prepared": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, u64, u64, vp, vp, vp]),
+            "oeq_conv_forward_noalloc": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, u64, u64, vp, vp]),
             "oeq_module_load": (C.c_int, [vp, sz, C.POINTER(vp)]),
             "oeq_module_unload": (None, [vp]),
             "oeq_module_launch": (C.c_int, [vp, C.c_char_p, C.c_uint32, C.c_uint32, C.c_uint32, vp, C.POINTER(vp)]),
@@ -116,7 +118,7 @@ EXPORTED_SYMBOLS = [
     "oeq_last_error", "oeq_device_props", "oeq_device_count", "oeq_compile", "oeq_free", "oeq_hiprtc_version",
     "oeq_tp_create", "oeq_tp_destroy", "oeq_tp_forward", "oeq_tp_backward",
     "oeq_conv_create", "oeq_conv_destroy", "oeq_conv_forward", "oeq_conv_backward",
-    "oeq_conv_forward_prepared", "oeq_conv_backward_prepared",
+    "oeq_conv_forward_prepared", "oeq_conv_backward_prepared", "oeq_conv_forward_noalloc",
     "oeq_module_load", "oeq_module_unload", "oeq_module_launch",
     "oeq_timer_create", "oeq_timer_destroy", "oeq_timer_start", "oeq_timer_stop", "oeq_timer_clear_cache",
     "oeq_buffer_alloc", "oeq_buffer_free", "oeq_buffer_h2d", "oeq_buffer_d2h", "oeq_buffer_zero",
@@ -226,6 +228,10 @@ class ConvImpl:
         oeq_conv_forward_prepared); the preparation kernels are then not launched."""
         fn = lib().oeq_conv_forward_prepared if prepared else lib().oeq_conv_forward
         _check(fn(self._h, L1, L2, W, L3, rows, cols, nnz, node_count, workspace, tperm, stream))
+
+    def exec_conv_noalloc(self, L1, L2, W, L3, rows, cols, nnz, node_count, tperm=0, stream=0):
+        """The forward with the library's static scratch as its workspace: allocates nothing."""
+        _check(lib().oeq_conv_forward_noalloc(self._h, L1, L2, W, L3, rows, cols, nnz, node_count, tperm, stream))
 
     def backward_rawptrs(self, L1, L1g, L2, L2g, W, Wg, L3g, rows, cols, nnz, node_count,
                          workspace=0, tperm=0, stream=0, prepared=False):

@@ -41,6 +41,11 @@ def test_step_struct_matches_header():
         assert value == getattr(rt, name[4:])
 
 
+def test_static_scratch_size_matches_header():
+    shift = re.search(r"#define OEQ_NOALLOC_SCRATCH_BYTES \((\d+)u << (\d+)\)", HEADER)
+    assert int(shift.group(1)) << int(shift.group(2)) == rt.NOALLOC_SCRATCH_BYTES
+
+
 def test_hiprtc_compiles_for_gfx950_without_a_gpu_and_reports_errors():
     code = rt.compile_source('extern "C" __global__ void k(float* p) { p[threadIdx.x] = 1.0f; }', use_cache=False)
     assert code[:4] == b"\x7fELF"
@@ -55,5 +60,7 @@ def test_error_reporting_without_device():
     for fn in (L.oeq_conv_forward, L.oeq_conv_forward_prepared):
         assert fn(None, None, None, None, None, None, None, 0, 0, None, None, None) != 0
         assert b"null handle" in L.oeq_last_error()
+    assert L.oeq_conv_forward_noalloc(None, None, None, None, None, None, None, 0, 0, None, None) != 0
+    assert b"null handle" in L.oeq_last_error()
     n = ctypes.c_int(-1)
     assert L.oeq_device_count(ctypes.byref(n)) == 0 and n.value >= 0
