@@ -22,6 +22,8 @@ vector stores or as coalesced atomics; loads stay register-direct.
 """
 from __future__ import annotations
 
+import os
+
 from ..problem import TPProblem
 from .common import WAVE, Emitter
 from .uvu import Block, Path, UVUGenerator
@@ -33,7 +35,6 @@ class UVUDirectGenerator(UVUGenerator):
         super().__init__(problem, kind)
         if (kind == "conv_det" and not getattr(self, "_allow_det", False)) or self.shared:
             raise NotImplementedError("direct schedule: batch product with per-row weights and atomic convolution")
-        import os
         self.waves_per_eu = waves_per_eu or int(os.environ.get("OEQ_AMD_WAVES_PER_EU", "0"))
         # False: outputs are written with dword-aligned record stores only (for callers whose
         # output tensor is not 16-byte aligned)
@@ -43,6 +44,16 @@ class UVUDirectGenerator(UVUGenerator):
         self.lds_elems = max(stage) if stage else 0
         self.ZB = 0
         self.unroll_bwd_chunks = 1
+        # Batch product: every tensor is read or written exactly once.  The backward's loads and stores
+        # carry the non-temporal hint (measured on the 128-channel MACE problem, warm and with flushed
+        # caches alike: 0.63 -> 0.56 ms); on the forward the hint measured slower (stores: 0.46 -> 0.52 ms
+        # with flushed caches), so it keeps plain accesses.  OEQ_AMD_TP_NT lists the accesses that get the
+        # hint (fl, fs, bl, bs = forward / backward loads / stores) for A/B runs.  Writing the backward's dX
+        # through the LDS slot as full-line vector stores (OEQ_AMD_TP_DX_LDS=1) measured a tie and costs
+        # 37 registers, so dX keeps its record stores.
+        self._nt_modes = set(os.environ.get("OEQ_AMD_TP_NT", "bl,bs").split(",")) if kind == "tp" else set()
+        self.nt_load = self.nt_store = False
+        self.dx_via_lds = (kind == "tp") and os.environ.get("OEQ_AMD_TP_DX_LDS", "0") == "1"
         # one row per wavefront: the row index is wave-uniform and an out-of-range wavefront exits
         self.uniform_rows = (self.R == 1)
         self._cur_c = None
@@ -102,7 +113,9 @@ class UVUDirectGenerator(UVUGenerator):
                 E(f"  const bool ok = {ok};")
                 guard = f"q < {total} && ok"
                 tgt = f"{ptr} + grow * {rowdim} + {blk.off} + (q - r * {per_row}) * {unit}"
-            if op == "store":
+            if op == "store" and self.nt_store:
+                E(f"  if ({guard}) __builtin_nontemporal_store(*(const VT*)(lds + {base} + q * {unit}), (VT*)({tgt})); }}")
+            elif op == "store":
                 E(f"  if ({guard}) *(VT*)({tgt}) = *(const VT*)(lds + {base} + q * {unit}); }}")
             else:
                 E(f"  if ({guard}) oeq_atomic_add({tgt}, lds[{base} + q]); }}")
@@ -140,17 +153,20 @@ class UVUDirectGenerator(UVUGenerator):
         lanes are clamped onto a valid row/channel).  Branch-free loads are what lets the compiler
         merge them into x3/x4 accesses and hoist them.  With ``zero`` idle lanes get 0 instead of
         the clamped lane's data (needed where the value feeds a cross-lane sum)."""
+        rd = (lambda p, k: f"oeq_ldnt({p} + {k})") if self.nt_load else (lambda p, k: f"{p}[{k}]")
         if zero and act != "true":
             E("T " + ", ".join(names) + ";")
-            E(f"{{ const T* __restrict__ p_ = {ptr}; " + " ".join(f"{n} = p_[{k}];" for k, n in enumerate(names)) + " }")
+            E(f"{{ const T* __restrict__ p_ = {ptr}; " + " ".join(f"{n} = {rd('p_', k)};" for k, n in enumerate(names)) + " }")
             E(f"if (!({act})) {{ " + " ".join(f"{n} = (T)0;" for n in names) + " }")
         else:
             E(f"const T* __restrict__ p_{names[0]} = {ptr};")
-            E("const T " + ", ".join(f"{n} = p_{names[0]}[{k}]" for k, n in enumerate(names)) + ";")
+            E("const T " + ", ".join(f"{n} = {rd('p_' + names[0], k)}" for k, n in enumerate(names)) + ";")
 
     def emit_record_store(self, E: Emitter, names, ptr: str, act: str, op: str = "store") -> None:
         if op == "atomic":
             E(f"if ({act}) {{ T* __restrict__ p_ = {ptr}; " + " ".join(f"oeq_atomic_add(p_ + {k}, {n});" for k, n in enumerate(names)) + " }")
+        elif self.nt_store:
+            E(f"if ({act}) {{ T* __restrict__ p_ = {ptr}; " + " ".join(f"oeq_stnt(p_ + {k}, {n});" for k, n in enumerate(names)) + " }")
         else:
             E(f"if ({act}) {{ T* __restrict__ p_ = {ptr}; " + " ".join(f"p_[{k}] = {n};" for k, n in enumerate(names)) + " }")
 
@@ -167,7 +183,8 @@ class UVUDirectGenerator(UVUGenerator):
         ue = self.uexpr(c)
         for p in self.paths:
             for v in range(p.mv):
-                E(f"const T W{tag}_{p.t}_{v} = {wptr}[{self.widx(p, self.uclamp(p.a, c), v)}];")
+                idx = self.widx(p, self.uclamp(p.a, c), v)
+                E(f"const T W{tag}_{p.t}_{v} = " + (f"oeq_ldnt({wptr} + {idx});" if self.nt_load else f"{wptr}[{idx}];"))
 
     def emit_x_preload(self, E: Emitter, c, xrow: str) -> None:
         tag = c if isinstance(c, int) else "c"
@@ -244,6 +261,7 @@ class UVUDirectGenerator(UVUGenerator):
     def direct_forward_body(self) -> str:
         E = Emitter()
         atomic = (self.kind == "conv_atomic")
+        self.nt_load, self.nt_store = "fl" in self._nt_modes, "fs" in self._nt_modes
         self.emit_lane_direct(E, lds=True)
         xrow, zrow, _ = self._rows(E)
         self.emit_y_load_direct(E)
@@ -279,7 +297,8 @@ class UVUDirectGenerator(UVUGenerator):
     def direct_backward_body(self) -> str:
         E = Emitter()
         atomic = (self.kind == "conv_atomic")
-        self.emit_lane_direct(E, lds=atomic)
+        self.nt_load, self.nt_store = "bl" in self._nt_modes, "bs" in self._nt_modes
+        self.emit_lane_direct(E, lds=atomic or self.dx_via_lds)
         xrow, zrow, srow = self._rows(E, backward=True)
         E(f"T* __restrict__ Wgr = Wg + {srow} * {self.WN};")
         self.emit_y_load_direct(E)
@@ -308,7 +327,10 @@ class UVUDirectGenerator(UVUGenerator):
                     E(f"const T g{k} = G{oi}_{k};")
 
                 def sink(E, p, v, expr):
-                    E(f"  if ({self.act(p.a)}) Wgr[{self.widx(p, 'u', v)}] = {expr};")
+                    if self.nt_store:
+                        E(f"  if ({self.act(p.a)}) oeq_stnt(Wgr + {self.widx(p, 'u', v)}, {expr});")
+                    else:
+                        E(f"  if ({self.act(p.a)}) Wgr[{self.widx(p, 'u', v)}] = {expr};")
                 self.emit_backward_block(E, o, "Wr", sink)
                 E.level -= 1
                 E("}")
@@ -317,7 +339,7 @@ class UVUDirectGenerator(UVUGenerator):
                     continue
                 if a.idx in self.used_in1:
                     self.emit_block_store(E, a, [f"dx{a.idx}_{m}" for m in range(a.D)], "Xg", self.D1, xrow,
-                                          self.xrow_of, "atomic" if atomic else "store", via_lds=atomic)
+                                          self.xrow_of, "atomic" if atomic else "store", via_lds=atomic or self.dx_via_lds)
                 elif not atomic:
                     self.emit_record_store(E, ["(T)0"] * a.D, f"Xg + (u64){xrow} * {self.D1} + {a.off} + u * {a.D}",
                                            self.act(a))
