@@ -39,7 +39,8 @@ class UVUDetGenerator(UVUDirectGenerator):
     SPLIT_WORDS = 80
 
     def __init__(self, problem: TPProblem, prefetch_backward=None, vector_stores: bool = True,
-                 forward_perm: bool = False, backward_perm: bool = False, idx_ctype: str = "i64"):
+                 forward_perm: bool = False, backward_perm: bool = False, idx_ctype: str = "i64",
+                 allow_split: bool = True):
         super().__init__(problem, "conv_det", vector_stores=vector_stores)
         self.idx_ctype = idx_ctype
         # True: the forward walks the receiver-grouped edge order listed in the workspace (built on
@@ -79,7 +80,7 @@ class UVUDetGenerator(UVUDirectGenerator):
         H = 1
         split_env = os.environ.get("OEQ_AMD_DET_SPLIT", "")           # "0": never; a number: threshold for A/B runs
         limit = int(split_env) if split_env.isdigit() and split_env != "0" else self.SPLIT_WORDS
-        if words > limit and split_env != "0":
+        if words > limit and split_env != "0" and allow_split:
             H = min(len(self.used_out), -(-words // 64))
         self.out_groups = [[] for _ in range(H)]
         for oi in sorted(self.used_out, key=lambda i: -(self.out[i].D + len(self.paths_into(i)))):
@@ -135,6 +136,11 @@ class UVUDetGenerator(UVUDirectGenerator):
     def backward_kernels(self):
         """(kernel name, group) of the backward launches, in launch order."""
         return [("backward" if h == 0 else f"backward_g{h}", h) for h in range(self.H)]
+
+    def backward_kernel_sources(self):
+        """The backward's compute kernels as the templates emit them: name, workgroup size, attributes, body."""
+        return [dict(name=name, threads=64, attr=self.backward_attr(), body=self.conv_det_backward_body(h))
+                for name, h in self.backward_kernels()]
 
     def act(self, blk):
         return "rv" if self.full(blk) else f"(rv && u < {blk.mul})"
@@ -312,7 +318,8 @@ class UVUDetGenerator(UVUDirectGenerator):
     def uclamp(self, blk, c) -> str:
         return "u" if self.full(blk) else f"min(u, {blk.mul - 1})"
 
-    def emit_pingpong_loop(self, E: Emitter, names, load_idx, load, compute, prefetch_first: bool = True) -> None:
+    def emit_pingpong_loop(self, E: Emitter, names, load_idx, load, compute, prefetch_first: bool = True,
+                           pre=None, index_decl: str = None) -> None:
         """The edge loop as a three-stage software pipeline.  Stage 1 (two iterations ahead) resolves
         the indices of an edge - a chain of dependent loads: position list, edge id, neighbour row - into
         one of two index sets; stage 2 (one iteration ahead) requests the edge's operands into one of two
@@ -322,11 +329,14 @@ class UVUDetGenerator(UVUDirectGenerator):
         index set q for iteration ``it``, ``load(E, h, q)`` register set h from index set q, and
         ``compute(E, h)`` sees the operand names without prefix and the edge as ``cur_e`` / ``cur_rv``.
         ``prefetch_first=False`` (large register footprints) keeps one register set and requests the next
-        edge's operands after the arithmetic; its indices are still resolved an iteration early."""
+        edge's operands after the arithmetic; its indices are still resolved an iteration early.
+        ``pre(E, h)``, when given, is emitted in front of the prefetch requests of every iteration (loads it
+        issues are then older than the prefetch and can be waited for without draining it); it sees the
+        current edge as index set h.  ``index_decl`` replaces the declaration of the two index sets."""
         nsets = 2 if prefetch_first else 1
         for h in range(nsets):
             E("T " + ", ".join(f"S{h}{n} = (T)0" for n in names) + ";")
-        E("u64 I0e = 0, I1e = 0, I0n = 0, I1n = 0; bool I0rv = false, I1rv = false;")
+        E(index_decl or "u64 I0e = 0, I1e = 0, I0n = 0, I1n = 0; bool I0rv = false, I1rv = false;")
         E("if (maxlen > 0) {")
         E.level += 1
         load_idx(E, "0", 0)
@@ -348,6 +358,8 @@ class UVUDetGenerator(UVUDirectGenerator):
             hs = h if prefetch_first else 0
             E("const T " + ", ".join(f"{n} = S{hs}{n}" for n in names) + ";")
             E(f"const u64 cur_e = I{h}e; const bool cur_rv = I{h}rv; (void)cur_e; (void)cur_rv;")
+            if pre:
+                pre(E, h)
             if prefetch_first:
                 E(f"if (it + {h + 1} < maxlen) {{")
                 E.level += 1

@@ -1,0 +1,254 @@
+"""Deterministic fused convolution whose backward walks the edges in receiver order, in two passes.
+
+The segmented backward of ``uvu_det.py`` owns one sender per wavefront and gathers a whole row of dZ
+per edge: with d3 values per row that is E * d3 words of gathered traffic, the largest stream of the
+kernel.  Here the edge list is walked in the order it is given (sorted by receiver):
+
+* pass 1 (``backward``): a wavefront owns a tile of consecutive edges and one 64-channel chunk.  It
+  keeps ``dZ[receiver]`` of the chunk in registers and reloads it only when the receiver changes
+  (about once per in-degree edges), gathers ``X[sender]`` per edge (d1 words instead of d3), streams W
+  and Y, writes dW[e] and dY[e], and writes the edge's contribution to dX[sender] into a spill row of
+  its own in the workspace.  Nothing is accumulated across edges, so every tile is independent and the
+  work is balanced whatever the degree distribution;
+* pass 2 (``backward_dx``): a wavefront owns (sender, chunk) and sums the spill rows of the sender's
+  edges in the order of the transpose permutation: fixed order, bit-reproducible.
+
+Traffic next to the sender-order backward: the gather shrinks from E * d3 to E * d1 words, and
+2 * E * d1 words of spill are added, so this order moves fewer bytes when d3 > 3 * d1 or so (the
+gathers of dZ are partly served by caches, the spill is not).  The spill layout is this generator's
+own: word w of lane u of chunk c of edge e at ``((e * chunks + c) * words + w) * P + u``, so that
+every spill access of a wavefront is one contiguous run.
+
+Workgroup ids map to (tile, chunk) so that each XCD (id modulo 8) sweeps a contiguous range of
+tiles: the dZ row of a receiver whose edges span two tiles is then re-read from that XCD's L2.
+"""
+from __future__ import annotations
+
+import os
+
+from ..problem import TPProblem
+from .common import Emitter
+from .uvu_det import UVUDetGenerator
+
+
+class UVURecvGenerator(UVUDetGenerator):
+    MIN_TILE_ITERS = 8           # edge-loop iterations of the smallest tile
+    MAX_TILES = 16384            # tiles per chunk of the largest launches (the tile then grows with the edge count)
+    DX_UNROLL = 4                # spill rows in flight per lane group in pass 2
+
+    def __init__(self, problem: TPProblem, vector_stores: bool = True, idx_ctype: str = "i64", prefetch=None):
+        # pass 1 is one launch: the per-edge dX rows cannot be split over launches of output-block groups
+        super().__init__(problem, vector_stores=vector_stores, idx_ctype=idx_ctype, allow_split=False)
+        assert self.H == 1
+        self.lds_backward = False
+        self.waves_per_eu = 0
+        self.ordered_backward = False
+        # words of dX one lane produces per edge (= spill words per lane)
+        self.NW = sum(self.in1[i].D for i in self.used_in1)
+        self.spill_row = self.NCH * self.NW * self.P              # words per edge
+        # registers: dZ of the receiver + one or two sets of (X records, weights, Y)
+        held = sum(self.out[i].D for i in self.used_out)
+        per_edge = self.NW + sum(p.mv for p in self.paths) + len(self.used_y)
+        env = os.environ.get("OEQ_AMD_RECV_PREFETCH")
+        self.prefetch_edges = (held + 2 * per_edge <= 190) if env not in ("0", "1") else env == "1"
+        if prefetch is not None:
+            self.prefetch_edges = prefetch
+        self.dypart_off = "(2 * (node_count + 1) + node_count) * sizeof(i64)"
+        self.spill_off = (f"((({self.dypart_off} + {self.dy_slots if self.dy_slots > 1 else 0}ull * nnz * {self.D2} * sizeof(T)) "
+                          "+ 255ull) & ~255ull)")
+
+    def describe(self) -> str:
+        return super().describe() + f" receiver-order backward (spill {self.spill_row} words/edge)"
+
+    # ------------------------------------------------------------------ plan
+    def backward_steps(self):
+        steps = [dict(kernel="backward", num_threads=64, grid_kind=1, work_per_block=self.MIN_TILE_ITERS * self.R,
+                      num_blocks=self.MAX_TILES, grid_y=self.NCH),
+                 dict(kernel="backward_dx", num_threads=64, grid_kind=2, work_per_block=1, grid_y=self.NCH)]
+        if self.dy_slots > 1:
+            steps.append(dict(kernel="backward_dy_reduce", num_threads=256, grid_kind=1,
+                              work_per_block=self.dy_rows_per_block))
+        return steps
+
+    def spill_bytes(self, nnz: int) -> int:
+        return nnz * self.spill_row * self.itemsize
+
+    def plan(self):
+        fwd, bwd, _ = super().plan()
+
+        def ws(nnz=0, nodes=0):
+            head = (2 * (nodes + 1) + nodes) * 8 + self.dy_partial_bytes(nnz)
+            return ((head + 255) & ~255) + self.spill_bytes(nnz)
+        return fwd, bwd, ws
+
+    def backward_kernel_sources(self):
+        w = int(os.environ.get("OEQ_AMD_RECV_WAVES", "0"))
+        attr = f" __attribute__((amdgpu_waves_per_eu({w}, {w})))" if w else ""
+        return [dict(name="backward", threads=64, attr=attr, body=self._edges_body()),
+                dict(name="backward_dx", threads=64, attr="", body=self._dx_body())]
+
+    # ---------------------------------------------------------------- pass 1
+    def _edges_body(self) -> str:
+        E = Emitter()
+        R, P, NCH = self.R, self.P, self.NCH
+        self.emit_lane_direct(E, lds=False)
+        E("// (tile, chunk) of this workgroup: ids are dealt to the 8 XCDs round robin, each XCD gets a contiguous run of items")
+        E(f"const u64 tiles = gridDim.x, items = tiles * {NCH};")
+        E("const u64 bid = blockIdx.x + (u64)blockIdx.y * gridDim.x;")
+        E("const u64 xcd = bid & 7, turn = bid >> 3;")
+        E("const u64 item = xcd * (items >> 3) + min(xcd, items & 7) + turn;")
+        E(f"const int c = (int)(item % {NCH}); (void)c;")
+        E(f"const u64 tile = item / {NCH};")
+        E(f"const int u = c * {P} + ul;")
+        E(f"const u64 per = ((nnz + tiles - 1) / tiles + {R - 1}) / {R} * {R};       // edges per tile")
+        E("const u64 beg = min(tile * per, nnz);")
+        E("const int len = (int)(min(beg + per, nnz) - beg);")
+        E(f"const int maxlen = (len + {R - 1}) / {R};")
+        E(f"T* __restrict__ spill = (T*)((char*)ws + {self.spill_off});")
+        self._cur_c = "e"
+        E("bool rv = false;")
+        for oi in self.used_out:
+            E("T " + ", ".join(f"G{oi}_{k} = (T)0" for k in range(self.out[oi].D)) + ";")
+        E("i64 cur_rcv = -1;")
+        names = []
+        for i in self.used_in1:
+            names += [f"x{i}_{m}" for m in range(self.in1[i].D)]
+        names += [f"We_{p.t}_{v}" for p in self.paths for v in range(p.mv)]
+        names += [f"y{f}" for f in self.used_y]
+
+        def load_idx(E, it, q):
+            E("{")
+            E.level += 1
+            E(f"const bool ev = {self.edge_pos(it)} < len;")
+            E(f"const u64 e = ev ? beg + (u64){self.edge_pos(it)} : nnz - 1;      // idle lane groups re-read the last edge, masked below")
+            E("const i64 snd = cols[e], rcv = rows[e];")
+            E("const bool ok = ev && snd >= 0 && snd < (i64)node_count && rcv >= 0 && rcv < (i64)node_count;")
+            E(f"I{q}e = e; I{q}ev = ev; I{q}rv = ok; I{q}n = ok ? (u64)snd : 0; I{q}r = ok ? rcv : -1;")
+            E.level -= 1
+            E("}")
+
+        def load(E, h, q):
+            E("{")
+            E.level += 1
+            E(f"const u64 e = I{q}e, sndc = I{q}n; const bool rv = I{q}rv;")
+            E(f"const T* __restrict__ Yr = Y + e * {self.D2};")
+            E(f"const T* __restrict__ Wr = W + e * {self.WN};")
+            for f in self.used_y:
+                E(f"S{h}y{f} = {self.ld('Yr', f)};")
+            for p in self.paths:
+                for v in range(p.mv):
+                    E(f"S{h}We_{p.t}_{v} = {self.ld('Wr', self.widx(p, self.uclamp(p.a, 0), v))};")
+            for i in self.used_in1:
+                a = self.in1[i]
+                E(f"{{ const T* __restrict__ p_ = X + sndc * {self.D1} + {a.off} + {self.uclamp(a, 0)} * {a.D}; "
+                  + " ".join(f"S{h}x{i}_{m} = p_[{m}];" for m in range(a.D)) + " }")
+                # dW and dY of an edge are proportional to x: zero it for idle lanes and invalid edges
+                E(f"if (!({self.act(a)})) {{ " + " ".join(f"S{h}x{i}_{m} = (T)0;" for m in range(a.D)) + " }")
+            E.level -= 1
+            E("}")
+
+        def pre(E, h):
+            """dZ of the current edge's receiver, when it differs from the one held.  (Index set h is
+            refilled for a later iteration before the arithmetic runs: what the arithmetic needs of it is
+            copied here.)"""
+            E(f"const bool cur_ev = I{h}ev;")
+            if R == 1:
+                # the receiver is the same for all lanes: a scalar branch, loads not predicated
+                E(f"const int rcv_u = __builtin_amdgcn_readfirstlane((int)I{h}r);")
+                E("if (rcv_u >= 0 && (i64)rcv_u != cur_rcv) {")
+                E.level += 1
+                E("cur_rcv = (i64)rcv_u;")
+            else:
+                E(f"if (I{h}r >= 0 && I{h}r != cur_rcv) {{")
+                E.level += 1
+                E(f"cur_rcv = I{h}r;")
+            for oi in self.used_out:
+                o = self.out[oi]
+                E(f"{{ const T* __restrict__ p_ = G + (u64)cur_rcv * {self.D3} + {o.off} + {self.uclamp(o, 0)} * {o.D}; "
+                  + " ".join(f"G{oi}_{k} = p_[{k}];" for k in range(o.D)) + " }")
+                if not self.full(o):
+                    E(f"if (!(u < {o.mul})) {{ " + " ".join(f"G{oi}_{k} = (T)0;" for k in range(o.D)) + " }")
+            E.level -= 1
+            E("}")
+
+        def compute(E, h):
+            E("const u64 e = cur_e; rv = cur_rv;")
+            E(f"T* __restrict__ Wgr = Wg + e * {self.WN};")
+            for f in self.used_y:
+                E(f"T dy{f} = (T)0;")
+            for i in self.used_in1:
+                E("T " + ", ".join(f"dx{i}_{m} = (T)0" for m in range(self.in1[i].D)) + ";")
+            for oi in self.used_out:
+                o = self.out[oi]
+                E("{")
+                E.level += 1
+                for k in range(o.D):
+                    E(f"const T g{k} = G{oi}_{k};")
+
+                def sink(E, p, v, expr):
+                    E(f"  if ({self.act(p.a)}) {self.st('Wgr', self.widx(p, 'u', v), expr)}")
+                self.emit_backward_block(E, o, "Wr", sink)
+                E.level -= 1
+                E("}")
+            self.emit_dy_sum(E)
+            writer = "ul == 0" if P < 64 else "lane == 63"
+            E(f"if (rv && {writer}) {{")
+            if self.dy_slots > 1:
+                E(f"    T* __restrict__ Ygr = (T*)((char*)ws + DYPART_OFF) + ((u64)c * nnz + e) * {self.D2};")
+            else:
+                E(f"    T* __restrict__ Ygr = Yg + e * {self.D2};")
+            for f in range(self.D2):
+                E(f"    Ygr[{f}] = " + (f"dy{f};" if f in self.used_y else "(T)0;"))
+            E("}")
+            # this edge's contribution to dX[sender]: every slot of an existing edge is written (zeros for an
+            # edge that names no node: the dZ held belongs to another edge then)
+            E("if (cur_ev) {")
+            E(f"    T* __restrict__ sp = spill + ((e * {NCH} + c) * {self.NW}) * {P} + ul;")
+            w = 0
+            for i in self.used_in1:
+                for m in range(self.in1[i].D):
+                    E(f"    oeq_stnt(sp + {w * P}, rv ? dx{i}_{m} : (T)0);")
+                    w += 1
+            E("}")
+        self.emit_pingpong_loop(E, names, load_idx, load, compute, prefetch_first=self.prefetch_edges, pre=pre,
+                                index_decl="u64 I0e = 0, I1e = 0, I0n = 0, I1n = 0; i64 I0r = -1, I1r = -1; "
+                                           "bool I0rv = false, I1rv = false, I0ev = false, I1ev = false;")
+        return E.text()
+
+    # ---------------------------------------------------------------- pass 2
+    def _dx_body(self) -> str:
+        E = Emitter()
+        P, NCH, U = self.P, self.NCH, self.DX_UNROLL
+        self.emit_lane_direct(E, lds=False)
+        self._node_setup(E, self.bwd_ptr_off)
+        E("const IDX* __restrict__ elist = tperm;     // edge ids in (sender, receiver) order")
+        E(f"const T* __restrict__ spill = (const T*)((const char*)ws + {self.spill_off});")
+        E("T " + ", ".join(f"acc{w} = (T)0" for w in range(self.NW)) + ";")
+        E(f"for (int it = 0; it < maxlen; it += {U}) {{")
+        E.level += 1
+        for k in range(U):
+            E(f"const bool ev{k} = {self.edge_pos(f'it + {k}')} < len;")
+            E(f"const i64 raw{k} = elist[ev{k} ? (u64)(beg + {self.edge_pos(f'it + {k}')}) : (u64)(nnz - 1)];")
+        for k in range(U):
+            E(f"const bool ok{k} = ev{k} && raw{k} >= 0 && raw{k} < (i64)nnz;")
+            E(f"const T* __restrict__ sp{k} = spill + (((u64)(ok{k} ? raw{k} : 0) * {NCH} + c) * {self.NW}) * {P} + ul;")
+            E("const T " + ", ".join(f"v{k}_{w} = oeq_ldnt(sp{k} + {w * P})" for w in range(self.NW)) + ";")
+        for k in range(U):
+            E(" ".join(f"acc{w} += ok{k} ? v{k}_{w} : (T)0;" for w in range(self.NW)))
+        E.level -= 1
+        E("}")
+        E("const bool rv = nv; (void)rv;")
+        names, w = {}, 0
+        for i in self.used_in1:
+            names[i] = [f"acc{w + m}" for m in range(self.in1[i].D)]
+            w += self.in1[i].D
+        for a in self.in1:
+            if a.dim == 0:
+                continue
+            dst = f"Xg + node * {self.D1} + {a.off} + u * {a.D}"
+            if a.idx in self.used_in1:
+                self.emit_sub_sum(E, names[a.idx])
+                self.emit_record_store(E, names[a.idx], dst, self.store_act(a))
+            else:
+                self.emit_record_store(E, ["(T)0"] * a.D, dst, self.store_act(a))
+        return E.text()

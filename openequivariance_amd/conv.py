@@ -25,6 +25,7 @@ from . import runtime as rt
 from .autograd_glue import double_backward_terms
 from .codegen.uvu_det import UVUDetGenerator
 from .codegen.uvu_direct import UVUDirectGenerator
+from .codegen.uvu_recv import UVURecvGenerator
 from .codegen.uvu_sorted import UVUSortedGenerator
 from .problem import TPProblem
 from .tensor_product import _make_steps, validate_problem
@@ -96,6 +97,8 @@ def select_conv_generator(config: TPProblem, deterministic: bool, vector_stores:
     backward with coalesced atomics."""
     idx_ctype = "i64" if np.dtype(idx_dtype) == np.dtype(np.int64) else "int"
     if deterministic:
+        if os.environ.get("OEQ_AMD_DET_BACKWARD", "send") == "recv":
+            return UVURecvGenerator(config, vector_stores=vector_stores, idx_ctype=idx_ctype)
         return UVUDetGenerator(config, vector_stores=vector_stores, idx_ctype=idx_ctype)
     if os.environ.get("OEQ_AMD_CONV_FORWARD", "sorted") == "atomic":     # A/B measurements only
         g = UVUDirectGenerator(config, "conv_atomic", vector_stores=vector_stores)

@@ -300,8 +300,8 @@ def run_conv(gen, steps: Sequence[Dict], X, Y, W, rows, cols, G=None, tperm=None
     if det is not None:
         if det.ordered_backward:
             extra += CONV_EXTRA_ORDER
-        for name, h in det.backward_kernels()[1:]:
-            extra += f'        else if (k == "{name}") BWD_CALL({name});\n'
+        for k in det.backward_kernel_sources()[1:]:
+            extra += f'        else if (k == "{k["name"]}") BWD_CALL({k["name"]});\n'
         if det.dy_slots > 1:
             extra += CONV_EXTRA_DYRED
     exe = build(gen.render(prelude=emu_prelude(gen.T)), CONV_MAIN.replace("@EXTRA@", extra))

@@ -125,6 +125,26 @@ def test_conv_blocks_no_path_touches_are_zero_filled():
         assert rel_err(got, ref) < TOL
 
 
+@pytest.mark.parametrize("irreps,nodes,nnz,prefetch", [
+    (("5x0e+3x1o+70x2e", "1x0e+1x1o+1x2e", "5x0e+3x1o+70x2e+7x3o"), 5, 11, None),      # two chunks, ragged
+    (("1x0e+1x1o+16x3o", "1x0e+1x1o", "16x0e+16x0o+16x1e+16x1o"), 21, 265, None),    # four lane groups, unused block
+    (("8x0e+8x1o", "1x0e+1x1o", "8x0e+8x1o"), 9, 100, False)])                       # eight lane groups, one register set
+def test_conv_receiver_order_backward(irreps, nodes, nnz, prefetch):
+    """The two-pass backward (per-edge dX rows spilled in receiver order, summed per sender in the order
+    of the transpose permutation): tiles that end inside a receiver's edges, idle lane groups in the last
+    iteration of a tile, self loops, nodes without edges."""
+    from openequivariance_amd.codegen.uvu_recv import UVURecvGenerator
+    prob, oprob = common.channelwise(irreps)
+    g = UVURecvGenerator(prob, prefetch=prefetch)
+    rows, cols, tperm, _ = otp.coord_graph(*common.random_graph(nodes, nnz, 7, self_loops=True))
+    X, Y, W, G = common.conv_inputs(prob, nodes, nnz, 8)
+    _, bwd, ws = g.plan()
+    assert [s["kernel"] for s in bwd][:3] == ["prep_backward", "backward", "backward_dx"]
+    out = emu.run_conv(g, bwd, X, Y, W, rows, cols, G=G, tperm=tperm, ws_bytes=ws(nnz, nodes))
+    for got, ref in zip((out["Xg"], out["Yg"], out["Wg"]), otp.conv_backward(oprob, X, Y, W, G, rows, cols)):
+        assert rel_err(got, ref) < TOL
+
+
 def test_conv_det_chunked_ragged():
     irreps = ("5x0e+3x1o+70x2e", "1x0e+1x1o+1x2e", "5x0e+3x1o+70x2e+7x3o")
     prob, oprob = common.channelwise(irreps)

@@ -94,6 +94,28 @@ def test_mace_conv_backward_split_over_output_blocks(cuda, deterministic):
     _run(prob, oprob, 60, 900, 39, deterministic, sh_lmax=3)
 
 
+@pytest.mark.parametrize("which", ["nequip", "large", "mace", "ragged"])
+def test_receiver_order_backward(cuda, which, monkeypatch):
+    """The two-pass backward of the deterministic variant (OEQ_AMD_DET_BACKWARD=recv): parity, and
+    bit-equal repeats."""
+    import torch
+    from openequivariance_amd.codegen.uvu_recv import UVURecvGenerator
+    monkeypatch.setenv("OEQ_AMD_DET_BACKWARD", "recv")
+    irreps = {"nequip": common.NEQUIP, "large": common.LARGE, "mace": common.MACE,
+              "ragged": ("5x0e+3x1o+70x2e", "1x0e+1x1o+1x2e", "5x0e+3x1o+70x2e+7x3o")}[which]
+    prob, oprob = common.channelwise(irreps)
+    nodes, nnz = (300, 9001) if which == "nequip" else (50, 1500)
+    conv, (x, y, w, idx, z, g) = _run(prob, oprob, nodes, nnz, 61, True)
+    assert isinstance(conv.generator, UVURecvGenerator)
+    first = [t.grad.clone() for t in (x, y, w)]
+    for t in (x, y, w):
+        t.grad = None
+    conv.forward(x, y, w, *idx).backward(g)
+    torch.cuda.synchronize()
+    for a, b in zip(first, (x.grad, y.grad, w.grad)):
+        assert torch.equal(a, b)
+
+
 STAGED_SHAPES = {
     # one full 64-channel list, a single path, D = 1 output: every staged Y read has a constant LDS address,
     # which the compiler once moved behind the next transfer into the same slab
