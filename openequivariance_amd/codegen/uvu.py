@@ -78,6 +78,11 @@ class Path:
     def nnz(self) -> int:
         return sum(len(v) for v in self.pairs.values())
 
+    @property
+    def looped(self) -> bool:
+        """The copies v of the second operand are walked by a run-time loop instead of unrolled code."""
+        return self.b.mul > MAX_UNROLLED_V
+
     def ordered_pairs(self):
         """(i, j) pairs sorted by j then i (the reference sorts its nonzeros by (j, i, k):
         openequivariance/implementations/ComputationSchedule.py:52-66)."""
@@ -122,8 +127,6 @@ class UVUGenerator:
             a, b, o = self.in1[ins.i_in1], self.in2[ins.i_in2], self.out[ins.i_out]
             if a.mul != o.mul:
                 raise ValueError(f"uvu instruction {t}: mul(in1)={a.mul} must equal mul(out)={o.mul}")
-            if b.mul > MAX_UNROLLED_V:
-                raise NotImplementedError(f"uvu with mul(in2) = {b.mul} > {MAX_UNROLLED_V} is not supported yet")
             c = wigner_3j(a.l, b.l, o.l) * ins.path_weight
             p = Path(t, a, b, o, ins.path_weight, woff)
             for i, j, k in np.argwhere(np.abs(c) > 1e-14):
@@ -141,7 +144,17 @@ class UVUGenerator:
 
         self.used_in1 = sorted({p.a.idx for p in self.paths})
         self.used_out = sorted({p.o.idx for p in self.paths})
-        self.used_y = sorted({p.b.off + v * p.b.D + j for p in self.paths for v in range(p.mv) for (_, j) in p.pairs})
+        # Y values held in registers: those of the unrolled paths.  A second-operand block with more than
+        # MAX_UNROLLED_V copies is walked by a run-time loop over v (reference: loop_unroll_tp.cuh:48-60 and
+        # :140-175 loop over the v chunk): its Y values are read inside the loop and its dY sums are kept in LDS
+        self.used_y = sorted({p.b.off + v * p.b.D + j for p in self.paths if not p.looped
+                              for v in range(p.mv) for (_, j) in p.pairs})
+        self.looped_y = {}                   # Y column of a looped block -> slot in the LDS accumulator
+        for p in self.paths:
+            if p.looped:
+                for q in range(p.b.off, p.b.off + p.b.dim):
+                    self.looped_y.setdefault(q, len(self.looped_y))
+        self.NLY = len(self.looped_y)
 
         # lanes <-> channels over the widest block of X or Z: blocks that no path touches are zero-filled
         # through the same mapping, so it has to cover them too
@@ -185,16 +198,17 @@ class UVUGenerator:
         w = getattr(self, "waves_per_eu", 0)
         return f" __attribute__((amdgpu_waves_per_eu({w})))" if w else ""
 
-    def widx(self, p: Path, u: str, v: int) -> str:
-        """oeq-order position of weight (u, v) of path ``p`` (see weight_order.py)."""
+    def widx(self, p: Path, u: str, v) -> str:
+        """oeq-order position of weight (u, v) of path ``p`` (see weight_order.py): chunks of 32 over u
+        and v enumerated (u-chunk, v-chunk), each stored [v_local][u_local], which for any v is
+        ``(u >> 5) * 32 * mv + width(u-chunk) * v + (u & 31)``.  ``v`` is a number or a C expression."""
         mu, mv = p.mu, p.mv
         if mv == 1:
             return f"{p.woff} + {u}"
-        if mu <= 32 and mv <= 32:
-            return f"{p.woff + v * mu} + {u}"
+        if mu <= 32:
+            return (f"{p.woff + v * mu} + {u}" if isinstance(v, int) else f"{p.woff} + ({v}) * {mu} + {u}")
         ulw = "32" if mu % 32 == 0 else f"min(32, {mu} - (({u}) >> 5) * 32)"
-        vc, vl = divmod(v, 32)
-        return f"{p.woff} + (({u}) >> 5) * {32 * mv} + {ulw} * {32 * vc + vl} + (({u}) & 31)"
+        return f"{p.woff} + (({u}) >> 5) * {32 * mv} + {ulw} * ({v}) + (({u}) & 31)"
 
     def full(self, blk: Block) -> bool:
         """True when every lane of every chunk maps to a valid channel of ``blk``."""
@@ -289,6 +303,9 @@ class UVUGenerator:
             for k in range(o.D):
                 E(f"T {zname}{k} = (T)0;")
         for p in self.paths_into(o.idx):
+            if p.looped:
+                self.emit_forward_looped(E, p, wptr, zname)
+                continue
             E(f"{{ // path {p.t}: l = {p.a.l} x {p.b.l} -> {p.o.l}, coefficient {p.coeff:.9g}")
             self.emit_weights(E, p, wptr)
             for v in range(p.mv):
@@ -310,12 +327,89 @@ class UVUGenerator:
                 E("}")
             E("}")
 
+    # ------------------------------------------------- run-time loop over the copies of in2
+    def looped_weight(self, p: Path, wptr: str) -> str:
+        """Weight (u, v) of a looped path inside its v loop (zero for idle lanes)."""
+        return f"({self.act(p.a)} ? {wptr}[{self.widx(p, 'u', 'v')}] : (T)0)"
+
+    def emit_forward_looped(self, E: Emitter, p: Path, wptr: str, zname: str) -> None:
+        E(f"// path {p.t}: l = {p.a.l} x {p.b.l} -> {p.o.l}, {p.mv} copies of the second operand walked at run time")
+        E(f"for (int v = 0; v < {p.mv}; ++v) {{")
+        E.level += 1
+        E(f"const T wv = {self.looped_weight(p, wptr)};")
+        E(f"const T* __restrict__ yv = Yr + {p.b.off} + v * {p.b.D};")
+        for j in sorted({j for (_, j) in p.pairs}):
+            E(f"const T yv{j} = yv[{j}];")
+        ks_all = sorted({k for ks in p.pairs.values() for (k, _) in ks})
+        E("T " + ", ".join(f"p{k} = (T)0" for k in ks_all) + ";")
+        seen = ks_all
+        for (i, j), ks in p.ordered_pairs():
+            E(f"{{ const T t = x{p.a.idx}_{i} * yv{j};")
+            for k, val in ks:
+                E(f"  p{k} = oeq_fma({self.lit(val)}, t, p{k});")
+            E("}")
+        for k in sorted(seen):
+            E(f"{zname}{k} = oeq_fma(wv, p{k}, {zname}{k});")
+        E.level -= 1
+        E("}")
+
+    def emit_backward_looped(self, E: Emitter, p: Path, wptr: str, dw_sink) -> None:
+        """The v loop of a looped path in the backward: dW per (u, v) goes to ``dw_sink`` with v = "v", dX
+        accumulates in registers, and the dY sums of this v (over the lanes of the row) are added to the
+        row's LDS accumulator by its writer lane."""
+        E(f"// path {p.t}: l = {p.a.l} x {p.b.l} -> {p.o.l}, {p.mv} copies of the second operand walked at run time")
+        E(f"for (int v = 0; v < {p.mv}; ++v) {{")
+        E.level += 1
+        E(f"const T wv = {self.looped_weight(p, wptr)};")
+        E(f"const T* __restrict__ yv = Yr + {p.b.off} + v * {p.b.D};")
+        js = sorted({j for (_, j) in p.pairs})
+        is_ = sorted({i for (i, _) in p.pairs})
+        for j in js:
+            E(f"const T yv{j} = yv[{j}]; const T wy{j} = wv * yv{j}; T dyv{j} = (T)0;")
+        for i in is_:
+            E(f"const T wx{i} = wv * x{p.a.idx}_{i};")
+        E("T dw = (T)0;")
+        for (i, j), ks in p.ordered_pairs():
+            E("{")
+            for n_, (k, val) in enumerate(ks):
+                E(f"  T s = {self.lit(val)} * g{k};" if n_ == 0 else f"  s = oeq_fma({self.lit(val)}, g{k}, s);")
+            E(f"  dw = oeq_fma(s, x{p.a.idx}_{i} * yv{j}, dw);")
+            E(f"  dx{p.a.idx}_{i} = oeq_fma(s, wy{j}, dx{p.a.idx}_{i});")
+            E(f"  dyv{j} = oeq_fma(s, wx{i}, dyv{j});")
+            E("}")
+        dw_sink(E, p, "v", "dw")
+        for j in js:
+            if self.P == WAVE:
+                E(f"dyv{j} = oeq_wave_sum63(dyv{j});")
+            else:
+                E(f"dyv{j} = oeq_group_sum<{self.P}>(dyv{j});")
+        writer = "lane == 63" if self.P == WAVE else "ul == 0"
+        E(f"if ({writer}) {{ T* __restrict__ a_ = ylds + sub * {self.NLY} + {self.looped_y[p.b.off]} + v * {p.b.D}; "
+          + " ".join(f"a_[{j}] += dyv{j};" for j in js) + " }")
+        E.level -= 1
+        E("}")
+
+    def emit_looped_dy_begin(self, E: Emitter) -> None:
+        """LDS accumulator of the dY columns of looped blocks: one run of NLY words per row of the wavefront,
+        touched by the row's writer lane only."""
+        if not self.NLY:
+            return
+        writer = "lane == 63" if self.P == WAVE else "ul == 0"
+        E(f"__shared__ T ylds[{self.R * self.NLY}];")
+        E(f"if ({writer}) for (int q = 0; q < {self.NLY}; ++q) ylds[sub * {self.NLY} + q] = (T)0;")
+
+    def looped_dy_value(self, f: int) -> str:
+        return f"ylds[sub * {self.NLY} + {self.looped_y[f]}]"
+
     # -------------------------------------------------------- backward arithmetic
     def emit_backward_block(self, E: Emitter, o: Block, wptr: str, dw_sink) -> None:
         """Given g_k = dZ[o][u, k] (registers g0..), update dx{a}_{i}, dy{f} and hand every
         dW value to ``dw_sink(E, path, v, expr)``.  Formulas: loop_unroll_tp.cuh:167-174 of the
         reference, regrouped per (i, j) pair: s = sum_k c_ijk g_k."""
         for p in self.paths_into(o.idx):
+            if p.looped:
+                self.emit_backward_looped(E, p, wptr, dw_sink)
+                continue
             E(f"{{ // path {p.t}: l = {p.a.l} x {p.b.l} -> {p.o.l}")
             self.emit_weights(E, p, wptr)
             for v in range(p.mv):
@@ -502,7 +596,7 @@ class UVUGenerator:
         E(f"const u64 row0 = tile * {R};")
         E("const u64 row = row0 + sub;")
         E("const bool rv = row < n;")
-        E(f"const T* __restrict__ Yr = Y + row * {self.D2};")
+        E(f"const T* __restrict__ Yr = Y + (rv ? row : 0) * {self.D2};")
         E("const T* __restrict__ Wr = W" + ("" if self.shared else f" + row * {self.WN}") + ";")
         self.emit_y_load(E, "Yr", "rv")
         E("oeq_sync();")
@@ -536,23 +630,33 @@ class UVUGenerator:
         R = self.R
         ntiles = f"(n + {R - 1}) / {R}"
         if self.shared:
-            # per-workgroup dW partial sums live in registers across the tile loop
+            # per-workgroup dW partial sums live in registers across the tile loop; those of looped paths
+            # (one value per copy of the second operand) are accumulated in the workgroup's partial row itself
+            E(f"T* __restrict__ part = (T*)ws + (u64)blockIdx.x * {self.WN};")
             for p in self.paths:
                 for c in range(self.NCH):
+                    if p.looped:
+                        E(f"{{ const int u = {c * self.P} + ul; if (sub == 0 && u < {p.mu}) "
+                          f"for (int v = 0; v < {p.mv}; ++v) part[{self.widx(p, 'u', 'v')}] = (T)0; }}")
+                        continue
                     for v in range(p.mv):
                         E(f"T dws{p.t}_{c}_{v} = (T)0;")
+        if self.NLY:
+            E(f"__shared__ T ylds[{self.R * self.NLY}];")
         E(f"for (u64 tile = blockIdx.x; tile < {ntiles}; tile += gridDim.x) {{")
         E.level += 1
         E(f"const u64 row0 = tile * {R};")
         E("const u64 row = row0 + sub;")
         E("const bool rv = row < n;")
-        E(f"const T* __restrict__ Yr = Y + row * {self.D2};")
+        E(f"const T* __restrict__ Yr = Y + (rv ? row : 0) * {self.D2};")
         E("const T* __restrict__ Wr = W" + ("" if self.shared else f" + row * {self.WN}") + ";")
         if not self.shared:
             E(f"T* __restrict__ Wgr = Wg + row * {self.WN};")
         self.emit_y_load(E, "Yr", "rv")
         for f in self.used_y:
             E(f"T dy{f} = (T)0;")
+        if self.NLY:
+            E(f"if (ul == 0) for (int q = 0; q < {self.NLY}; ++q) ylds[sub * {self.NLY} + q] = (T)0;")
         E("oeq_sync();")
         self.emit_x_stage(E)
         E("oeq_sync();")
@@ -571,7 +675,15 @@ class UVUGenerator:
                 self.emit_block_in(E, o, "g", "G", self.D3, own, row_of)
 
                 def sink(E, p, v, expr):
-                    if self.shared:
+                    if self.shared and p.looped:
+                        # rows of the same wavefront hold separate sums for the same (u, v): fold them, then the
+                        # first row's lane adds to the workgroup's partial row (its own words: no other lane touches them)
+                        m = 32
+                        while m >= self.P:
+                            E(f"{expr} += oeq_shfl_xor({expr}, {m});")
+                            m //= 2
+                        E(f"if (sub == 0 && u < {p.mu}) part[{self.widx(p, 'u', v)}] += {expr};")
+                    elif self.shared:
                         if self.NCH == 1:
                             E(f"  dws{p.t}_0_{v} += {expr};")
                         else:
@@ -601,13 +713,15 @@ class UVUGenerator:
         E("if (rv && ul == 0) {")
         E(f"    T* __restrict__ Ygr = Yg + row * {self.D2};")
         for f in range(self.D2):
-            E(f"    Ygr[{f}] = " + (f"dy{f};" if f in self.used_y else "(T)0;"))
+            E(f"    Ygr[{f}] = " + (f"dy{f};" if f in self.used_y else
+                                   f"{self.looped_dy_value(f)};" if f in self.looped_y else "(T)0;"))
         E("}")
         E.level -= 1
         E("}")
         if self.shared:
-            E(f"T* __restrict__ part = (T*)ws + (u64)blockIdx.x * {self.WN};")
             for p in self.paths:
+                if p.looped:
+                    continue
                 for c in range(self.NCH):
                     for v in range(p.mv):
                         E(f"{{ const int u = {c * self.P} + ul;")

@@ -178,10 +178,17 @@ class UVUDirectGenerator(UVUGenerator):
         for v in range(p.mv):
             E(f"const T w{p.t}_{v} = W{self._cur_c}_{p.t}_{v};")
 
+    def looped_weight(self, p: Path, wptr: str) -> str:
+        """Unconditional load from the clamped channel, like every other load of this schedule."""
+        idx = self.widx(p, self.uclamp(p.a, self._loop_c), "v")
+        return f"oeq_ldnt({wptr} + {idx})" if self.nt_load else f"{wptr}[{idx}]"
+
     def emit_weight_preload(self, E: Emitter, c, wptr: str = "Wr") -> None:
         tag = c if isinstance(c, int) else "c"
-        ue = self.uexpr(c)
+        self._loop_c = c
         for p in self.paths:
+            if p.looped:
+                continue
             for v in range(p.mv):
                 idx = self.widx(p, self.uclamp(p.a, c), v)
                 E(f"const T W{tag}_{p.t}_{v} = " + (f"oeq_ldnt({wptr} + {idx});" if self.nt_load else f"{wptr}[{idx}];"))
@@ -269,7 +276,7 @@ class UVUDirectGenerator(UVUGenerator):
             self.emit_x_preload(E, c, xrow)
             self.emit_weight_preload(E, c)
         for c in range(self.NCH):
-            self._cur_c = c
+            self._cur_c = self._loop_c = c
             E("{")
             E.level += 1
             E(f"const int c = {c}; (void)c;")
@@ -304,6 +311,7 @@ class UVUDirectGenerator(UVUGenerator):
         self.emit_y_load_direct(E)
         for f in self.used_y:
             E(f"T dy{f} = (T)0;")
+        self.emit_looped_dy_begin(E)
 
         def chunk(E, c):
             tag = c if isinstance(c, int) else "c"
@@ -377,7 +385,8 @@ class UVUDirectGenerator(UVUGenerator):
             E(f"if (e < nnz && {writer}) {{")
             E(f"    T* __restrict__ Ygr = Yg + e * {self.D2};")
         for f in range(self.D2):
-            E(f"    Ygr[{f}] = " + (f"dy{f};" if f in self.used_y else "(T)0;"))
+            E(f"    Ygr[{f}] = " + (f"dy{f};" if f in self.used_y else
+                                   f"{self.looped_dy_value(f)};" if f in self.looped_y else "(T)0;"))
         E("}")
         if self.kind != "tp":
             E("if (e < nnz && !rv) {")

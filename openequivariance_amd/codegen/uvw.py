@@ -24,8 +24,9 @@ Tiling (lane = 16 * g + c, g = lane / 16, c = lane % 16; a batch tile is 16 rows
 Nothing is staged in LDS (only the 4-wave dY sum uses 2.3 KB): operands are per-lane records of
 the ``mul x irrep`` layout, loaded straight from global memory / L2.
 
-Scope of this generator: shared weights and multiplicity 1 on the second operand (the case the
-benchmarks and MACE/NequIP-style models use).  Other uvw problems raise NotImplementedError.
+Scope of this generator: shared weights.  A second operand with several copies per irrep (mul(in2) > 1)
+is handled as one contraction over u per copy v, with the slice W[:, v, :] of the weights; the
+benchmarks and MACE/NequIP-style models use a single copy.
 """
 from __future__ import annotations
 
@@ -57,6 +58,9 @@ class WPath:
     pairs: Dict[Tuple[int, int], List[Tuple[int, float]]] = field(default_factory=dict)
     wb: int = 0                     # offset (elements) of the forward-packed copy
     wa: int = 0                     # offset of the backward-packed copy
+    v: int = 0                      # which copy of the second operand this path contracts with ...
+    mv: int = 1                     # ... out of this many (the instruction's weights are [u][v][w])
+    poff: int = 0                   # offset of this path's [u][w] slice in the dense dW partial rows
 
     @property
     def mu(self) -> int:
@@ -122,14 +126,17 @@ class UVWGenerator:
             if not ins.has_weight:
                 raise NotImplementedError("instructions without weights are not supported")
             a, b, o = self.in1[ins.i_in1], self.in2[ins.i_in2], self.out[ins.i_out]
-            if b.mul != 1:
-                raise NotImplementedError("uvw tensor products need multiplicity 1 on the second operand")
             c = wigner_3j(a.l, b.l, o.l) * ins.path_weight
-            p = WPath(t, a, b, o, ins.path_weight, woff)
-            for i, j, k in np.argwhere(np.abs(c) > 1e-14):
-                p.pairs.setdefault((int(i), int(j)), []).append((int(k), float(c[i, j, k])))
-            self.paths.append(p)
-            woff += a.mul * o.mul
+            # An instruction whose second operand has mv copies is mv contractions over u, one per copy v,
+            # each with the slice W[:, v, :] of the instruction's weights and the v-th record of the Y block:
+            # it is emitted as mv paths over single-copy blocks (reference: loop_unroll_tp.cuh:48-60 walks v)
+            for v in range(b.mul):
+                bv = Block(b.idx, 1, b.l, b.off + v * b.D)
+                p = WPath(len(self.paths), a, bv, o, ins.path_weight, woff, v=v, mv=b.mul, poff=woff + v * a.mul * o.mul)
+                for i, j, k in np.argwhere(np.abs(c) > 1e-14):
+                    p.pairs.setdefault((int(i), int(j)), []).append((int(k), float(c[i, j, k])))
+                self.paths.append(p)
+            woff += a.mul * b.mul * o.mul
         if not self.paths:
             raise ValueError("Tensor product problem has no valid instructions!")
         self.used_in1 = sorted({p.a.idx for p in self.paths})
@@ -210,14 +217,18 @@ class UVWGenerator:
         return [p for p in self.paths if p.a.idx == a]
 
     def oeq_index(self, p: WPath, u: str, w: str) -> str:
-        """Position of W_t[u, w] in the external (oeq) weight vector: 32 x 32 blocks enumerated
-        (u-block, w-block), each stored [u_local][w_local] (weight_order.py)."""
-        mu, mw = p.mu, p.mw
+        """Position of W_t[u, v, w] (v = the path's copy of the second operand) in the external (oeq)
+        weight vector: chunks of 32 enumerated (u-chunk, v-chunk, w-chunk), each stored
+        [v_local][u_local][w_local] (weight_order.py)."""
+        mu, mv, mw = p.mu, p.mv, p.mw
+        vc, vl = divmod(p.v, 32)
+        vlw = min(32, mv - 32 * vc)
         if mu <= 32 and mw <= 32:
-            return f"{p.woff} + ({u}) * {mw} + ({w})"
+            return f"{p.woff + 32 * vc * mu * mw + vl * mu * mw} + ({u}) * {mw} + ({w})"
         ul = "32" if mu % 32 == 0 else f"min(32, {mu} - (({u}) >> 5) * 32)"
         wl = "32" if mw % 32 == 0 else f"min(32, {mw} - (({w}) >> 5) * 32)"
-        return f"{p.woff} + (({u}) >> 5) * {32 * mw} + {ul} * ((({w}) >> 5) * 32) + (({u}) & 31) * {wl} + (({w}) & 31)"
+        return (f"{p.woff} + (({u}) >> 5) * {32 * mv * mw} + {ul} * ({32 * vc * mw} + {vlw} * ((({w}) >> 5) * 32) + {vl} * {wl})"
+                f" + (({u}) & 31) * {wl} + (({w}) & 31)")
 
     def emit_cg_forward(self, E: Emitter, p: WPath, x: str, y: str, out: str) -> None:
         """out{k} = sum_ij c_ijk {x}{i} * {y}{off+j}  (declares out0..)."""
@@ -785,7 +796,7 @@ class UVWGenerator:
                     for nt in range(p.NTW):
                         for r in range(4):
                             E(f"    {{ const int u = 16 * (wave + {4 * q}) + {self.row(r)}; const int w = {16 * nt} + c;")
-                            E(f"      if (u < {p.mu} && w < {p.mw}) part[{p.woff} + u * {p.mw} + w] = acc{p.t}_{q}_{nt}[{r}]; }}")
+                            E(f"      if (u < {p.mu} && w < {p.mw}) part[{p.poff} + u * {p.mw} + w] = acc{p.t}_{q}_{nt}[{r}]; }}")
                     E("}")
             E.level -= 1
             E("}")
@@ -800,7 +811,7 @@ class UVWGenerator:
         E(f"for (int b = 0; b < {self.DW_WORKGROUPS}; ++b) acc += part[(u64)b * {self.WN} + q];")
         E("int dst = q;")
         for p in self.paths:
-            E(f"if (q >= {p.woff} && q < {p.woff + p.mu * p.mw}) {{ const int e = q - {p.woff}; const int u = e / {p.mw}; const int w = e - u * {p.mw}; dst = {self.oeq_index(p, 'u', 'w')}; }}")
+            E(f"if (q >= {p.poff} && q < {p.poff + p.mu * p.mw}) {{ const int e = q - {p.poff}; const int u = e / {p.mw}; const int w = e - u * {p.mw}; dst = {self.oeq_index(p, 'u', 'w')}; }}")
         E("Wg[dst] = acc;")
         return E.text()
 

@@ -178,6 +178,53 @@ def test_uvw_matrix_core_kernels(dtype, monkeypatch):
     assert rel_err(ow.oeq_to_e3nn(oprob, out["Wg"]), dW) < tol
 
 
+@pytest.mark.parametrize("shared", [False, True])
+def test_uvu_run_time_loop_over_second_operand_copies(shared, monkeypatch):
+    """mul(in2) = 11 > 8: v is walked at run time; dY sums through the LDS accumulator, shared dW through
+    the workgroup's partial row."""
+    from openequivariance_amd.tensor_product import select_generator
+    import openequivariance_amd as oeq
+    ins = [(0, 0, 0, "uvu", True), (0, 1, 1, "uvu", True), (1, 0, 2, "uvu", True), (1, 1, 0, "uvu", True)]
+    a = ("12x0e+12x1o", "11x0e+3x1o", "12x0e+12x1o+12x1o")
+    prob = oeq.TPProblem(*a, ins, shared_weights=shared, internal_weights=False)
+    oprob = spec.Problem(*a, ins, shared_weights=shared)
+    g = select_generator(prob)
+    assert [p.looped for p in g.paths] == [True, False, True, False]
+    X, Y, We, G = common.tp_inputs(prob, 9, 1, w_scale=0.3)
+    W = ow.e3nn_to_oeq(oprob, We)
+    fwd, bwd, ws = g.plan()
+    if shared:
+        g.dw_partials = 3
+        for s in bwd:
+            if s["kernel"] == "backward":
+                s["num_blocks"] = 3
+    out = emu.run_tp(g, fwd, X, Y, W, ws_bytes=ws())
+    assert rel_err(out["Z"], otp.forward(oprob, X, Y, We)) < TOL
+    out = emu.run_tp(g, bwd, X, Y, W, G, ws_bytes=ws())
+    dX, dY, dW = otp.backward(oprob, X, Y, We, G)
+    assert rel_err(out["Xg"], dX) < TOL and rel_err(out["Yg"], dY) < TOL
+    assert rel_err(ow.oeq_to_e3nn(oprob, out["Wg"]), dW) < TOL
+
+
+@pytest.mark.parametrize("shared", [True, False])
+def test_uvw_several_copies_of_the_second_operand(shared, monkeypatch):
+    monkeypatch.setattr(UVWGenerator, "DW_WORKGROUPS", 3)
+    from openequivariance_amd.tensor_product import select_generator
+    a = ("5x0e+21x1o", "3x0e+2x1o", "18x0e+7x1o")
+    prob, oprob = common.fully_connected(a, shared=shared)
+    g = select_generator(prob)
+    assert len(g.paths) == 10 and {p.mv for p in g.paths} == {2, 3}
+    X, Y, We, G = common.tp_inputs(prob, 21 if shared else 5, 9, w_scale=0.3)
+    W = ow.e3nn_to_oeq(oprob, We)
+    fwd, bwd, ws = g.plan()
+    out = emu.run_tp(g, fwd, X, Y, W, ws_bytes=ws())
+    assert rel_err(out["Z"], otp.forward(oprob, X, Y, We)) < TOL
+    out = emu.run_tp(g, bwd, X, Y, W, G, ws_bytes=ws())
+    dX, dY, dW = otp.backward(oprob, X, Y, We, G)
+    assert rel_err(out["Xg"], dX) < TOL and rel_err(out["Yg"], dY) < TOL
+    assert rel_err(ow.oeq_to_e3nn(oprob, out["Wg"]), dW) < TOL
+
+
 def test_uvw_per_row_weights():
     from openequivariance_amd.codegen.uvw_batched import UVWBatchedGenerator
     a = ("5x0e+21x1o", "1x0e+1x1o+1x2e", "18x0e+7x1o+3x2e")

@@ -112,9 +112,7 @@ def test_tensor_product_rejects_host_tensors_among_gpu_tensors(cuda):
 
 def test_unsupported_problems_raise():
     import openequivariance_amd as oeq
-    with pytest.raises(NotImplementedError):      # uvw needs multiplicity 1 on the second operand
-        oeq.TensorProduct(oeq.FullyConnectedTPProblem("4x0e", "2x0e", "4x0e", shared_weights=True, internal_weights=False))
-    with pytest.raises(AssertionError):           # the convolution too
+    with pytest.raises(AssertionError):           # the convolution needs multiplicity 1 on the second operand
         oeq.TensorProductConv(oeq.TPProblem("2x0e", "2x0e", "2x0e", [(0, 0, 0, "uvu", True)], shared_weights=False,
                                             internal_weights=False))
     with pytest.raises(NotImplementedError):

@@ -94,3 +94,51 @@ def test_random_tensor_product(cuda, seed):
     assert rel_err(z.detach().cpu().numpy(), otp.forward(oprob, X, Y, We)) <= tol
     for got, ref in zip((x.grad.cpu().numpy(), y.grad.cpu().numpy(), dW), otp.backward(oprob, X, Y, We, G)):
         assert rel_err(got, ref) <= tol
+
+
+@pytest.mark.parametrize("seed", range(5000, 5016))
+def test_random_second_operand_multiplicities(cuda, seed):
+    """Random multiplicities on the second operand as well (1 to 40 copies per irrep, unrolled and walked
+    at run time), uvu and uvw, shared and per-row weights, through the chunk-of-32 external weight order."""
+    import torch
+    import openequivariance_amd as oeq
+    rng = np.random.default_rng(seed)
+    mode = rng.choice(["uvu", "uvw"])
+    shared = bool(rng.random() < 0.5)
+    dtype = np.float64 if rng.random() < 0.25 else np.float32
+    tol = FP32_TOL if dtype == np.float32 else FP64_TOL
+    n = int(rng.choice([1, 7, 40, 200]))
+    l1 = sorted(rng.choice(3, size=rng.integers(1, 3), replace=False))
+    l2 = sorted(rng.choice(3, size=rng.integers(1, 3), replace=False))
+    mul1 = int(rng.choice([3, 16, 33, 70]))
+    in1 = "+".join(f"{mul1}x{l}{_par(l)}" for l in l1)
+    # (uvw unrolls one contraction per copy: fewer copies there keep the kernels small)
+    copies = [1, 2, 5, 9, 12, 40] if mode == "uvu" else [1, 2, 3, 5, 9]
+    in2 = "+".join(f"{int(rng.choice(copies))}x{l}{_par(l)}" for l in l2)
+    lo = range(int(rng.integers(1, 4)))
+    if mode == "uvu":
+        out = "+".join(f"{mul1}x{l}{_par(l)}" for l in lo)
+        ins = [(i, j, k, "uvu", True) for i, a in enumerate(l1) for j, b in enumerate(l2) for k, c in enumerate(lo)
+               if abs(a - b) <= c <= a + b and (a + b + c) % 2 == 0]
+        if not ins:
+            ins, out = [(0, 0, 0, "uvu", True)], f"{mul1}x{abs(l1[0] - l2[0])}{_par(abs(l1[0] - l2[0]))}"
+        prob = oeq.TPProblem(in1, in2, out, ins, shared_weights=shared, internal_weights=False,
+                             irrep_dtype=dtype, weight_dtype=dtype)
+        from oracle import spec
+        oprob = spec.Problem(in1, in2, out, ins, shared_weights=shared)
+    else:
+        out = "+".join(f"{int(rng.choice([4, 20, 48]))}x{l}{_par(l)}" for l in range(3))
+        prob, oprob = common.fully_connected((in1, in2, out), shared=shared, dtype=dtype)
+    print(f"seed={seed} {mode} shared={shared} {dtype.__name__} {in1} (x) {in2} -> {out} paths={len(prob.instructions)} n={n}",
+          flush=True)
+    tp = oeq.TensorProduct(prob, torch_op=True)
+    X, Y, We, G = common.tp_inputs(prob, n, seed, dtype, w_scale=0.2)
+    W = ow.e3nn_to_oeq(oprob, We)
+    x, y, w = (torch.tensor(a, device=cuda, requires_grad=True) for a in (X, Y, W))
+    z = tp(x, y, w)
+    z.backward(torch.tensor(G, device=cuda))
+    torch.cuda.synchronize()
+    assert rel_err(z.detach().cpu().numpy(), otp.forward(oprob, X, Y, We)) <= tol
+    dW = ow.oeq_to_e3nn(oprob, w.grad.cpu().numpy())
+    for got, ref in zip((x.grad.cpu().numpy(), y.grad.cpu().numpy(), dW), otp.backward(oprob, X, Y, We, G)):
+        assert rel_err(got, ref) <= tol

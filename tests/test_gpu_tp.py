@@ -106,6 +106,51 @@ def test_mul2_greater_than_one(cuda):
     assert rel_err(ow.oeq_to_e3nn(oprob, w.grad.cpu().numpy()), dWr) <= FP32_TOL
 
 
+UVU_LOOPED = {
+    # more than 8 copies of a second-operand irrep: the kernels walk v with a run-time loop
+    "11_copies_two_rows_per_wave": ("12x0e+12x1o", "11x0e+3x1o", "12x0e+12x1o+12x1o"),
+    "ragged_v_3x0e+35x1o": ("40x0e+40x1o", "3x0e+35x1o", "40x0e+40x1o+40x1o"),
+    "two_chunks_35_copies": ("70x0e+70x1o", "35x0e+2x1o", "70x0e+70x1o+70x1o"),
+}
+
+
+@pytest.mark.parametrize("name", sorted(UVU_LOOPED))
+@pytest.mark.parametrize("shared", [False, True])
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_uvu_many_copies_of_the_second_operand(cuda, name, shared, dtype):
+    """uvu with mul(in2) > 8 (reference: ComputationSchedule.py:146-230 chunks v as well as u,
+    loop_unroll_tp.cuh:48-60 and :140-175 loop over it), per-row and shared weights, through the
+    chunk-of-32 [v][u] external weight order."""
+    import openequivariance_amd as oeq
+    from oracle import spec, weights as ow
+    import torch
+    tol = FP32_TOL if dtype == np.float32 else 1e-12
+    ins = [(0, 0, 0, "uvu", True), (0, 1, 1, "uvu", True), (1, 0, 2, "uvu", True), (1, 1, 0, "uvu", True)]
+    a = UVU_LOOPED[name]
+    prob = oeq.TPProblem(*a, ins, shared_weights=shared, internal_weights=False, irrep_dtype=dtype, weight_dtype=dtype)
+    oprob = spec.Problem(*a, ins, shared_weights=shared)
+    n = 2100 if shared else 61                       # shared: more rows than persistent workgroups
+    X, Y, W, G = common.tp_inputs(prob, n, 17, dtype, w_scale=0.2)
+    tp = oeq.TensorProduct(prob, torch_op=True)
+    assert any(p.looped for p in tp.generator.paths)
+    W_oeq = np.zeros_like(W)
+    tp.reorder_weights_e3nn_to_oeq(W, W_oeq, not shared)
+    assert np.array_equal(W_oeq, ow.e3nn_to_oeq(oprob, W))
+    x, y, w = (torch.tensor(t, device=cuda, requires_grad=True) for t in (X, Y, W_oeq))
+    z = tp(x, y, w)
+    z.backward(torch.tensor(G, device=cuda))
+    torch.cuda.synchronize()
+    dXr, dYr, dWr = otp.backward(oprob, X, Y, W, G)
+    assert rel_err(z.detach().cpu().numpy(), otp.forward(oprob, X, Y, W)) <= tol
+    assert rel_err(x.grad.cpu().numpy(), dXr) <= tol
+    assert rel_err(y.grad.cpu().numpy(), dYr) <= tol
+    assert rel_err(ow.oeq_to_e3nn(oprob, w.grad.cpu().numpy()), dWr) <= tol
+    if shared:
+        w2 = w.detach().clone().requires_grad_(True)
+        tp(x.detach(), y.detach(), w2).backward(torch.tensor(G, device=cuda))
+        assert torch.equal(w.grad, w2.grad), "shared-weight dW must be bit-reproducible"
+
+
 def test_shared_weights_uvu(cuda):
     """shared_weights=True: dW is the sum over the batch (deterministic two-stage reduction)."""
     import openequivariance_amd as oeq

@@ -127,12 +127,41 @@ def test_uvw_tensors_beyond_two_giga_elements(cuda):
         assert v <= FP32_TOL, f"{k}: relative error {v:.3e}"
 
 
-def test_uvw_unsupported_cases_raise(cuda):
+UVW_MUL2 = {
+    "small": ("5x0e+21x1o", "3x0e+2x1o", "18x0e+7x1o"),
+    "ragged_v_3x0e+35x1o": ("20x0e+33x1o", "3x0e+35x1o", "17x0e+40x1o"),        # v beyond one 32-chunk
+    "wide": ("70x0e", "4x0e+2x1o", "66x0e+33x1o"),
+}
+
+
+@pytest.mark.parametrize("name", sorted(UVW_MUL2))
+@pytest.mark.parametrize("shared", [True, False])
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_uvw_several_copies_of_the_second_operand(cuda, name, shared, dtype):
+    """uvw with mul(in2) > 1, shared and per-row weights, through reorder_weights_e3nn_to_oeq: the external
+    order stores each 32-chunk block [v][u][w] (reference: ComputationSchedule.py:146-230, :427-471;
+    loop_unroll_tp.cuh:48-60 walks v)."""
+    import torch
     import openequivariance_amd as oeq
-    for shared in (True, False):
-        prob, _ = common.fully_connected(("4x0e", "2x0e", "4x0e"), shared=shared)
-        with pytest.raises(NotImplementedError):
-            oeq.TensorProduct(prob, torch_op=True)
+    if name.startswith("ragged") and dtype == np.float64 and not shared:
+        pytest.skip("same code path as fp32, 38 per-row weight matrices of 8-byte words")
+    tol = FP32_TOL if dtype == np.float32 else FP64_TOL
+    prob, oprob = common.fully_connected(UVW_MUL2[name], shared=shared, dtype=dtype)
+    n = 37
+    X, Y, We, G = common.tp_inputs(prob, n, 47, dtype, w_scale=0.1)
+    tp = oeq.TensorProduct(prob, torch_op=True)
+    W = np.zeros_like(We)
+    tp.reorder_weights_e3nn_to_oeq(We, W, not shared)
+    assert np.array_equal(W, ow.e3nn_to_oeq(oprob, We))
+    x, y, w = (torch.tensor(a, device=cuda, requires_grad=True) for a in (X, Y, W))
+    z = tp(x, y, w)
+    z.backward(torch.tensor(G, device=cuda))
+    torch.cuda.synchronize()
+    dXr, dYr, dWr = otp.backward(oprob, X, Y, We, G)
+    assert rel_err(z.detach().cpu().numpy(), otp.forward(oprob, X, Y, We)) <= tol
+    assert rel_err(x.grad.cpu().numpy(), dXr) <= tol
+    assert rel_err(y.grad.cpu().numpy(), dYr) <= tol
+    assert rel_err(ow.oeq_to_e3nn(oprob, w.grad.cpu().numpy()), dWr) <= tol
 
 
 DIFFDOCK = {"DiffDock-L=1": ("10x1o+10x1e+48x0e+48x0o", "1x0e+1x1o", "10x1o+10x1e+48x0e+48x0o"),
