@@ -151,8 +151,23 @@ class TensorProductConv:
         # the deterministic backward walks the caller's transpose permutation
         self.backward_needs_tperm = deterministic
         self.jit_kernel = self.generator.render()
+        self._ws_fns = []
         self.internal = self._build(self.generator, self.jit_kernel)
         self._workspaces: typing.Dict[int, _StreamWorkspace] = {}
+        # Unsorted edge lists: whether the backward scatters dX with float atomics or groups the edges by
+        # sender first depends on the row length AND on the graph (atomics per edge against the gathers of
+        # the segmented kernel); the generator's rule of thumb is only the starting point.  The torch
+        # operator times both on the first backward call of each size class and keeps the faster one
+        # (OEQ_AMD_CONV_BACKWARD=atomic|grouped or OEQ_AMD_AUTOTUNE=0 switch the measurement off).  The
+        # deterministic operator never chooses by timing: which kernel runs must not depend on a stopwatch
+        # if results are to repeat bit for bit from one process to the next.
+        self._bwd_variants = {}
+        self._bwd_choice: typing.Dict[tuple, str] = {}
+        if isinstance(self.generator, UVUSortedGenerator):
+            self._bwd_default = "grouped" if self.generator.grouped_backward else "atomic"
+            self._bwd_variants[self._bwd_default] = (self.internal, self.backward_overwrites)
+        self.autotune = (bool(self._bwd_variants) and os.environ.get("OEQ_AMD_AUTOTUNE", "1") != "0"
+                         and os.environ.get("OEQ_AMD_CONV_BACKWARD") not in ("atomic", "grouped"))
         self.graph_cache = os.environ.get("OEQ_AMD_GRAPH_CACHE", "1") != "0"
         self._internal_unaligned = None
         self._reorder = WeightReorder(config)
@@ -162,11 +177,28 @@ class TensorProductConv:
             self._setup_torch_module()
 
     def _build(self, generator, source=None) -> "rt.ConvImpl":
-        fwd, bwd, self._ws_bytes = generator.plan()
-        need_ws = rt.STEP_NEEDS_WORKSPACE if self._ws_bytes(1, 1) > 0 else 0
+        """Compile one kernel set of this operator.  Every set shares the operator's workspace, which is
+        sized for the largest of them."""
+        fwd, bwd, ws = generator.plan()
+        self._ws_fns.append(ws)
+        need_ws = rt.STEP_NEEDS_WORKSPACE if ws(1, 1) > 0 else 0
         need_tp = rt.STEP_NEEDS_TPERM if self.backward_needs_tperm else 0
         code = rt.compile_source(source if source is not None else generator.render())
         return rt.ConvImpl(code, _make_steps(fwd, need_ws), _make_steps(bwd, need_ws | need_tp))
+
+    def _ws_bytes(self, nnz: int, node_count: int) -> int:
+        return max(f(nnz, node_count) for f in self._ws_fns)
+
+    def _backward_variant(self, name: str):
+        """(kernel set, whether its backward overwrites dX) of a backward variant of the unsorted operator,
+        compiled on first need."""
+        if name not in self._bwd_variants:
+            g = UVUSortedGenerator(self.config, grouped_backward=(name == "grouped"),
+                                   idx_ctype="i64" if self.idx_dtype == np.int64 else "int")
+            self._bwd_variants[name] = (self._build(g), name == "grouped")
+            for rec in self._workspaces.values():            # the workspace may have to grow: sizes are re-checked per call
+                rec.bwd_key = None
+        return self._bwd_variants[name]
 
     @staticmethod
     def name():
@@ -243,9 +275,7 @@ class TensorProductConv:
         if any(int(p) % 16 for p in ptrs):
             if self._internal_unaligned is None:
                 g = select_conv_generator(self.config, self.deterministic, vector_stores=False, idx_dtype=self.idx_dtype)
-                ws_bytes = self._ws_bytes
                 self._internal_unaligned = self._build(g)
-                self._ws_bytes = ws_bytes
             return self._internal_unaligned
         return self.internal
 
@@ -268,15 +298,17 @@ class TensorProductConv:
                                workspace, transpose_perm, self._stream() if stream is None else stream, prepared)
 
     def backward_rawptrs(self, L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_grad, rows, cols, nnz,
-                         node_count, workspace=0, transpose_perm=0, stream=None, prepared=False):
+                         node_count, workspace=0, transpose_perm=0, stream=None, prepared=False, impl=None):
         """reference: extension/convolution.hpp:149-173; ``workspace`` and ``prepared`` as in
-        exec_conv_rawptrs (the backward keeps its own preparation in the workspace)."""
+        exec_conv_rawptrs (the backward keeps its own preparation in the workspace).  ``impl`` selects
+        another kernel set of this operator (see _backward_variant) instead of the default one."""
         nnz, node_count = int(nnz), int(node_count)
         if nnz > 0 and not (rows and cols):
             raise ValueError("rows / cols must be device pointers")
         if self.backward_needs_tperm and nnz > 0 and not transpose_perm:
             raise ValueError("the deterministic backward needs transpose_perm (a device pointer), got 0")
-        impl = self._pick(L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_grad)
+        if impl is None:
+            impl = self._pick(L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_grad)
         if not workspace:
             rec = self._workspace_record(nnz, node_count, stream)
             rec.bwd_key = None
@@ -285,7 +317,25 @@ class TensorProductConv:
                               nnz, node_count, workspace, transpose_perm,
                               self._stream() if stream is None else stream, prepared)
 
-    def _cached_call(self, which: str, rows, cols, tperm, E: int, N: int, launch) -> None:
+    def _time_backward_variants(self, run, names=("atomic", "grouped"), repeats: int = 3) -> str:
+        """Fastest of the backward variants on the caller's own tensors: one untimed call each (compilation,
+        graph preparation), then the best of ``repeats`` timed calls between HIP events."""
+        best = {}
+        for name in names:
+            run(name)
+            times = []
+            for _ in range(repeats):
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                run(name)
+                b.record()
+                b.synchronize()
+                times.append(a.elapsed_time(b))
+            best[name] = min(times)
+        self.last_tuning = best
+        return min(best, key=best.get)
+
+    def _cached_call(self, which: str, rows, cols, tperm, E: int, N: int, launch, tag: str = "") -> None:
         """Run ``launch(workspace pointer, prepared)`` for the torch operators.  The graph preparation a
         call leaves in the stream's workspace is reused by the next call of the same direction when it
         names the same graph: same index tensors (address and in-place version counter), same sizes.  The
@@ -300,7 +350,7 @@ class TensorProductConv:
             rec.captured = True
         key = None
         if self.graph_cache and not rec.captured:
-            key = (E, N) + tuple((t.data_ptr(), t._version) for t in (rows, cols, tperm) if t is not None)
+            key = (tag, E, N) + tuple((t.data_ptr(), t._version) for t in (rows, cols, tperm) if t is not None)
         attr = which + "_key"
         prepared = key is not None and getattr(rec, attr) == key
         setattr(rec, attr, None)
@@ -329,20 +379,35 @@ class TensorProductConv:
                     ws, tperm.data_ptr() if tperm is not None else 0, prepared=prepared))
             return out
 
+        def bwd_run(x, y, w, g, rows, cols, tperm, E, N, variant=None):
+            """One backward pass into fresh outputs with the default kernel set or a named variant."""
+            impl, overwrites = (None, self.backward_overwrites) if variant is None else self._backward_variant(variant)
+            if variant is not None and any(int(t.data_ptr()) % 16 for t in (x, y, w, g)):
+                impl, overwrites, variant = None, self.backward_overwrites, None     # misaligned views: the default set only
+            xg = (torch.empty_like if overwrites else torch.zeros_like)(x)
+            yg, wg = torch.empty_like(y), torch.empty_like(w)
+            self._cached_call("bwd", rows, cols, tperm, E, N, lambda ws, prepared: self.backward_rawptrs(
+                x.data_ptr(), xg.data_ptr(), y.data_ptr(), yg.data_ptr(), w.data_ptr(), wg.data_ptr(), g.data_ptr(),
+                rows.data_ptr(), cols.data_ptr(), E, N, ws, tperm.data_ptr() if tperm is not None else 0,
+                prepared=prepared, impl=impl), tag=variant or "")
+            return [xg, yg, wg]
+
         def bwd_impl(L1_in, L2_in, weights, L3_grad, rows, cols, tperm):
             x, y, w, g = L1_in.contiguous(), L2_in.contiguous(), weights.contiguous(), L3_grad.contiguous()
             rows, cols = rows.contiguous(), cols.contiguous()
             tperm = tperm.contiguous() if tperm is not None else None
             self._check(x, y, w, rows, cols, tperm, g)
             E, N = rows.shape[0], x.shape[0]
-            xg = (torch.empty_like if self.backward_overwrites else torch.zeros_like)(x)
-            yg, wg = torch.empty_like(y), torch.empty_like(w)
             with torch.cuda.device(x.device):
-                self._cached_call("bwd", rows, cols, tperm, E, N, lambda ws, prepared: self.backward_rawptrs(
-                    x.data_ptr(), xg.data_ptr(), y.data_ptr(), yg.data_ptr(), w.data_ptr(), wg.data_ptr(), g.data_ptr(),
-                    rows.data_ptr(), cols.data_ptr(), E, N, ws, tperm.data_ptr() if tperm is not None else 0,
-                    prepared=prepared))
-            return [xg, yg, wg]
+                if not self.autotune or E == 0:
+                    return bwd_run(x, y, w, g, rows, cols, tperm, E, N)
+                size_class = (E.bit_length(), N.bit_length())
+                if size_class not in self._bwd_choice:
+                    if torch.cuda.is_current_stream_capturing():       # no clocks inside a capture: rule of thumb
+                        return bwd_run(x, y, w, g, rows, cols, tperm, E, N)
+                    self._bwd_choice[size_class] = self._time_backward_variants(
+                        lambda name: bwd_run(x, y, w, g, rows, cols, tperm, E, N, name))
+                return bwd_run(x, y, w, g, rows, cols, tperm, E, N, self._bwd_choice[size_class])
 
         # the two variants differ only in the trailing transpose_perm argument, which torch's operator
         # schemas need spelled out

@@ -151,3 +151,28 @@ def test_raw_entry_points_with_prepared_workspace(cuda, deterministic):
     if deterministic:
         for a, b in zip(outs[0], outs[2]):
             assert torch.equal(a, b)
+
+
+def test_unsorted_backward_variant_is_chosen_by_measurement(cuda, monkeypatch):
+    """The first backward call of a size class times the atomic and the grouped backward on the caller's
+    tensors and keeps the faster; both give the oracle's gradients; overrides switch the timing off."""
+    import openequivariance_amd as oeq
+    monkeypatch.delenv("OEQ_AMD_CONV_BACKWARD", raising=False)
+    monkeypatch.delenv("OEQ_AMD_AUTOTUNE", raising=False)
+    prob, oprob = common.channelwise(common.NEQUIP)
+    conv = oeq.TensorProductConv(prob, torch_op=True, deterministic=False)
+    assert conv.autotune and conv._bwd_default == "atomic"
+    host, graph, t, index, g = _inputs(prob, 70, 1500, 13, False, cuda)
+    _check(oprob, host, graph, conv, t, index, g)
+    assert set(conv.last_tuning) == {"atomic", "grouped"} and len(conv._bwd_choice) == 1
+    chosen = next(iter(conv._bwd_choice.values()))
+    assert chosen == min(conv.last_tuning, key=conv.last_tuning.get)
+    conv.last_tuning = None
+    _check(oprob, host, graph, conv, t, index, g)            # same size class: no second measurement
+    assert conv.last_tuning is None
+    for name in ("atomic", "grouped"):                       # either variant, forced, against the oracle
+        conv._bwd_choice = {k: name for k in conv._bwd_choice}
+        _check(oprob, host, graph, conv, t, index, g)
+    monkeypatch.setenv("OEQ_AMD_AUTOTUNE", "0")
+    assert not oeq.TensorProductConv(prob, torch_op=True, deterministic=False).autotune
+    assert not oeq.TensorProductConv(prob, torch_op=True, deterministic=True).autotune
