@@ -39,7 +39,10 @@ class UVUDirectGenerator(UVUGenerator):
         # False: outputs are written with dword-aligned record stores only (for callers whose
         # output tensor is not 16-byte aligned)
         self.vector_stores = vector_stores
-        self.VW = 16 // self.itemsize
+        # words per vector store of the LDS-slot route (16 bytes; OEQ_AMD_TP_STORE_BYTES=8 for A/B runs)
+        self.store_bytes = int(os.environ.get("OEQ_AMD_TP_STORE_BYTES", "16")) if kind == "tp" else 16
+        self.VW = max(1, self.store_bytes // self.itemsize)
+        self.VTYPE = "VT" if self.VW * self.itemsize == 16 else "VT8"
         stage = [WAVE * b.D for b in list(self.out) + list(self.in1) if b.D > 1 and b.dim]
         self.lds_elems = max(stage) if stage else 0
         self.ZB = 0
@@ -114,9 +117,9 @@ class UVUDirectGenerator(UVUGenerator):
                 guard = f"q < {total} && ok"
                 tgt = f"{ptr} + grow * {rowdim} + {blk.off} + (q - r * {per_row}) * {unit}"
             if op == "store" and self.nt_store:
-                E(f"  if ({guard}) __builtin_nontemporal_store(*(const VT*)(lds + {base} + q * {unit}), (VT*)({tgt})); }}")
+                E(f"  if ({guard}) __builtin_nontemporal_store(*(const {self.VTYPE}*)(lds + {base} + q * {unit}), ({self.VTYPE}*)({tgt})); }}")
             elif op == "store":
-                E(f"  if ({guard}) *(VT*)({tgt}) = *(const VT*)(lds + {base} + q * {unit}); }}")
+                E(f"  if ({guard}) *({self.VTYPE}*)({tgt}) = *(const {self.VTYPE}*)(lds + {base} + q * {unit}); }}")
             else:
                 E(f"  if ({guard}) oeq_atomic_add({tgt}, lds[{base} + q]); }}")
 

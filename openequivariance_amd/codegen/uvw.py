@@ -92,6 +92,7 @@ class WPath:
 
 class UVWGenerator:
     DW_WORKGROUPS = 256          # persistent dW workgroups: one per compute unit of an MI355X
+    FWD_ACC_LIMIT = 80           # accumulator registers of one forward work item
 
     def __init__(self, problem: TPProblem):
         self.problem = problem
@@ -143,7 +144,22 @@ class UVWGenerator:
         self.used_out = sorted({p.o.idx for p in self.paths})
         self.used_y = sorted({p.b.off + j for p in self.paths for (_, j) in p.pairs})
         cost = lambda o: sum(p.o.D * p.NTW * p.SU for p in self.paths if p.o.idx == o.idx)
-        self.fwd_order = sorted([o for o in self.out if o.dim > 0], key=lambda o: -cost(o))
+        # forward work items: (output block, range of its 16-wide w tiles), most expensive first.  A block
+        # whose accumulator tile (D * tiles * 4 registers) exceeds FWD_ACC_LIMIT is cut into w ranges, each
+        # a work item of its own: fewer accumulators per wavefront buy a third wavefront per SIMD, which
+        # hides one wavefront's vector-ALU phases behind another's matrix-core phases
+        limit = int(os.environ.get("OEQ_AMD_UVW_FWD_ACC", str(self.FWD_ACC_LIMIT)))
+        self.fwd_order = []
+        for o in sorted([o for o in self.out if o.dim > 0], key=lambda o: -cost(o)):
+            nt_all = _ceil(o.mul, 16)
+            parts = 1
+            if o.idx in self.used_out:
+                while 4 * o.D * _ceil(nt_all, parts) > limit and parts < nt_all:
+                    parts += 1
+            step = _ceil(nt_all, parts)
+            for lo in range(0, nt_all, step):
+                self.fwd_order.append((o, lo, min(nt_all, lo + step)))
+        self.fwd_order.sort(key=lambda it: -cost(it[0]) * (it[2] - it[1]) / _ceil(it[0].mul, 16))
         # dW kernel: output blocks split into two groups of similar MFMA work
         # (f64 accumulators are twice as wide: one group, four wavefronts, the whole register file)
         work = {o: sum(p.o.D * p.NTW * p.NTU for p in self.paths if p.o.idx == o) for o in self.used_out}
@@ -341,9 +357,10 @@ class UVWGenerator:
         # One work item = (batch tile, output block): blockIdx.y walks the output blocks from the most
         # to the least expensive, so the dispatcher fills the tail of the launch with the cheap ones
         # (whole tiles per wavefront leave a third of the machine idle in the last round).
-        for slot, o in enumerate(self.fwd_order):
+        for slot, (o, nt_lo, nt_hi) in enumerate(self.fwd_order):
             NT = _ceil(o.mul, 16)
-            E(f"if (slot == {slot}) {{ // output block {o.idx}: {o.mul}x l={o.l}")
+            NTS = range(nt_lo, nt_hi)
+            E(f"if (slot == {slot}) {{ // output block {o.idx}: {o.mul}x l={o.l}, w tiles {nt_lo} .. {nt_hi - 1} of {NT}")
             E.level += 1
             if o.idx not in self.used_out:
                 for r in range(4):
@@ -352,7 +369,7 @@ class UVWGenerator:
                 E("}")
                 continue
             for k in range(o.D):
-                for nt in range(NT):
+                for nt in NTS:
                     E(f"V4 acc{k}_{nt} = {{0, 0, 0, 0}};")
             for p in self.paths_into(o.idx):
                 E(f"{{ // path {p.t}: l = {p.a.l} x {p.b.l} -> {p.o.l}, coefficient {p.coeff:.9g}")
@@ -364,12 +381,15 @@ class UVWGenerator:
                 # more than anything else here.
                 GS = self.fwd_group
                 NG = _ceil(p.SU, GS)
-                regs = [f"nx{j}_{i}" for j in range(GS) for i in range(p.a.D)] + [f"nb{j}_{nt}" for j in range(GS) for nt in range(NT)]
+                pingpong = (self.fwd_unroll == 0)
+                sets = ("a", "b") if pingpong else ("n",)
+                regs = [f"{q}x{j}_{i}" for q in sets for j in range(GS) for i in range(p.a.D)] \
+                    + [f"{q}b{j}_{nt}" for q in sets for j in range(GS) for nt in NTS]
                 E("T " + ", ".join(regs) + ";")
                 if self.fwd_row_matrix:
                     self.emit_cg_matrix(E, p, "y", "m")
 
-                def load(E, gexp):
+                def load(E, gexp, q="n"):
                     for j in range(GS):
                         sexp = f"({gexp}) * {GS} + {j}"
                         need_clamp = (NG * GS != p.SU)
@@ -378,42 +398,56 @@ class UVWGenerator:
                         # four steps of a group read four adjacent records of a row (one wide load per lane)
                         uexp = f"16 * (({sexp}) >> 2) + 4 * g + (({sexp}) & 3)"
                         ucl = uexp if (p.mu % 16 == 0 and not need_clamp) else f"min({uexp}, {p.mu - 1})"
-                        E(f"{{ const T* __restrict__ xp = Xr + {p.a.off} + ({ucl}) * {p.a.D}; " + " ".join(f"nx{j}_{i} = xp[{i}];" for i in range(p.a.D)))
-                        E(f"  const T* __restrict__ bp = wsT + {p.wb} + (({scl}) * 64 + lane) * {NT}; " + " ".join(f"nb{j}_{nt} = bp[{nt}];" for nt in range(NT)) + " }")
-                load(E, "0")
-                E(f"#pragma unroll {self.fwd_unroll}")
-                E(f"for (int sg = 0; sg < {NG}; ++sg) {{")
-                E.level += 1
-                E("const T " + ", ".join(f"c{r} = {r}" for r in regs) + ";")
-                E(f"if (sg + 1 < {NG}) {{")
-                E.level += 1
-                load(E, "sg + 1")
-                E.level -= 1
-                E("}")
-                for j in range(GS):
-                    E("{")
+                        E(f"{{ const T* __restrict__ xp = Xr + {p.a.off} + ({ucl}) * {p.a.D}; " + " ".join(f"{q}x{j}_{i} = xp[{i}];" for i in range(p.a.D)))
+                        E(f"  const T* __restrict__ bp = wsT + {p.wb} + (({scl}) * 64 + lane) * {NT}; " + " ".join(f"{q}b{j}_{nt} = bp[{nt}];" for nt in NTS) + " }")
+
+                def steps(E, sgexp, q):
+                    """The GS K steps of group ``sgexp`` on the operands of register set q."""
+                    for j in range(GS):
+                        E("{")
+                        E.level += 1
+                        E("const T " + ", ".join(f"x{i} = {q}x{j}_{i}" for i in range(p.a.D)) + ";")
+                        if self.fwd_row_matrix:
+                            self.emit_cg_apply(E, p, "x", "m", "t")
+                        else:
+                            self.emit_cg_forward(E, p, "x", "y", "t")
+                        if p.mu % 16 != 0 or NG * GS != p.SU:
+                            E(f"if (16 * ((({sgexp}) * {GS} + {j}) >> 2) + 4 * g + ((({sgexp}) * {GS} + {j}) & 3) >= {p.mu}) {{ " + " ".join(f"t{k} = (T)0;" for k in range(o.D)) + " }")
+                        for k in range(o.D):
+                            for nt in NTS:
+                                E(f"acc{k}_{nt} = oeq_mfma(t{k}, {q}b{j}_{nt}, acc{k}_{nt});")
+                        E.level -= 1
+                        E("}")
+                if pingpong:
+                    # the groups are written out one after the other on alternating register sets: the operands
+                    # of the next group are requested into the other set, nothing is copied between sets
+                    load(E, "0", "a")
+                    for sg in range(NG):
+                        cur, nxt = ("a", "b") if sg % 2 == 0 else ("b", "a")
+                        if sg + 1 < NG:
+                            load(E, str(sg + 1), nxt)
+                        steps(E, str(sg), cur)
+                else:
+                    load(E, "0")
+                    E(f"#pragma unroll {self.fwd_unroll}")
+                    E(f"for (int sg = 0; sg < {NG}; ++sg) {{")
                     E.level += 1
-                    E("const T " + ", ".join(f"x{i} = cnx{j}_{i}" for i in range(p.a.D)) + ";")
-                    if self.fwd_row_matrix:
-                        self.emit_cg_apply(E, p, "x", "m", "t")
-                    else:
-                        self.emit_cg_forward(E, p, "x", "y", "t")
-                    if p.mu % 16 != 0 or NG * GS != p.SU:
-                        E(f"if (16 * ((sg * {GS} + {j}) >> 2) + 4 * g + ((sg * {GS} + {j}) & 3) >= {p.mu}) {{ " + " ".join(f"t{k} = (T)0;" for k in range(o.D)) + " }")
-                    for k in range(o.D):
-                        for nt in range(NT):
-                            E(f"acc{k}_{nt} = oeq_mfma(t{k}, cnb{j}_{nt}, acc{k}_{nt});")
+                    E("const T " + ", ".join(f"c{r} = {r}" for r in regs) + ";")
+                    E(f"if (sg + 1 < {NG}) {{")
+                    E.level += 1
+                    load(E, "sg + 1")
                     E.level -= 1
                     E("}")
-                E.level -= 1
-                E("}")
+                    steps(E, "sg", "cn")
+                    E.level -= 1
+                    E("}")
                 E.level -= 1
                 E("}")
             # lane holds, for each of its 4 rows, w = NT*c + nt (nt < NT) and all k: a contiguous run
             for r in range(4):
                 E(f"{{ const u64 row = row0 + {self.row(r)};")
                 E(f"  if (row < n) {{ T* __restrict__ zp = Z + row * {self.D3} + {o.off} + {NT} * c * {o.D};")
-                for nt in range(NT):
+                for nt in NTS:
                     guard = "" if o.mul % 16 == 0 else f"if ({NT} * c + {nt} < {o.mul}) "
                     E(f"    {guard}{{ " + " ".join(f"zp[{nt * o.D + k}] = acc{k}_{nt}[{r}];" for k in range(o.D)) + " }")
                 E("  } }")

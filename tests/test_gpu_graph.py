@@ -110,3 +110,43 @@ def test_convolution_in_a_graph(cuda, deterministic):
             if first is None:
                 first = now
             assert all(torch.equal(p, q) for p, q in zip(first, now)), rep
+
+
+@pytest.mark.parametrize("deterministic", [True, False])
+def test_torch_operator_in_a_graph_prepares_the_graph_itself(cuda, deterministic):
+    """The torch operator under capture: the capture always records the graph-preparation kernels (it
+    does not rely on what an earlier eager call left in the workspace), so replays stay correct after
+    eager calls with another graph, and eager calls stay correct after replays."""
+    import torch
+    import openequivariance_amd as oeq
+    prob, oprob = common.channelwise(common.NEQUIP)
+    conv = oeq.TensorProductConv(prob, torch_op=True, deterministic=deterministic)
+
+    def make(nodes, nnz, seed):
+        rows, cols = common.random_graph(nodes, nnz, seed)
+        idx = (rows, cols)
+        if deterministic:
+            rows, cols, tperm, _ = otp.coord_graph(rows, cols)
+            idx = (rows, cols, tperm)
+        X, Y, W, _ = common.conv_inputs(prob, nodes, nnz, seed, np.float32, 2)
+        ref = otp.conv_forward(oprob, X, Y, W, rows, cols)
+        return [torch.tensor(a, device=cuda) for a in (X, Y, W)], [torch.tensor(a, device=cuda) for a in idx], ref
+    (x, y, w), idx, ref = make(120, 3000, 51)
+    (x2, y2, w2), idx2, ref2 = make(120, 3000, 52)          # same sizes, other graph: same workspace
+
+    out = {}
+
+    def step():
+        out["z"] = conv.forward(x, y, w, *idx)
+    graph = _capture(torch, step)
+    for rep in range(3):
+        out["z"].fill_(float("nan"))
+        z_other = conv.forward(x2, y2, w2, *idx2)           # eager call between replays, other graph
+        torch.cuda.synchronize()
+        assert rel_err(z_other.cpu().numpy(), ref2) <= FP32_TOL, rep
+        graph.replay()
+        torch.cuda.synchronize()
+        assert rel_err(out["z"].cpu().numpy(), ref) <= FP32_TOL, rep
+    z_again = conv.forward(x2, y2, w2, *idx2)
+    torch.cuda.synchronize()
+    assert rel_err(z_again.cpu().numpy(), ref2) <= FP32_TOL

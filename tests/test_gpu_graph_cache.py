@@ -49,7 +49,8 @@ def test_preparation_is_reused_and_rebuilt(cuda, deterministic, irreps):
     nodes, nnz = 60, 900
     host, graph, t, index, g = _inputs(prob, nodes, nnz, 5, deterministic, cuda)
     rec = lambda: conv._workspace_record(nnz, nodes)
-    z1 = _check(oprob, host, graph, conv, t, index, g)
+    _check(oprob, host, graph, conv, t, index, g)     # first call: the unsorted operator may compile a second backward
+    z1 = _check(oprob, host, graph, conv, t, index, g)  # variant while timing, and grow its workspace for it
     assert rec().fwd_key is not None and rec().bwd_key is not None
     key = (rec().fwd_key, rec().bwd_key)
     # second call on the same tensors: the preparation kernels are skipped, results unchanged
@@ -62,7 +63,7 @@ def test_preparation_is_reused_and_rebuilt(cuda, deterministic, irreps):
     host2, graph2, _, index2, _ = _inputs(prob, nodes, nnz, 6, deterministic, cuda)
     for dst, src in zip(index, index2):
         dst.copy_(src)
-    assert tuple(i.data_ptr() for i in index) == tuple(k[0] for k in key[0][2:])
+    assert tuple(i.data_ptr() for i in index) == tuple(k[0] for k in key[0][3:])
     _check(oprob, (host[0], host[1], host[2], host[3]), graph2, conv, t, index, g)
     assert rec().fwd_key != key[0]
 

@@ -55,3 +55,36 @@ def test_fake_tensor_shapes_without_running_kernels(cuda):
         assert tuple(z.shape) == (7, 1120) and z.device.type == "cuda"
         gx, gy, gw = tp.backward_helper(x, y, w, z)
         assert gx.shape == x.shape and gy.shape == y.shape and gw.shape == w.shape
+
+
+@pytest.mark.parametrize("deterministic", [False, True])
+def test_compiled_function_matches_eager(cuda, deterministic):
+    """torch.compile traces through the operators with their fake kernels and differentiates through
+    their registered backward (backend aot_eager: tracing, functionalisation and the joint graph, no
+    code generation): same numbers as eager."""
+    import torch
+    import openequivariance_amd as oeq
+    prob, _ = common.channelwise(common.NEQUIP)
+    tp = oeq.TensorProduct(prob, torch_op=True)
+    conv = oeq.TensorProductConv(prob, torch_op=True, deterministic=deterministic)
+    rows, cols = common.random_graph(12, 90, 3)
+    index = [rows, cols]
+    if deterministic:
+        rows, cols, tperm, _ = otp.coord_graph(rows, cols)
+        index = [rows, cols, tperm]
+    index = [torch.tensor(a, device=cuda) for a in index]
+
+    def model(x, y, w, xe):
+        return conv.forward(x, y, w, *index).square().sum() + tp.forward(xe, y, w).sum()
+    x = torch.randn(12, 288, device=cuda, requires_grad=True)
+    xe = torch.randn(90, 288, device=cuda, requires_grad=True)
+    y, w = (torch.randn(90, d, device=cuda, requires_grad=True) for d in (9, 352))
+    eager = model(x, y, w, xe)
+    g_eager = torch.autograd.grad(eager, (x, y, w, xe))
+    compiled = torch.compile(model, backend="aot_eager", fullgraph=True)
+    got = compiled(x, y, w, xe)
+    g_got = torch.autograd.grad(got, (x, y, w, xe))
+    torch.cuda.synchronize()
+    assert torch.allclose(got, eager, rtol=1e-5, atol=1e-5)
+    for a, b in zip(g_got, g_eager):
+        assert torch.allclose(a, b, rtol=1e-4, atol=1e-4)
