@@ -11,10 +11,10 @@ floating-point sums may differ in the last bits between runs, like the atomic ke
 (reference: templates/loop_unroll_conv_atomic.cuh:25-141 scatters with atomicAdd).
 
 The backward scatters only d1 values per edge (dX), dW and dY being per-edge outputs.  While d1 is
-small it keeps the register-direct kernel with coalesced atomics; from ATOMIC_BACKWARD_MAX_D1
-values per edge on, the atomics retire slower than the row gathers of the segmented backward, and
-the backward groups the edges by sender in the same way and runs the deterministic variant's
-backward over that order.
+very small it keeps the register-direct kernel with coalesced atomics; from ATOMIC_BACKWARD_MAX_D1
+values per edge on, the backward groups the edges by sender in the same way and runs the
+deterministic variant's backward over that order (the atomics retire slower than the row gathers of
+the segmented backward, and the grouping is reused from the workspace while the graph stays the same).
 
 Workspace: (node_count + 1) group pointers, (node_count + 1) fill cursors and nnz edge positions,
 all int64, for the forward; behind them the same three arrays of the grouped backward (by sender), its
@@ -35,9 +35,13 @@ class UVUSortedGenerator:
     kind = "conv_atomic"
     SCAN_THREADS = 1024
 
-    # dX values per edge from which the grouped backward is used (measured: 288 per edge - atomic 202 us,
-    # grouped 200 us, a tie; 2304 per edge - atomic 9.1 ms, grouped 7.7 ms)
-    ATOMIC_BACKWARD_MAX_D1 = 1024
+    # dX values per edge from which the grouped backward is the starting choice.  Measured with the grouping
+    # rebuilt on every call: 288 per edge - atomic 202 us, grouped 200 us, a tie; 2304 per edge - atomic
+    # 9.1 ms, grouped 7.7 ms.  With the grouping reused from the workspace (a model calls one graph many
+    # times): 288 per edge - atomic 204 us, grouped 161 us; 1152 per edge - atomic 2.90 ms, grouped 2.22 ms.
+    # Below a couple of cache lines per edge the atomics are few and the starting choice stays atomic; the
+    # torch operator measures both on first use either way.
+    ATOMIC_BACKWARD_MAX_D1 = 128
 
     def __init__(self, problem: TPProblem, vector_stores: bool = True, grouped_backward=None, idx_ctype: str = "i64"):
         self.problem = problem

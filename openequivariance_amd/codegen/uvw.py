@@ -654,6 +654,38 @@ class UVWGenerator:
         return E.text()
 
     # ============================================================ backward: dW
+    # accumulator registers (32-bit) live in one pass of the dW kernel.  fp64: the 352 accumulators of the
+    # 64-channel benchmark problem in one pass leave one wavefront per SIMD and no room for anything else;
+    # two passes of 192 + 160 measured 0.70 -> 0.63 ms for that kernel, three or more passes lose again
+    DW_ACC_BUDGET = {4: 352, 8: 192}
+
+    def dw_passes(self):
+        """(wavefront group, paths) of the passes of the dW kernel.  The accumulators of all paths of a
+        pass are live at once (4 registers per 16 x 16 tile, 8 in fp64); problems with many paths - every
+        copy of a second operand with mul > 1 is a path of its own - are cut into passes of at most
+        DW_ACC_BUDGET accumulator registers, each walking the batch again, so that the register file is
+        never oversubscribed (a kernel spilling hundreds of accumulators is slow, and its fp64 results
+        were not exact on the device)."""
+        per_tile = 4 * (self.itemsize // 4)
+        budget = int(os.environ.get("OEQ_AMD_UVW_DW_ACC", str(self.DW_ACC_BUDGET[self.itemsize])))
+        passes = []
+        for grp in range(self.dw_groups):
+            mine = [p for p in self.paths if self.dw_group[p.o.idx] == grp]
+            need = {p.t: _ceil(p.NTU, 4) * p.NTW * per_tile for p in mine}
+            total = sum(need.values())
+            count = max(1, _ceil(total, budget))
+            target = total / count                   # passes of about equal accumulator count
+            cur, used = [], 0
+            for p in mine:
+                if cur and (used + need[p.t] > budget or used >= target):
+                    passes.append((grp, cur))
+                    cur, used = [], 0
+                cur.append(p)
+                used += need[p.t]
+            if cur:
+                passes.append((grp, cur))
+        return passes
+
     def backward_dw_body(self) -> str:
         E = Emitter()
         # eight wavefronts: wave & 3 selects the 16-channel u-subtile, wave >> 2 one of two groups of
@@ -663,11 +695,12 @@ class UVWGenerator:
         E("const int lane = threadIdx.x & 63, wave = (threadIdx.x >> 6) & 3, grp = threadIdx.x >> 8, c = lane & 15, g = lane >> 4;")
         E("const u64 ntiles = (n + 15) / 16;")
         E(f"T* __restrict__ part = (T*)ws + {self.PART_OFF} + (u64)blockIdx.x * {self.WN};")
-        for grp in range(self.dw_groups):
-            outs = [oi for oi in self.used_out if self.dw_group[oi] == grp]
-            paths = [p for p in self.paths if p.o.idx in outs]
+        for grp, paths in self.dw_passes():
+            # a pass: these paths' accumulators are the only ones live while the batch is walked once
+            outs = sorted({p.o.idx for p in paths})
             ins = sorted({p.a.idx for p in paths})
             ys = sorted({p.b.off + j for p in paths for (_, j) in p.pairs})
+            into = lambda oi, paths=paths: [p for p in paths if p.o.idx == oi]
             E(f"if (grp == {grp}) {{")
             E.level += 1
             for p in paths:
@@ -717,11 +750,11 @@ class UVWGenerator:
                     E.level -= 1
                     E("}")
 
-                def compute(E, outs=outs):
+                def compute(E, outs=outs, into=into):
                     for oi in outs:
                         o = self.out[oi]
                         NT = _ceil(o.mul, 16)
-                        for p in self.paths_into(oi):
+                        for p in into(oi):
                             for q in range(_ceil(p.NTU, 4)):
                                 E(f"if (wave + {4 * q} < {p.NTU}) {{  // path {p.t}")
                                 E.level += 1
@@ -807,7 +840,7 @@ class UVWGenerator:
                         wcl = wexp if o.mul % 16 == 0 else f"min({wexp}, {o.mul - 1})"
                         E(f"const T* __restrict__ gp{nt} = Gr + {o.off} + ({wcl}) * {o.D};")
                         E("const T " + ", ".join(f"gz{nt}_{k} = gp{nt}[{k}]" for k in range(o.D)) + ";")
-                    for p in self.paths_into(oi):
+                    for p in into(oi):
                         for q in range(_ceil(p.NTU, 4)):
                             E(f"if (wave + {4 * q} < {p.NTU}) {{  // path {p.t}")
                             E.level += 1

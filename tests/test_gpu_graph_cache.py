@@ -162,7 +162,7 @@ def test_unsorted_backward_variant_is_chosen_by_measurement(cuda, monkeypatch):
     monkeypatch.delenv("OEQ_AMD_AUTOTUNE", raising=False)
     prob, oprob = common.channelwise(common.NEQUIP)
     conv = oeq.TensorProductConv(prob, torch_op=True, deterministic=False)
-    assert conv.autotune and conv._bwd_default == "atomic"
+    assert conv.autotune and conv._bwd_default == "grouped"
     host, graph, t, index, g = _inputs(prob, 70, 1500, 13, False, cuda)
     _check(oprob, host, graph, conv, t, index, g)
     assert set(conv.last_tuning) == {"atomic", "grouped"} and len(conv._bwd_choice) == 1

@@ -120,13 +120,14 @@ def test_staged_conv_selection(monkeypatch):
 
 
 def test_unsorted_conv_backward_selection(monkeypatch):
-    """Unsorted edge lists: the backward scatters dX with atomics while a row of X is short, and groups
+    """Unsorted edge lists: the backward scatters dX with atomics while a row of X is very short, and groups
     the edges by sender (four more grouping launches, the segmented backward, larger workspace) from
-    1024 values per edge on."""
+    128 values per edge on."""
     from openequivariance_amd.codegen.uvu_sorted import UVUSortedGenerator
     from openequivariance_amd.problem import ChannelwiseTPP
     monkeypatch.delenv("OEQ_AMD_CONV_BACKWARD", raising=False)
-    small = UVUSortedGenerator(ChannelwiseTPP("32x0e+32x1o+32x2e", "1x0e+1x1o+1x2e", "32x0e+32x1o+32x2e"))
+    small = UVUSortedGenerator(ChannelwiseTPP("8x0e+8x1o+8x2e", "1x0e+1x1o+1x2e", "8x0e+8x1o+8x2e"))
+    assert UVUSortedGenerator(ChannelwiseTPP("32x0e+32x1o+32x2e", "1x0e+1x1o+1x2e", "32x0e+32x1o+32x2e")).grouped_backward
     large = UVUSortedGenerator(ChannelwiseTPP("256x0e+256x1o+256x2e", "1x0e+1x1o+1x2e+1x3o", "256x0e+256x1o+256x2e"))
     assert not small.grouped_backward and large.grouped_backward
     _, bwd, ws = small.plan()
