@@ -88,6 +88,10 @@ class UVUDetGenerator(UVUDirectGenerator):
         self.out_groups = [sorted(g_) for g_ in self.out_groups]
         self.H = H
         self.dy_slots = self.NCH * H               # dY partial rows per edge (summed by backward_dy_reduce)
+        # behind the dY partials: one int per 256 edges, set by the preparation when one of those edges names
+        # a node that does not exist (see emit_invalid_edge_rows)
+        part = f" + {self.dy_slots}ull * nnz * {self.D2} * sizeof(T)" if self.dy_slots > 1 else ""
+        self.flags_off = f"((({self.dypart_off}{part}) + 7ull) & ~7ull)"
         words = max(words_of(g_) for g_ in self.out_groups)
         # fetch the next edge's operands while the current edge is being computed; pays when the
         # per-edge register footprint is small enough to keep several wavefronts per SIMD
@@ -218,6 +222,44 @@ class UVUDetGenerator(UVUDirectGenerator):
     def dy_partial_bytes(self, nnz: int) -> int:
         return self.dy_slots * nnz * self.D2 * self.itemsize if self.dy_slots > 1 else 0
 
+    @staticmethod
+    def flag_bytes(nnz: int) -> int:
+        """Alignment slack + one int per 256 edges (flags of edges naming no node)."""
+        return 8 + 4 * ((nnz + 255) // 256)
+
+    def emit_invalid_edge_rows(self, E: Emitter, grp: int) -> None:
+        """Edges whose sender or receiver is out of range contribute nothing and are never visited by a
+        sender's wavefront (or are visited and skipped), so nobody would write their dW / dY rows.  The
+        preparation kernels leave one flag per 256 edges; the first workgroup of every (chunk, group)
+        launch row ORs them and, only if some edge is flagged, walks the edge list and writes zeros into
+        the rows of those edges: dW and dY (or this launch's dY partial slot)."""
+        E("if (blockIdx.x == 0) {")
+        E.level += 1
+        E("const int* __restrict__ bad_ = (const int*)((const char*)ws + FLAGS_OFF);")
+        E("int any_ = 0;")
+        E("for (u64 q = lane; q < (nnz + 255) / 256; q += 64) any_ |= bad_[q];")
+        for m in (32, 16, 8, 4, 2, 1):
+            E(f"any_ |= oeq_shfl_xor_i32(any_, {m});")
+        E("if (any_) {")
+        E.level += 1
+        E("for (u64 e = lane; e < nnz; e += 64) {")
+        E.level += 1
+        E("const i64 s_ = cols[e], r_ = rows[e];")
+        E("if (s_ >= 0 && s_ < (i64)node_count && r_ >= 0 && r_ < (i64)node_count) continue;")
+        if grp == 0:
+            E(f"if (c == 0) for (int q = 0; q < {self.WN}; ++q) Wg[e * {self.WN} + q] = (T)0;")
+        if self.dy_slots > 1:
+            E(f"{{ T* __restrict__ p_ = (T*)((char*)ws + DYPART_OFF) + ((u64)(c * {self.H} + {grp}) * nnz + e) * {self.D2}; "
+              f"for (int q = 0; q < {self.D2}; ++q) p_[q] = (T)0; }}")
+        elif grp == 0:
+            E(f"if (c == 0) for (int q = 0; q < {self.D2}; ++q) Yg[e * {self.D2} + q] = (T)0;")
+        E.level -= 1
+        E("}")
+        E.level -= 1
+        E("}")
+        E.level -= 1
+        E("}")
+
     def plan(self):
         fwd, bwd, _ = super().plan()
         for s in fwd:
@@ -226,7 +268,7 @@ class UVUDetGenerator(UVUDirectGenerator):
         bwd = [s for s in bwd if s["kernel"] == "prep_backward"] + self.backward_steps()
 
         def ws(nnz=0, nodes=0):
-            return 2 * (nodes + 1) * 8 + self.order_bytes(nodes) + self.dy_partial_bytes(nnz)
+            return 2 * (nodes + 1) * 8 + self.order_bytes(nodes) + self.dy_partial_bytes(nnz) + self.flag_bytes(nnz)
         return fwd, bwd, ws
 
     # ================================================================= forward
@@ -494,6 +536,7 @@ class UVUDetGenerator(UVUDirectGenerator):
         self._node_setup(E, self.bwd_ptr_off, self.bwd_order if self.ordered_backward else None)
         list_t = "IDX" if self.bwd_list == "tperm" else "i64"
         E(f"const {list_t}* __restrict__ elist = {self.bwd_list};     // edge ids in (sender, ...) order")
+        self.emit_invalid_edge_rows(E, grp)
         self._cur_c = "e"
         # this node's own X chunk (fixed over the edge loop)
         E("bool rv = nv;")

@@ -56,6 +56,9 @@ class UVURecvGenerator(UVUDetGenerator):
         self.dypart_off = "(2 * (node_count + 1) + node_count) * sizeof(i64)"
         self.spill_off = (f"((({self.dypart_off} + {self.dy_slots if self.dy_slots > 1 else 0}ull * nnz * {self.D2} * sizeof(T)) "
                           "+ 255ull) & ~255ull)")
+        # the preparation's per-256-edge flags are not used here (pass 1 visits every edge and writes the
+        # rows of edges naming no node itself): they go behind the spill
+        self.flags_off = f"({self.spill_off} + nnz * {self.spill_row}ull * sizeof(T))"
 
     def describe(self) -> str:
         return super().describe() + f" receiver-order backward (spill {self.spill_row} words/edge)"
@@ -78,7 +81,7 @@ class UVURecvGenerator(UVUDetGenerator):
 
         def ws(nnz=0, nodes=0):
             head = (2 * (nodes + 1) + nodes) * 8 + self.dy_partial_bytes(nnz)
-            return ((head + 255) & ~255) + self.spill_bytes(nnz)
+            return ((head + 255) & ~255) + self.spill_bytes(nnz) + self.flag_bytes(nnz)
         return fwd, bwd, ws
 
     def backward_kernel_sources(self):
@@ -186,13 +189,15 @@ class UVURecvGenerator(UVUDetGenerator):
                     E(f"const T g{k} = G{oi}_{k};")
 
                 def sink(E, p, v, expr):
-                    E(f"  if ({self.act(p.a)}) {self.st('Wgr', self.widx(p, 'u', v), expr)}")
+                    # (an edge that names no node has x = 0, hence dW = dY = 0: its rows are written like any other)
+                    ok = "cur_ev" if self.full(p.a) else f"(cur_ev && u < {p.a.mul})"
+                    E(f"  if ({ok}) {self.st('Wgr', self.widx(p, 'u', v), expr)}")
                 self.emit_backward_block(E, o, "Wr", sink)
                 E.level -= 1
                 E("}")
             self.emit_dy_sum(E)
             writer = "ul == 0" if P < 64 else "lane == 63"
-            E(f"if (rv && {writer}) {{")
+            E(f"if (cur_ev && {writer}) {{")
             if self.dy_slots > 1:
                 E(f"    T* __restrict__ Ygr = (T*)((char*)ws + DYPART_OFF) + ((u64)c * nnz + e) * {self.D2};")
             else:

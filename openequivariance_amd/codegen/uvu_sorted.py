@@ -92,5 +92,5 @@ class UVUSortedGenerator:
         bwd += b.backward_steps()
 
         def ws(nnz=0, nodes=0):
-            return 2 * (2 * (nodes + 1) + nnz) * 8 + b.order_bytes(nodes) + b.dy_partial_bytes(nnz)
+            return 2 * (2 * (nodes + 1) + nnz) * 8 + b.order_bytes(nodes) + b.dy_partial_bytes(nnz) + b.flag_bytes(nnz)
         return fwd, bwd, ws

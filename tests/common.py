@@ -77,3 +77,26 @@ def conv_inputs(prob, nodes, nnz, seed, dtype=np.float32, sh_lmax=None):
     W = rng.standard_normal((nnz, prob.weight_numel))
     G = rng.standard_normal((nodes, d3))
     return tuple(np.ascontiguousarray(a.astype(dtype)) for a in (X, Y, W, G))
+
+
+def with_invalid_edges(rows, cols, nodes, seed, count=7):
+    """A copy of the edge list in which ``count`` edges name a node that does not exist (sender or
+    receiver negative or >= nodes), and the mask of the edges left valid."""
+    rng = np.random.default_rng(seed)
+    rows, cols = rows.copy(), cols.copy()
+    bad = rng.choice(rows.size, size=min(count, rows.size), replace=False)
+    for k, e in enumerate(bad):
+        target = rows if k % 2 == 0 else cols
+        target[e] = (-1 - k) if k % 3 == 0 else nodes + k
+    valid = (rows >= 0) & (rows < nodes) & (cols >= 0) & (cols < nodes)
+    return rows, cols, valid
+
+
+def conv_reference_on_valid_edges(otp, oprob, X, Y, W, G, rows, cols, valid):
+    """Oracle outputs when edges outside ``valid`` contribute nothing: Z and dX from the valid sub-graph,
+    dY / dW rows of the other edges zero."""
+    Z = otp.conv_forward(oprob, X, Y[valid], W[valid], rows[valid], cols[valid])
+    dX, dYv, dWv = otp.conv_backward(oprob, X, Y[valid], W[valid], G, rows[valid], cols[valid])
+    dY, dW = np.zeros_like(Y, dtype=np.float64), np.zeros_like(W, dtype=np.float64)
+    dY[valid], dW[valid] = dYv, dWv
+    return Z, dX, dY, dW

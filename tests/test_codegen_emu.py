@@ -145,6 +145,36 @@ def test_conv_receiver_order_backward(irreps, nodes, nnz, prefetch):
         assert rel_err(got, ref) < TOL
 
 
+@pytest.mark.parametrize("variant", ["det", "det_two_chunks", "grouped", "recv"])
+def test_conv_edges_naming_no_node(variant):
+    """Edges whose sender or receiver is out of range contribute nothing, and their dW / dY rows come
+    out as zeros from every backward variant (the emulator starts all outputs from junk)."""
+    from openequivariance_amd.codegen.uvu_recv import UVURecvGenerator
+    irreps = ("70x0e+70x1o", "1x0e+1x1o", "70x0e+70x1o") if variant == "det_two_chunks" else \
+        ("8x0e+8x1o", "1x0e+1x1o+1x2e", "8x0e+8x1o+8x2e")
+    prob, oprob = common.channelwise(irreps)
+    nodes, nnz = 9, 300 if variant != "det_two_chunks" else 40
+    rows, cols = common.random_graph(nodes, nnz, 5, self_loops=True)
+    rows, cols, valid = common.with_invalid_edges(rows, cols, nodes, 6)
+    tperm = None
+    if variant != "grouped":
+        order = np.lexsort((cols, rows))
+        rows, cols, valid = rows[order], cols[order], valid[order]
+        tperm = np.lexsort((np.arange(nnz), rows, cols)).astype(np.int64)
+    g = {"det": UVUDetGenerator, "det_two_chunks": UVUDetGenerator, "recv": UVURecvGenerator,
+         "grouped": lambda p: UVUSortedGenerator(p, grouped_backward=True)}[variant](prob)
+    X, Y, W, G = common.conv_inputs(prob, nodes, nnz, 8)
+    Zr, dXr, dYr, dWr = common.conv_reference_on_valid_edges(otp, oprob, X, Y, W, G, rows, cols, valid)
+    fwd, bwd, ws = g.plan()
+    junk = np.full(nnz, 12345, dtype=np.int64)
+    tp = junk if variant == "grouped" else tperm
+    out = emu.run_conv(g, fwd, X, Y, W, rows, cols, tperm=tp, ws_bytes=ws(nnz, nodes))
+    assert rel_err(out["Z"], Zr) < TOL
+    out = emu.run_conv(g, bwd, X, Y, W, rows, cols, G=G, tperm=tp, ws_bytes=ws(nnz, nodes))
+    assert rel_err(out["Xg"], dXr) < TOL and rel_err(out["Yg"], dYr) < TOL and rel_err(out["Wg"], dWr) < TOL
+    assert not out["Wg"][~valid].any() and not out["Yg"][~valid].any()
+
+
 def test_conv_det_chunked_ragged():
     irreps = ("5x0e+3x1o+70x2e", "1x0e+1x1o+1x2e", "5x0e+3x1o+70x2e+7x3o")
     prob, oprob = common.channelwise(irreps)

@@ -110,6 +110,48 @@ def test_tensor_product_rejects_host_tensors_among_gpu_tensors(cuda):
     torch.cuda.synchronize()
 
 
+@pytest.mark.parametrize("variant", ["det", "det_recv", "unsorted_atomic", "unsorted_grouped"])
+@pytest.mark.parametrize("irreps", [common.NEQUIP, common.LARGE], ids=["nequip", "large"])
+def test_edges_naming_no_node_contribute_nothing(cuda, variant, irreps, monkeypatch):
+    """Out-of-range senders / receivers: no fault, Z and dX as if those edges were absent, and their dW /
+    dY rows are zeros from every backward variant."""
+    import torch
+    import openequivariance_amd as oeq
+    from oracle import tp as otp
+    monkeypatch.setenv("OEQ_AMD_AUTOTUNE", "0")
+    if variant == "det_recv":
+        monkeypatch.setenv("OEQ_AMD_DET_BACKWARD", "recv")
+    if variant.startswith("unsorted"):
+        monkeypatch.setenv("OEQ_AMD_CONV_BACKWARD", variant.split("_")[1])
+    deterministic = variant.startswith("det")
+    prob, oprob = common.channelwise(irreps)
+    nodes, nnz = 40, 900
+    rows, cols = common.random_graph(nodes, nnz, 71, self_loops=True)
+    rows, cols, valid = common.with_invalid_edges(rows, cols, nodes, 72, count=9)
+    index = [rows, cols]
+    if deterministic:
+        order = np.lexsort((cols, rows))
+        rows, cols, valid = rows[order], cols[order], valid[order]
+        index = [rows, cols, np.lexsort((np.arange(nnz), rows, cols)).astype(np.int64)]
+    X, Y, W, G = common.conv_inputs(prob, nodes, nnz, 73)
+    Zr, dXr, dYr, dWr = common.conv_reference_on_valid_edges(otp, oprob, X, Y, W, G, rows, cols, valid)
+    conv = oeq.TensorProductConv(prob, torch_op=True, deterministic=deterministic)
+    x, y, w = (torch.tensor(a, device=cuda, requires_grad=True) for a in (X, Y, W))
+    idx = [torch.tensor(a, device=cuda) for a in index]
+    for _ in range(2):                               # second pass: graph preparation reused
+        for t in (x, y, w):
+            t.grad = None
+        z = conv.forward(x, y, w, *idx)
+        z.backward(torch.tensor(G, device=cuda))
+        torch.cuda.synchronize()
+        assert common.rel_err(z.detach().cpu().numpy(), Zr) <= common.FP32_TOL
+        assert common.rel_err(x.grad.cpu().numpy(), dXr) <= common.FP32_TOL
+        assert common.rel_err(y.grad.cpu().numpy(), dYr) <= common.FP32_TOL
+        assert common.rel_err(w.grad.cpu().numpy(), dWr) <= common.FP32_TOL
+        bad = torch.tensor(~valid, device=cuda)
+        assert not w.grad[bad].any() and not y.grad[bad].any()
+
+
 def test_unsupported_problems_raise():
     import openequivariance_amd as oeq
     with pytest.raises(AssertionError):           # the convolution needs multiplicity 1 on the second operand

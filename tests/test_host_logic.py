@@ -45,7 +45,8 @@ def test_launch_plans():
     assert [s["kernel"] for s in fwd] == ["prep_forward", "forward"] and fwd[1]["grid_y"] == 4
     assert [s["kernel"] for s in bwd] == ["prep_backward", "order_backward", "backward", "backward_dy_reduce"]
     assert bwd[1]["num_blocks"] == 1
-    assert ws(1000, 10) == 2 * 11 * 8 + 10 * 8 + 4 * 1000 * 16 * 4       # pointers | node order | dY partials
+    flags = 8 + 4 * 4                                                   # one int per 256 edges (+ alignment slack)
+    assert ws(1000, 10) == 2 * 11 * 8 + 10 * 8 + 4 * 1000 * 16 * 4 + flags       # pointers | node order | dY partials | flags
     prob, _ = common.fully_connected(common.DENSE)
     fwd, bwd, ws = UVWGenerator(prob).plan()
     assert [s["kernel"] for s in bwd] == ["prep_backward", "backward", "backward_dw", "backward_reduce"]
@@ -138,7 +139,7 @@ def test_unsorted_conv_backward_selection(monkeypatch):
                                           "group_fill_backward", "order_backward", "backward", "backward_dy_reduce"]
     assert bwd[5]["grid_y"] == 4 and bwd[5]["work_per_block"] == 1
     # the forward's grouping and the backward's lie side by side (a prepared workspace serves both)
-    assert ws(1000, 10) == (2 * (2 * 11 + 1000) + 10) * 8 + 4 * 1000 * 16 * 4
+    assert ws(1000, 10) == (2 * (2 * 11 + 1000) + 10) * 8 + 4 * 1000 * 16 * 4 + 8 + 4 * 4
     assert all(s.get("prep") for s in bwd[:5]) and not any(s.get("prep") for s in bwd[5:])
     src = large.render()
     for name in ("group_fill_backward", "backward_dy_reduce", "void backward("):
@@ -157,7 +158,7 @@ def test_backward_split_over_output_block_groups():
     assert sorted(sum(mace.out_groups, [])) == mace.used_out and all(mace.out_groups)
     _, bwd, ws = mace.plan()
     assert [s["kernel"] for s in bwd] == ["prep_backward", "order_backward", "backward", "backward_g1", "backward_dy_reduce"]
-    assert ws(1000, 10) == (2 * 11 + 10) * 8 + 4 * 1000 * 16 * 4
+    assert ws(1000, 10) == (2 * 11 + 10) * 8 + 4 * 1000 * 16 * 4 + 8 + 4 * 4
     src = mace.render()
     assert "void backward_g1(" in src and "c * 2 + 1" in src
     with mace._group(1):
