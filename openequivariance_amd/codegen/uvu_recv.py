@@ -49,10 +49,15 @@ class UVURecvGenerator(UVUDetGenerator):
         # registers: dZ of the receiver + one or two sets of (X records, weights, Y)
         held = sum(self.out[i].D for i in self.used_out)
         per_edge = self.NW + sum(p.mv for p in self.paths) + len(self.used_y)
-        env = os.environ.get("OEQ_AMD_RECV_PREFETCH")
-        self.prefetch_edges = (held + 2 * per_edge <= 190) if env not in ("0", "1") else env == "1"
+        # One register set measured faster than two on every shape tried (config 3: 0.182 vs 0.202 ms,
+        # config 5: 7.93 vs 8.01 ms, the 128-channel MACE problem: 2.14 vs 5.05 ms, where two sets leave one
+        # wavefront per SIMD); OEQ_AMD_RECV_PREFETCH=1 turns the second set on for A/B runs.
+        self.prefetch_edges = os.environ.get("OEQ_AMD_RECV_PREFETCH", "0") == "1"
         if prefetch is not None:
             self.prefetch_edges = prefetch
+        # large per-edge footprints: hold the allocation to two wavefronts per SIMD (a handful of spilled
+        # words) instead of one
+        self.waves_hint = 2 if held + per_edge > 100 else 0
         self.dypart_off = "(2 * (node_count + 1) + node_count) * sizeof(i64)"
         self.spill_off = (f"((({self.dypart_off} + {self.dy_slots if self.dy_slots > 1 else 0}ull * nnz * {self.D2} * sizeof(T)) "
                           "+ 255ull) & ~255ull)")
@@ -85,7 +90,7 @@ class UVURecvGenerator(UVUDetGenerator):
         return fwd, bwd, ws
 
     def backward_kernel_sources(self):
-        w = int(os.environ.get("OEQ_AMD_RECV_WAVES", "0"))
+        w = int(os.environ.get("OEQ_AMD_RECV_WAVES", str(self.waves_hint)))
         attr = f" __attribute__((amdgpu_waves_per_eu({w}, {w})))" if w else ""
         return [dict(name="backward", threads=64, attr=attr, body=self._edges_body()),
                 dict(name="backward_dx", threads=64, attr="", body=self._dx_body())]
