@@ -32,9 +32,9 @@ from .uvu_det import UVUDetGenerator
 
 
 class UVURecvGenerator(UVUDetGenerator):
-    MIN_TILE_ITERS = 8           # edge-loop iterations of the smallest tile
-    MAX_TILES = 16384            # tiles per chunk of the largest launches (the tile then grows with the edge count)
-    DX_UNROLL = 4                # spill rows in flight per lane group in pass 2
+    MIN_TILE_ITERS = int(os.environ.get("OEQ_AMD_RECV_MIN_ITERS", "8"))       # edge-loop iterations of the smallest tile
+    MAX_TILES = int(os.environ.get("OEQ_AMD_RECV_MAX_TILES", "16384"))       # tiles per chunk of the largest launches (the tile then grows with the edge count)
+    DX_UNROLL = int(os.environ.get("OEQ_AMD_RECV_DX_UNROLL", "4"))           # spill rows in flight per lane group in pass 2
 
     def __init__(self, problem: TPProblem, vector_stores: bool = True, idx_ctype: str = "i64", prefetch=None):
         # pass 1 is one launch: the per-edge dX rows cannot be split over launches of output-block groups
