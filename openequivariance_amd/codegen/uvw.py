@@ -93,6 +93,12 @@ class WPath:
 class UVWGenerator:
     DW_WORKGROUPS = 256          # persistent dW workgroups: one per compute unit of an MI355X
     FWD_ACC_LIMIT = 80           # accumulator registers of one forward work item
+    # forward with the X tile in LDS, one workgroup per tile: "0", "1" or "auto" (when the tile fits the bound
+    # below).  Measured slower than one wavefront per work item (fp32 394 vs 359 us, fp64 747 vs 620 us on
+    # 64x0e+64x1o+64x2e: the wavefronts of a tile differ 7 : 4 : 1 in work and hold the tile's LDS until the
+    # longest is done), so it is off.
+    FWD_LDS_DEFAULT = "0"
+    FWD_LDS_MAX_BYTES = 40 * 1024
 
     def __init__(self, problem: TPProblem):
         self.problem = problem
@@ -173,6 +179,12 @@ class UVWGenerator:
         # conflicts of the B-operand reads: lanes c = 0..15 read 16 different rows at the same column)
         self.bwd_rs = self._pick_row_stride()
         self.bwd_lds = self._bwd_lds_env and 16 * self.bwd_rs * self.itemsize <= 80 * 1024    # gfx950: 160 KB per CU
+        # forward: the 16-row X tile staged in LDS once per workgroup, one wavefront per work item
+        self.fwd_xrs = self._pick_x_row_stride()
+        mode = os.environ.get("OEQ_AMD_UVW_FWD_LDS", self.FWD_LDS_DEFAULT)
+        fits = 16 * self.fwd_xrs * self.itemsize <= self.FWD_LDS_MAX_BYTES
+        self.fwd_lds = (mode == "1") or (mode == "auto" and fits)
+        self.fwd_waves = min(len(self.fwd_order), 8) if self.fwd_lds else 1
         # packed weight copies in the workspace
         pos = 0
         for p in self.paths:
@@ -190,6 +202,21 @@ class UVWGenerator:
         self.ws_elems = self.PART_OFF + self.DW_WORKGROUPS * self.WN
 
     # ------------------------------------------------------------------ helpers
+    def fwd_group_of(self, o: Block) -> int:
+        """K steps fetched per batch of loads in the forward work item of output block ``o``: the fewer matrix
+        instructions a step has (2l+1 per w tile), the more steps one batch must cover for the next batch's
+        operands to arrive in time."""
+        per_l = os.environ.get("OEQ_AMD_UVW_GROUPS", "")
+        if per_l:
+            tab = [int(v) for v in per_l.split(",")]
+            return tab[min(o.l, len(tab) - 1)]
+        return self.fwd_group
+
+    def forward_attr(self) -> str:
+        """Occupancy target of the forward kernel (wavefronts per SIMD), when one is set."""
+        w = int(os.environ.get("OEQ_AMD_UVW_FWD_OCC", "0"))
+        return f" __attribute__((amdgpu_waves_per_eu({w}, {w})))" if w else ""
+
     def backward_attr(self) -> str:
         """Occupancy target of the dX/dY kernel: as many workgroups per CU (one wavefront per SIMD
         each) as the LDS tile allows; the register allocator then stays within that budget."""
@@ -197,6 +224,26 @@ class UVWGenerator:
             return ""
         per_cu = max(1, min(4, (160 * 1024) // (16 * self.bwd_rs * self.itemsize + 4 * 16 * max(1, self.D2) * self.itemsize)))
         return f" __attribute__((amdgpu_waves_per_eu({per_cu}, {per_cu})))" if per_cu >= 3 else ""
+
+    def _pick_x_row_stride(self) -> int:
+        """Row stride (elements) of the X tile in LDS: a multiple of the 16-byte vector the tile is written
+        with, padded so that the 16 rows x 2 lane groups of one LDS pass spread best over the 32 banks."""
+        words, vw = self.itemsize // 4, 16 // self.itemsize
+        base = _ceil(self.D1, vw) * vw
+        best = None
+        for pad in range(0, 33, vw):
+            rs = base + pad
+            worst = 0
+            for d in {a.D for a in self.in1 if a.dim}:
+                hits = {}
+                for c in range(16):
+                    for g in range(2):
+                        bank = ((c * rs + g * 4 * d) * words) % 32
+                        hits[bank] = hits.get(bank, 0) + 1
+                worst = max(worst, max(hits.values()))
+            if best is None or worst < best[0]:
+                best = (worst, rs)
+        return best[1]
 
     def _pick_row_stride(self) -> int:
         """Row stride (elements) of the dZ tile in LDS: the smallest padding for which the 32 lanes of
@@ -333,18 +380,24 @@ class UVWGenerator:
     def forward_body(self) -> str:
         E = Emitter()
         NO = len(self.fwd_order)
+        if self.fwd_lds:
+            return self._forward_items(E, self._forward_lds_head(E))
         E("const int lane = threadIdx.x, c = lane & 15, g = lane >> 4;")
         if self.fwd_xcd_map:
             # Work item = (batch tile, output block).  Workgroups are handed to the 8 XCDs round robin by
             # their linear id, and every XCD has an L2 of its own: the items of one tile get ids 8 apart,
             # i.e. consecutive turns of the same XCD, so that the X rows fetched for the first output
-            # block are still in that L2 for the others.  The tiles beyond the last multiple of 8 are
-            # mapped plainly.
+            # block are still in that L2 for the others.
             E("const u64 ntiles = gridDim.x, lin = blockIdx.x + (u64)blockIdx.y * gridDim.x;")
-            E(f"const u64 full = (ntiles >> 3) * {8 * NO};")
+            # The last fifth of the tiles is laid out item-major instead (all their most expensive items, then
+            # the next ...): the launch then ends on the cheap items, which shortens its ragged end
+            # (measured: forward 356 -> 346 us in fp32, 616 -> 598 us in fp64; a third or a half: no better).
+            tail = int(os.environ.get("OEQ_AMD_UVW_FWD_TAIL", "5"))
+            head8 = f"((ntiles - ntiles / {tail}) >> 3)" if tail else "(ntiles >> 3)"
+            E(f"const u64 head = {head8} << 3, full = head * {NO};")
             E("u64 tile; int slot;")
             E(f"if (lin < full) {{ const u64 j = lin >> 3; slot = (int)(j % {NO}); tile = (j / {NO}) * 8 + (lin & 7); }}")
-            E("else { const u64 rem = ntiles & 7, l2 = lin - full; slot = (int)(l2 / rem); tile = (ntiles & ~(u64)7) + l2 % rem; }")
+            E("else { const u64 rem = ntiles - head, l2 = lin - full; slot = (int)(l2 / rem); tile = head + l2 % rem; }")
         else:
             E("const u64 tile = blockIdx.x; const int slot = blockIdx.y;")
         E("const u64 row0 = tile * 16;")
@@ -357,10 +410,55 @@ class UVWGenerator:
         # One work item = (batch tile, output block): blockIdx.y walks the output blocks from the most
         # to the least expensive, so the dispatcher fills the tail of the launch with the cheap ones
         # (whole tiles per wavefront leave a third of the machine idle in the last round).
+        return self._forward_items(E, lambda slot: f"slot == {slot}")
+
+    def _forward_lds_head(self, E: Emitter):
+        """Workgroup = one batch tile, one wavefront per work item.  The 16 rows of X are contiguous in
+        memory: the workgroup copies them into LDS with 16-byte vectors that are all requested before the
+        first is written, and the K loops read their X records from there - X crosses the memory system
+        once, with one exposed round trip per tile instead of one per path and work item.  Returns the
+        condition that selects a work item."""
+        NWV, RS, VW = self.fwd_waves, self.fwd_xrs, self.VW
+        NTH = 64 * NWV
+        E("const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;")
+        E("const u64 row0 = (u64)blockIdx.x * 16;")
+        E("if (row0 >= n) return;")
+        E("const u64 rowA = min(row0 + (u64)c, n - 1);       // rows past the end repeat the last row, never stored")
+        E("const T* __restrict__ wsT = (const T*)ws;")
+        E(f"__shared__ T xl[16 * {RS}];")
+        for f in self.used_y:
+            E(f"const T y{f} = Y[rowA * {self.D2} + {f}];")
+        if self.D1 % VW == 0:
+            NV, RV = 16 * self.D1 // VW, self.D1 // VW
+            NQ = _ceil(NV, NTH)
+            E("if ((((unsigned long long)X) & 15ull) == 0) {")
+            E.level += 1
+            E(f"VT xv[{NQ}];")
+            for q in range(NQ):
+                idx = f"(int)threadIdx.x + {NTH * q}"
+                guard = "" if NTH * (q + 1) <= NV else f"if ({idx} < {NV}) "
+                E(f"{guard}{{ const int r_ = ({idx}) / {RV}, v_ = ({idx}) - r_ * {RV}; "
+                  f"xv[{q}] = *(const VT*)(X + min(row0 + (u64)r_, n - 1) * {self.D1} + v_ * {VW}); }}")
+            for q in range(NQ):
+                idx = f"(int)threadIdx.x + {NTH * q}"
+                guard = "" if NTH * (q + 1) <= NV else f"if ({idx} < {NV}) "
+                E(f"{guard}{{ const int r_ = ({idx}) / {RV}, v_ = ({idx}) - r_ * {RV}; T* __restrict__ d_ = xl + r_ * {RS} + v_ * {VW}; "
+                  + " ".join(f"d_[{i}] = xv[{q}][{i}];" for i in range(VW)) + " }")
+            E.level -= 1
+            E("} else")
+        E(f"for (int q = threadIdx.x; q < 16 * {self.D1}; q += {NTH}) {{")
+        E(f"    const int r_ = q / {self.D1}, col_ = q - r_ * {self.D1};")
+        E(f"    xl[r_ * {RS} + col_] = X[min(row0 + (u64)r_, n - 1) * {self.D1} + col_];")
+        E("}")
+        E("__syncthreads();")
+        E(f"const T* __restrict__ Xr = xl + c * {RS};")
+        return lambda slot: f"wave == {slot % NWV}"
+
+    def _forward_items(self, E: Emitter, select) -> str:
         for slot, (o, nt_lo, nt_hi) in enumerate(self.fwd_order):
             NT = _ceil(o.mul, 16)
             NTS = range(nt_lo, nt_hi)
-            E(f"if (slot == {slot}) {{ // output block {o.idx}: {o.mul}x l={o.l}, w tiles {nt_lo} .. {nt_hi - 1} of {NT}")
+            E(f"if ({select(slot)}) {{ // output block {o.idx}: {o.mul}x l={o.l}, w tiles {nt_lo} .. {nt_hi - 1} of {NT}")
             E.level += 1
             if o.idx not in self.used_out:
                 for r in range(4):
@@ -379,7 +477,7 @@ class UVWGenerator:
                 # matrix core.  What bounds this kernel is the L2 -> L1 stream of operands (every
                 # wavefront re-reads the packed weights), so the bytes in flight per wavefront matter
                 # more than anything else here.
-                GS = self.fwd_group
+                GS = self.fwd_group_of(o)
                 NG = _ceil(p.SU, GS)
                 pingpong = (self.fwd_unroll == 0)
                 sets = ("a", "b") if pingpong else ("n",)
@@ -896,7 +994,8 @@ class UVWGenerator:
     def plan(self):
         FIXED, ROW = 0, 1
         fwd = [dict(kernel="prep_forward", num_threads=256, grid_kind=FIXED, num_blocks=self.prep_blocks),
-               dict(kernel="forward", num_threads=64, grid_kind=ROW, work_per_block=16, grid_y=len(self.fwd_order))]
+               dict(kernel="forward", num_threads=64 * self.fwd_waves, grid_kind=ROW, work_per_block=16,
+                    grid_y=1 if self.fwd_lds else len(self.fwd_order))]
         bwd = [dict(kernel="prep_backward", num_threads=256, grid_kind=FIXED, num_blocks=self.prep_blocks),
                dict(kernel="backward", num_threads=256, grid_kind=ROW, work_per_block=16),
                dict(kernel="backward_dw", num_threads=256 * self.dw_groups, grid_kind=FIXED,

@@ -208,6 +208,36 @@ def test_uvw_matrix_core_kernels(dtype, monkeypatch):
     assert rel_err(ow.oeq_to_e3nn(oprob, out["Wg"]), dW) < tol
 
 
+def test_uvw_forward_work_item_mapping_over_many_tiles():
+    """19 batch tiles: 16 of them in groups of 8 with the items of a tile 8 workgroup ids apart, the last three
+    item-major; every (tile, item) pair must be visited exactly once."""
+    a = ("4x0e+4x1o", "1x0e+1x1o", "4x0e+4x1o+4x1e")
+    prob, oprob = common.fully_connected(a, shared=True)
+    g = UVWGenerator(prob)
+    X, Y, We, _ = common.tp_inputs(prob, 300, 12, w_scale=0.3)
+    fwd, _, ws = g.plan()
+    out = emu.run_tp(g, fwd, X, Y, ow.e3nn_to_oeq(oprob, We), ws_bytes=ws())
+    assert rel_err(out["Z"], otp.forward(oprob, X, Y, We)) < TOL
+
+
+@pytest.mark.parametrize("dtype,a,n", [(np.float32, ("5x0e+21x1o", "1x0e+1x1o+1x2e", "18x0e+7x1o+3x2e"), 21),
+                                       (np.float64, ("16x0e+16x1o+4x2e", "1x0e+1x1o", "16x0e+20x1o"), 16),
+                                       (np.float32, ("3x0e+2x1o+1x2e", "1x0e+1x1o", "4x0e+4x1o+4x1e+4x2e+2x2o"), 35)])
+def test_uvw_forward_with_the_x_tile_in_lds(dtype, a, n, monkeypatch):
+    """One workgroup per batch tile, one wavefront per output block, X read through LDS (vector fill when the
+    row length allows it, element-wise otherwise; last tile partial)."""
+    monkeypatch.setenv("OEQ_AMD_UVW_FWD_LDS", "1")
+    prob, oprob = common.fully_connected(a, shared=True, dtype=dtype)
+    g = UVWGenerator(prob)
+    assert g.fwd_lds and g.fwd_waves == len(g.fwd_order)
+    X, Y, We, _ = common.tp_inputs(prob, n, 11, dtype, w_scale=0.3)
+    W = ow.e3nn_to_oeq(oprob, We)
+    fwd, _, ws = g.plan()
+    assert fwd[1]["num_threads"] == 64 * g.fwd_waves and fwd[1]["grid_y"] == 1
+    out = emu.run_tp(g, fwd, X, Y, W, ws_bytes=ws())
+    assert rel_err(out["Z"], otp.forward(oprob, X, Y, We)) < (TOL if dtype == np.float32 else 1e-13)
+
+
 @pytest.mark.parametrize("shared", [False, True])
 def test_uvu_run_time_loop_over_second_operand_copies(shared, monkeypatch):
     """mul(in2) = 11 > 8: v is walked at run time; dY sums through the LDS accumulator, shared dW through
