@@ -252,6 +252,60 @@ def copy_calibration(steps):
                       "bytes_written_per_launch": nbytes, "launches": steps}))
 
 
+ROW_SHAPE_SRC = r"""
+// Copy kernel in the shape of the uvu batch product: one workgroup of WPR wavefronts per row reads RD
+// and writes WR pieces of 1 KB of that row (the pieces dealt to the wavefronts in contiguous ranges),
+// all loads issued before the first store.  NT = 1: non-temporal accesses.
+typedef float v4 __attribute__((ext_vector_type(4)));
+extern "C" __global__ __launch_bounds__(64 * WPR) void oeq_row_shape_probe(const v4* __restrict__ in, v4* __restrict__ out) {
+    const unsigned row = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const v4* ip = in + (unsigned long long)row * (RD * 64) + lane;
+    v4* op = out + (unsigned long long)row * (WR * 64) + lane;
+    constexpr int NR = (RD + WPR - 1) / WPR, NW = (WR + WPR - 1) / WPR;
+    v4 r[NR], acc = (v4)(0.f);
+#pragma unroll
+    for (int i = 0; i < NR; ++i) { const int pc = wave * NR + i; r[i] = pc < RD ? (NT ? __builtin_nontemporal_load(ip + pc * 64) : ip[pc * 64]) : (v4)(0.f); }
+#pragma unroll
+    for (int i = 0; i < NR; ++i) acc += r[i];
+#pragma unroll
+    for (int i = 0; i < NW; ++i) {
+        const int pc = wave * NW + i;
+        if (pc < WR) { const v4 v = acc + (float)i; if (NT) __builtin_nontemporal_store(v, op + pc * 64); else op[pc * 64] = v; }
+    }
+}
+"""
+
+
+def row_shape_probe(read_kb, write_kb, rows=50000, reps=5):
+    """GB/s of copy kernels that move ``read_kb`` in and ``write_kb`` out per row with 1, 2 or 4 wavefronts
+    per row, temporal and non-temporal: what the memory system sustains for the row-per-workgroup shape of
+    the uvu batch kernels (forward 13 : 36 KB, backward 49 : 13 KB per row of the 128-channel MACE problem)."""
+    import ctypes as C
+    import torch
+    from openequivariance_amd import runtime as rt
+    stream = torch.cuda.current_stream().cuda_stream
+    src = torch.zeros(rows * read_kb * 256, dtype=torch.float32, device="cuda")
+    dst = torch.empty(rows * write_kb * 256, dtype=torch.float32, device="cuda")
+    table = {}
+    for wpr in (1, 2, 4):
+        for nt in (0, 1):
+            opts = tuple(rt.DEFAULT_OPTIONS) + (f"-DWPR={wpr}", f"-DNT={nt}", f"-DRD={read_kb}", f"-DWR={write_kb}")
+            mod = rt.Module(rt.compile_source(ROW_SHAPE_SRC, options=opts))
+            args = [C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr())]
+            best = float("inf")
+            for r in range(reps + 2):
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                mod.launch("oeq_row_shape_probe", rows, 64 * wpr, args, stream=stream)
+                b.record()
+                b.synchronize()
+                if r >= 2:
+                    best = min(best, a.elapsed_time(b))
+            table[f"{wpr} wavefront{'s' if wpr > 1 else ''} per row, {'non-temporal' if nt else 'plain'}"] = \
+                {"GB/s": round(rows * (read_kb + write_kb) * 1024 / (best * 1e-3) / 1e9, 1), "us": round(best * 1e3, 1)}
+    return table
+
+
 def stream_calibration():
     """Sustained rate of plain streaming kernels for several read:write mixes: the whole sweep per
     mix, its best variant, and torch's own elementwise kernels beside it."""
@@ -260,6 +314,8 @@ def stream_calibration():
         best, label, table = stream_probe(nr, nw)
         out["mixes"][f"read{nr}_write{nw}"] = {"best": best, "best_variant": label, "sweep": table}
     out["torch"] = torch_stream_reference()
+    out["row_shape"] = {"uvu forward, 13 KB in / 36 KB out per row": row_shape_probe(13, 36),
+                        "uvu backward, 49 KB in / 13 KB out per row": row_shape_probe(49, 13)}
     print(json.dumps(out))
 
 

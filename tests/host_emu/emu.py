@@ -51,7 +51,8 @@ static pthread_barrier_t g_bar;
 static T g_xT[1024];
 static int g_xi[1024];
 static std::mutex g_atomic_mutex;
-static inline void oeq_sync() { pthread_barrier_wait(&g_bar); }
+static pthread_barrier_t g_wbar[16];             // one per wavefront of the workgroup
+static inline void oeq_sync() { pthread_barrier_wait(&g_wbar[threadIdx.x >> 6]); }
 static inline T oeq_fma(T a, T b, T c) { return std::fma(a, b, c); }
 static inline void oeq_atomic_add(T* p, T v) { std::lock_guard<std::mutex> g(g_atomic_mutex); *p += v; }
 static inline T oeq_shfl_xor(T v, int mask) { g_xT[threadIdx.x] = v; oeq_sync(); T r = g_xT[threadIdx.x ^ mask]; oeq_sync(); return r; }
@@ -74,7 +75,6 @@ static inline void __syncthreads() { pthread_barrier_wait(&g_bar); }
 template <class V> static inline V __hip_atomic_fetch_add(V* p, V v, int, int) { std::lock_guard<std::mutex> g(g_atomic_mutex); V o = *p; *p += v; return o; }
 // matrix-core step of one wavefront, emulated collectively by its 64 threads
 struct V4 { T v[4]; T& operator[](int i) { return v[i]; } const T& operator[](int i) const { return v[i]; } };
-static pthread_barrier_t g_wbar[16];
 static T g_mA[16][16][4], g_mB[16][4][16];
 static inline V4 oeq_mfma(T a, T b, V4 c) {
     const int wv = threadIdx.x >> 6, l = threadIdx.x & 63;

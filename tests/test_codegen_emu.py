@@ -39,6 +39,20 @@ def test_direct_tp_ragged_two_chunks():
     _tp(UVUDirectGenerator, ("5x0e+3x1o+70x2e", "1x0e+1x1o+1x2e", "5x0e+3x1o+70x2e+7x3o"), 3, 2)
 
 
+@pytest.mark.parametrize("irreps,waves", [(("64x0e+64x1o+64x2e", "1x0e+1x1o+1x2e", "64x0e+64x1o+64x2e+64x1e"), 4),
+                                          (("70x0e+100x1o", "1x0e+1x1o+1x2e", "70x0e+70x1o+100x1o+100x2e"), 3),
+                                          (("128x0e+128x1o", "1x0e+1x1o", "128x0e+128x1o+128x1o+128x0e"), 2)])
+def test_direct_tp_row_dealt_to_several_wavefronts(irreps, waves, monkeypatch):
+    """One row per workgroup of 2-4 wavefronts: contiguous parts of the Z / dZ row each, dX and dY combined
+    through LDS in a fixed order (full and ragged chunks, one and two chunks, blocks nobody writes)."""
+    monkeypatch.setenv("OEQ_AMD_TP_ROW_WAVES", str(waves))
+    prob, _ = common.channelwise(irreps)
+    g = UVUDirectGenerator(prob, "tp")
+    assert g.row_waves == waves and all(g.row_items())
+    assert g.plan()[0][0]["num_threads"] == 64 * waves
+    _tp(UVUDirectGenerator, irreps, 3, 5)
+
+
 def test_direct_tp_record_stores_only():
     _tp(UVUDirectGenerator, common.NEQUIP, 3, 3, vector_stores=False)
 
