@@ -10,19 +10,19 @@ openequivariance/templates/wmm.cuh:1-88 called from loop_unroll_tp.cuh:74-78, :1
 
 Tiling (lane = 16 * g + c, g = lane / 16, c = lane % 16; a batch tile is 16 rows):
 
-* forward, one wavefront per tile:  A[i=c][k=g] = T[b=c, u=4s+g] (VALU),  B[k=g][j=c] = W[u=4s+g][w]
-  from a pre-packed copy of W, accumulators = the 16 x mul_out tile of one output block; each lane
+* forward, one wavefront per (tile, output block):  A[i=c][k=g] = T[b=c, u] (VALU),  B[k=g][j=c] = W[u][w]
+  from a pre-packed copy of W, accumulators = the 16 x mul_out tile of the output block; each lane
   ends up with contiguous runs of Z, so Z is stored with vector stores straight from registers.
 * backward dX/dY, four wavefronts per tile (one 16-channel u-subtile each):
-  dT^T[u, b] = sum_w W[u][w] dZ[b][w]:  A = W (pre-packed), B = dZ held in registers for the whole
-  output block, then the CG transpose on the VALU accumulates dX (registers) and dY.
-* backward dW, four wavefronts per workgroup, persistent over batch tiles:
+  dT^T[u, b] = sum_w W[u][w] dZ[b][w]:  A = W (pre-packed), B = the 16-row dZ tile, staged in LDS once per
+  workgroup when it fits; then the CG transpose on the VALU accumulates dX (registers) and dY.
+* backward dW, four or eight wavefronts per workgroup, persistent over batch tiles:
   dW[u, w] = sum_{b,k} T[b,u,k] dZ[b,w,k]:  A = T (VALU), B = dZ, accumulators = this wavefront's
-  u-subtile of every path; per-workgroup partial sums go to the workspace and a last kernel adds
+  u-subtile of the paths of one pass; per-workgroup partial sums go to the workspace and a last kernel adds
   them in workgroup order (reproducible; no floating-point atomics).
 
-Nothing is staged in LDS (only the 4-wave dY sum uses 2.3 KB): operands are per-lane records of
-the ``mul x irrep`` layout, loaded straight from global memory / L2.
+X records, packed weights and (forward, dW) dZ are per-lane records of the ``mul x irrep`` layout, loaded
+straight from global memory / L2.
 
 Scope of this generator: shared weights.  A second operand with several copies per irrep (mul(in2) > 1)
 is handled as one contraction over u per copy v, with the slice W[:, v, :] of the weights; the
@@ -409,7 +409,7 @@ class UVWGenerator:
             E(f"const T y{f} = Y[rowA * {self.D2} + {f}];")
         # One work item = (batch tile, output block): blockIdx.y walks the output blocks from the most
         # to the least expensive, so the dispatcher fills the tail of the launch with the cheap ones
-        # (whole tiles per wavefront leave a third of the machine idle in the last round).
+        # (whole tiles per wavefront leave a third of the machine idle while the last ones finish).
         return self._forward_items(E, lambda slot: f"slot == {slot}")
 
     def _forward_lds_head(self, E: Emitter):
