@@ -165,7 +165,24 @@ class UVWGenerator:
             step = _ceil(nt_all, parts)
             for lo in range(0, nt_all, step):
                 self.fwd_order.append((o, lo, min(nt_all, lo + step)))
-        self.fwd_order.sort(key=lambda it: -cost(it[0]) * (it[2] - it[1]) / _ceil(it[0].mul, 16))
+        seg_cost = lambda it: cost(it[0]) * (it[2] - it[1]) / _ceil(it[0].mul, 16)
+        self.fwd_order.sort(key=lambda it: -seg_cost(it))
+        # Work items of a tile: one segment each.  OEQ_AMD_UVW_FWD_ITEMS packs the segments (longest first, into
+        # the lightest item) into that many items per tile (-1: as many as the total work holds copies of the
+        # largest segment), a wavefront then runs the segments of its item one after the other.  Measured on
+        # 64x0e+64x1o+64x2e, [l=2], [l=1, l=0] (work 20 : 15) against three items (20 : 12 : 3): fp32 353 vs
+        # 350 us, fp64 670 vs 604 us, so the segments stay separate.
+        costs = [seg_cost(it) for it in self.fwd_order]
+        nitems = int(os.environ.get("OEQ_AMD_UVW_FWD_ITEMS", "0"))
+        if nitems < 0:
+            nitems = max(1, -(-int(sum(costs)) // max(1, int(max(costs))))) if max(costs) > 0 else 1
+        if nitems == 0 or nitems >= len(self.fwd_order):
+            self.fwd_items = [[i] for i in range(len(self.fwd_order))]
+        else:
+            bins = [[] for _ in range(nitems)]
+            for i in range(len(self.fwd_order)):
+                min(bins, key=lambda b: sum(costs[j] for j in b)).append(i)
+            self.fwd_items = sorted([b for b in bins if b], key=lambda b: -sum(costs[j] for j in b))
         # dW kernel: output blocks split into two groups of similar MFMA work
         # (f64 accumulators are twice as wide: one group, four wavefronts, the whole register file)
         work = {o: sum(p.o.D * p.NTW * p.NTU for p in self.paths if p.o.idx == o) for o in self.used_out}
@@ -184,7 +201,7 @@ class UVWGenerator:
         mode = os.environ.get("OEQ_AMD_UVW_FWD_LDS", self.FWD_LDS_DEFAULT)
         fits = 16 * self.fwd_xrs * self.itemsize <= self.FWD_LDS_MAX_BYTES
         self.fwd_lds = (mode == "1") or (mode == "auto" and fits)
-        self.fwd_waves = min(len(self.fwd_order), 8) if self.fwd_lds else 1
+        self.fwd_waves = min(len(self.fwd_items), 8) if self.fwd_lds else 1
         # packed weight copies in the workspace
         pos = 0
         for p in self.paths:
@@ -379,7 +396,7 @@ class UVWGenerator:
     # =============================================================== forward
     def forward_body(self) -> str:
         E = Emitter()
-        NO = len(self.fwd_order)
+        NO = len(self.fwd_items)
         if self.fwd_lds:
             return self._forward_items(E, self._forward_lds_head(E))
         E("const int lane = threadIdx.x, c = lane & 15, g = lane >> 4;")
@@ -455,17 +472,27 @@ class UVWGenerator:
         return lambda slot: f"wave == {slot % NWV}"
 
     def _forward_items(self, E: Emitter, select) -> str:
-        for slot, (o, nt_lo, nt_hi) in enumerate(self.fwd_order):
+        for slot, item in enumerate(self.fwd_items):
+            E(f"if ({select(slot)}) {{")
+            E.level += 1
+            for i in item:
+                self._forward_segment(E, *self.fwd_order[i])
+            E.level -= 1
+            E("}")
+        return E.text()
+
+    def _forward_segment(self, E: Emitter, o: Block, nt_lo: int, nt_hi: int) -> None:
+        if True:
             NT = _ceil(o.mul, 16)
             NTS = range(nt_lo, nt_hi)
-            E(f"if ({select(slot)}) {{ // output block {o.idx}: {o.mul}x l={o.l}, w tiles {nt_lo} .. {nt_hi - 1} of {NT}")
+            E(f"{{ // output block {o.idx}: {o.mul}x l={o.l}, w tiles {nt_lo} .. {nt_hi - 1} of {NT}")
             E.level += 1
             if o.idx not in self.used_out:
                 for r in range(4):
                     E(f"{{ const u64 row = row0 + {self.row(r)}; if (row < n) for (int q = c; q < {o.dim}; q += 16) Z[row * {self.D3} + {o.off} + q] = (T)0; }}")
                 E.level -= 1
                 E("}")
-                continue
+                return
             for k in range(o.D):
                 for nt in NTS:
                     E(f"V4 acc{k}_{nt} = {{0, 0, 0, 0}};")
@@ -551,7 +578,6 @@ class UVWGenerator:
                 E("  } }")
             E.level -= 1
             E("}")
-        return E.text()
 
     # ====================================================== backward: dX, dY
     def backward_body(self) -> str:
@@ -995,7 +1021,7 @@ class UVWGenerator:
         FIXED, ROW = 0, 1
         fwd = [dict(kernel="prep_forward", num_threads=256, grid_kind=FIXED, num_blocks=self.prep_blocks),
                dict(kernel="forward", num_threads=64 * self.fwd_waves, grid_kind=ROW, work_per_block=16,
-                    grid_y=1 if self.fwd_lds else len(self.fwd_order))]
+                    grid_y=1 if self.fwd_lds else len(self.fwd_items))]
         bwd = [dict(kernel="prep_backward", num_threads=256, grid_kind=FIXED, num_blocks=self.prep_blocks),
                dict(kernel="backward", num_threads=256, grid_kind=ROW, work_per_block=16),
                dict(kernel="backward_dw", num_threads=256 * self.dw_groups, grid_kind=FIXED,

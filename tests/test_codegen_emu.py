@@ -243,7 +243,7 @@ def test_uvw_forward_with_the_x_tile_in_lds(dtype, a, n, monkeypatch):
     monkeypatch.setenv("OEQ_AMD_UVW_FWD_LDS", "1")
     prob, oprob = common.fully_connected(a, shared=True, dtype=dtype)
     g = UVWGenerator(prob)
-    assert g.fwd_lds and g.fwd_waves == len(g.fwd_order)
+    assert g.fwd_lds and g.fwd_waves == len(g.fwd_items)
     X, Y, We, _ = common.tp_inputs(prob, n, 11, dtype, w_scale=0.3)
     W = ow.e3nn_to_oeq(oprob, We)
     fwd, _, ws = g.plan()
