@@ -161,13 +161,23 @@ class UVUDetGenerator(UVUDirectGenerator):
         interleaved sub-lists of the node's edges (edge beg + it*R + sub) and their partial sums are
         combined in a fixed order at the end, which shortens the serial edge loop R-fold."""
         R = self.R
-        E("const int c = blockIdx.y; (void)c;")
+        if self.NCH > 1 and os.environ.get("OEQ_AMD_DET_CHUNK_MINOR", "0") == "1":
+            # A/B switch: the chunks of a node get consecutive workgroup ids and run at the same time.  Measured
+            # slower (256 channels: forward 2.58 -> 2.75 ms, backward 7.49 -> 9.72 ms): with the launch ordered
+            # chunk by chunk, the wavefronts in flight gather from one chunk's share of X / dZ only, a quarter
+            # of the tensor, which the 256 MB Infinity Cache can hold.
+            E("const u64 lin_ = blockIdx.x + (u64)blockIdx.y * gridDim.x;")
+            E(f"const int c = (int)(lin_ % {self.NCH}); (void)c;")
+            E(f"const u64 bx_ = lin_ / {self.NCH};")
+        else:
+            E("const int c = blockIdx.y; (void)c;")
+            E("const u64 bx_ = blockIdx.x;")
         E(f"const int u = c * {self.P} + ul;")
         if order:
-            E(f"const i64 nd_ = blockIdx.x < node_count ? {order}[blockIdx.x] : -1;")
+            E(f"const i64 nd_ = bx_ < node_count ? {order}[bx_] : -1;")
             E("const u64 node = nd_ >= 0 ? (u64)nd_ : node_count;")
         else:
-            E("const u64 node = blockIdx.x;")
+            E("const u64 node = bx_;")
         E("const bool nv = node < node_count;")
         E(f"const i64* __restrict__ ptr = (const i64*)ws + {ptr_off};")
         E("i64 beg = 0, end = 0;")
@@ -233,7 +243,7 @@ class UVUDetGenerator(UVUDirectGenerator):
         preparation kernels leave one flag per 256 edges; the first workgroup of every (chunk, group)
         launch row ORs them and, only if some edge is flagged, walks the edge list and writes zeros into
         the rows of those edges: dW and dY (or this launch's dY partial slot)."""
-        E("if (blockIdx.x == 0) {")
+        E("if (bx_ == 0) {")
         E.level += 1
         E("const int* __restrict__ bad_ = (const int*)((const char*)ws + FLAGS_OFF);")
         E("int any_ = 0;")
