@@ -150,6 +150,14 @@ def test_conv_fp64(cuda):
     _run(prob, oprob, 64, 900, 36, False, dtype=np.float64, sh_lmax=2)
 
 
+@pytest.mark.parametrize("deterministic", [False, True])
+def test_conv_fp64_ragged_chunks(cuda, deterministic):
+    """fp64 with multiplicities above one wavefront (two chunks, the second partly filled) and below it."""
+    irreps = ("70x0e+100x1o+5x2e", "1x0e+1x1o+1x2e", "70x0e+100x1o+70x1o+5x2e+100x2e")
+    prob, oprob = common.channelwise(irreps, dtype=np.float64)
+    _run(prob, oprob, 30, 500, 37, deterministic, dtype=np.float64, sh_lmax=2)
+
+
 def test_isolated_nodes_and_asymmetric_graph(cuda):
     """Nodes without incoming or outgoing edges get zero rows; the graph is not symmetric."""
     prob, oprob = common.channelwise(common.NEQUIP)
