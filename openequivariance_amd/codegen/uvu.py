@@ -369,25 +369,16 @@ class UVUGenerator:
         accumulates in registers, and the dY sums of this v (over the lanes of the row) are added to the
         row's LDS accumulator by its writer lane."""
         E(f"// path {p.t}: l = {p.a.l} x {p.b.l} -> {p.o.l}, {p.mv} copies of the second operand walked at run time")
+        E("{")
+        self._emit_cg_products(E, p)
         E(f"for (int v = 0; v < {p.mv}; ++v) {{")
         E.level += 1
         E(f"const T wv = {self.looped_weight(p, wptr)};")
         E(f"const T* __restrict__ yv = Yr + {p.b.off} + v * {p.b.D};")
         js = sorted({j for (_, j) in p.pairs})
-        is_ = sorted({i for (i, _) in p.pairs})
         for j in js:
-            E(f"const T yv{j} = yv[{j}]; const T wy{j} = wv * yv{j}; T dyv{j} = (T)0;")
-        for i in is_:
-            E(f"const T wx{i} = wv * x{p.a.idx}_{i};")
-        E("T dw = (T)0;")
-        for (i, j), ks in p.ordered_pairs():
-            E("{")
-            for n_, (k, val) in enumerate(ks):
-                E(f"  T s = {self.lit(val)} * g{k};" if n_ == 0 else f"  s = oeq_fma({self.lit(val)}, g{k}, s);")
-            E(f"  dw = oeq_fma(s, x{p.a.idx}_{i} * yv{j}, dw);")
-            E(f"  dx{p.a.idx}_{i} = oeq_fma(s, wy{j}, dx{p.a.idx}_{i});")
-            E(f"  dyv{j} = oeq_fma(s, wx{i}, dyv{j});")
-            E("}")
+            E(f"const T yv{j} = yv[{j}]; T dyv{j} = (T)0;")
+        self._emit_backward_pairs(E, p, "wv", lambda j: f"yv{j}", lambda j: f"dyv{j}")
         dw_sink(E, p, "v", "dw")
         for j in js:
             if self.P == WAVE:
@@ -398,6 +389,7 @@ class UVUGenerator:
         E(f"if ({writer}) {{ T* __restrict__ a_ = ylds + sub * {self.NLY} + {self.looped_y[p.b.off]} + v * {p.b.D}; "
           + " ".join(f"a_[{j}] += dyv{j};" for j in js) + " }")
         E.level -= 1
+        E("}")
         E("}")
 
     def emit_looped_dy_begin(self, E: Emitter) -> None:
@@ -416,36 +408,67 @@ class UVUGenerator:
     def emit_backward_block(self, E: Emitter, o: Block, wptr: str, dw_sink) -> None:
         """Given g_k = dZ[o][u, k] (registers g0..), update dx{a}_{i}, dy{f} and hand every
         dW value to ``dw_sink(E, path, v, expr)``.  Formulas: loop_unroll_tp.cuh:167-174 of the
-        reference, regrouped per (i, j) pair: s = sum_k c_ijk g_k."""
+        reference, regrouped so that every (i, j) pair costs two multiply-adds beyond its
+        s_ij = sum_k c_ijk g_k:  t_i = sum_j s_ij y_j,  dy_j += s_ij (w x_i),  and per path
+        dw = sum_i x_i t_i,  dx_i += w t_i.  A product c g_k that several pairs share (same k, same
+        |c|) is computed once; its sign rides on the multiply-add."""
         for p in self.paths_into(o.idx):
             if p.looped:
                 self.emit_backward_looped(E, p, wptr, dw_sink)
                 continue
             E(f"{{ // path {p.t}: l = {p.a.l} x {p.b.l} -> {p.o.l}")
             self.emit_weights(E, p, wptr)
+            self._emit_cg_products(E, p)
             for v in range(p.mv):
                 ya = lambda j: f"y{p.b.off + v * p.b.D + j}"
-                E(f"{{ T dw = (T)0;")
-                js = sorted({j for (_, j) in p.pairs})
-                is_ = sorted({i for (i, _) in p.pairs})
-                for j in js:
-                    E(f"  const T wy{j} = w{p.t}_{v} * {ya(j)};")
-                for i in is_:
-                    E(f"  const T wx{i} = w{p.t}_{v} * x{p.a.idx}_{i};")
-                for (i, j), ks in p.ordered_pairs():
-                    E("  {")
-                    for n_, (k, val) in enumerate(ks):
-                        if n_ == 0:
-                            E(f"    T s = {self.lit(val)} * g{k};")
-                        else:
-                            E(f"    s = oeq_fma({self.lit(val)}, g{k}, s);")
-                    E(f"    dw = oeq_fma(s, x{p.a.idx}_{i} * {ya(j)}, dw);")
-                    E(f"    dx{p.a.idx}_{i} = oeq_fma(s, wy{j}, dx{p.a.idx}_{i});")
-                    E(f"    dy{p.b.off + v * p.b.D + j} = oeq_fma(s, wx{i}, dy{p.b.off + v * p.b.D + j});")
-                    E("  }")
+                E("{")
+                self._emit_backward_pairs(E, p, f"w{p.t}_{v}", ya, lambda j: f"dy{p.b.off + v * p.b.D + j}")
                 dw_sink(E, p, v, "dw")
                 E("}")
             E("}")
+
+    def _cg_key(self, k: int, val: float):
+        return (k, float(np.float64(abs(val)).round(12)))
+
+    def _emit_cg_products(self, E: Emitter, p: Path) -> None:
+        """c * g_k for the pairs of ``p`` with a single output component, once per distinct (k, |c|)."""
+        self._cg_names = {}
+        for (i, j), ks in p.ordered_pairs():
+            if len(ks) == 1:
+                key = self._cg_key(*ks[0])
+                if key not in self._cg_names:
+                    self._cg_names[key] = f"cg{len(self._cg_names)}"
+                    E(f"  const T {self._cg_names[key]} = {self.lit(abs(ks[0][1]))} * g{ks[0][0]};")
+
+    def _emit_backward_pairs(self, E: Emitter, p: Path, w: str, ya, dya) -> None:
+        """The (i, j) pairs of one copy of the second operand: declares and fills ``dw``, updates dx and dy."""
+        is_ = sorted({i for (i, _) in p.pairs})
+        for i in is_:
+            E(f"  const T wx{i} = {w} * x{p.a.idx}_{i};")
+        started = set()
+        E("  T " + ", ".join(f"t{i}" for i in is_) + ";")
+        for (i, j), ks in p.ordered_pairs():
+            if len(ks) == 1:
+                neg = "-" if ks[0][1] < 0 else ""
+                s = f"{neg}{self._cg_names[self._cg_key(*ks[0])]}"
+            else:
+                E("  {")
+                for n_, (k, val) in enumerate(ks):
+                    E(f"    T s = {self.lit(val)} * g{k};" if n_ == 0 else f"    s = oeq_fma({self.lit(val)}, g{k}, s);")
+                s = "s"
+            if i in started:
+                E(f"    t{i} = oeq_fma({s}, {ya(j)}, t{i});")
+            else:
+                E(f"    t{i} = {s} * {ya(j)};")
+                started.add(i)
+            E(f"    {dya(j)} = oeq_fma({s}, wx{i}, {dya(j)});")
+            if len(ks) > 1:
+                E("  }")
+        E(f"  T dw = x{p.a.idx}_{is_[0]} * t{is_[0]};")
+        for i in is_[1:]:
+            E(f"  dw = oeq_fma(x{p.a.idx}_{i}, t{i}, dw);")
+        for i in is_:
+            E(f"  dx{p.a.idx}_{i} = oeq_fma({w}, t{i}, dx{p.a.idx}_{i});")
 
     # --------------------------------------------------------------- LDS slots
     def emit_slot_write(self, E: Emitter, blk: Block, name: str, act: str) -> None:

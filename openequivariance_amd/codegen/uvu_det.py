@@ -115,6 +115,9 @@ class UVUDetGenerator(UVUDirectGenerator):
         self.lds_backward = fits and env != "0"
         if self.lds_backward:
             self.waves_per_eu = min(3, stage_waves)
+        elif self.prefetch_backward:
+            # two register sets: hold the allocation to what two wavefronts per SIMD leave each (256 registers)
+            self.waves_per_eu = 2
         # the forward likewise when the multiplicity fits one chunk: few wavefronts per node, so the
         # registers saved buy a fifth wavefront per SIMD (with several chunks per node it measured 1 % slower)
         fwd_words = self._forward_slabs()[1]
