@@ -28,7 +28,6 @@ schedule is new):
 """
 from __future__ import annotations
 
-import os
 from dataclasses import dataclass, field
 from typing import Dict, List, Tuple
 
@@ -194,18 +193,10 @@ class UVUGenerator:
     def lit(self, v: float) -> str:
         return literal(v, self.T)
 
-    row_waves = 1       # wavefronts per workgroup of the batch kernels (the register-direct schedule may use more)
-
-    def forward_attr(self) -> str:
-        """Extra kernel attributes of the batch forward kernel: an upper bound on the wavefronts per SIMD."""
-        w = int(os.environ.get("OEQ_AMD_TP_FWD_OCC", str(getattr(self, "fwd_waves_per_eu", 0))))
-        return f" __attribute__((amdgpu_waves_per_eu({w}, {w})))" if w else ""
-
     def backward_attr(self) -> str:
-        """Extra kernel attributes of the backward kernel (occupancy hint)."""
-        cap = int(os.environ.get("OEQ_AMD_TP_BWD_OCC", "0")) if self.kind == "tp" else 0
-        if cap:
-            return f" __attribute__((amdgpu_waves_per_eu({cap}, {cap})))"
+        """Extra kernel attributes of the backward kernel: the wavefronts per SIMD the register allocation
+        must leave room for, when the schedule sets one (capping the wavefronts per SIMD of the batch
+        kernels at 2, 3 or 4 helped plain copies of their shape by up to 5 % and the kernels not at all)."""
         w = getattr(self, "waves_per_eu", 0)
         return f" __attribute__((amdgpu_waves_per_eu({w})))" if w else ""
 

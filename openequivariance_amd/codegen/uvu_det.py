@@ -27,8 +27,8 @@ kernel reads both at the unpermuted position: templates/loop_unroll_conv_det.cuh
 from __future__ import annotations
 
 import contextlib
-import os
 
+from .. import tunables
 from ..problem import TPProblem
 from .common import Emitter, WAVE
 from .uvu_direct import UVUDirectGenerator
@@ -40,7 +40,7 @@ class UVUDetGenerator(UVUDirectGenerator):
 
     def __init__(self, problem: TPProblem, prefetch_backward=None, vector_stores: bool = True,
                  forward_perm: bool = False, backward_perm: bool = False, idx_ctype: str = "i64",
-                 allow_split: bool = True):
+                 allow_split: bool = True, lds=None):
         super().__init__(problem, "conv_det", vector_stores=vector_stores)
         self.idx_ctype = idx_ctype
         # True: the forward walks the receiver-grouped edge order listed in the workspace (built on
@@ -53,8 +53,8 @@ class UVUDetGenerator(UVUDirectGenerator):
         # the backward launches the nodes in descending order of their edge count (order_backward writes
         # the node list behind the pointers): with two launch rounds of wavefronts the long nodes then
         # run first and the short ones fill the tail
-        self.ordered_backward = os.environ.get("OEQ_AMD_DET_ORDER", "1") != "0"
-        extra = " + node_count" if self.ordered_backward else ""
+        self.ordered_backward = True
+        extra = " + node_count"
         if backward_perm:
             # behind the forward's grouping (pointers | cursors | position list), so that both stay valid
             # side by side and a graph prepared once serves forward and backward calls alike
@@ -78,9 +78,9 @@ class UVUDetGenerator(UVUDirectGenerator):
                     + len({p.b.off + v * p.b.D + j for p in ps for v in range(p.mv) for (_, j) in p.pairs}))
         words = words_of(self.used_out)
         H = 1
-        split_env = os.environ.get("OEQ_AMD_DET_SPLIT", "")           # "0": never; a number: threshold for A/B runs
-        limit = int(split_env) if split_env.isdigit() and split_env != "0" else self.SPLIT_WORDS
-        if words > limit and split_env != "0" and allow_split:
+        split = tunables.current.det_split                      # 0: never; a number: threshold for A/B runs
+        limit = split if split else self.SPLIT_WORDS
+        if words > limit and split != 0 and allow_split:
             H = min(len(self.used_out), -(-words // 64))
         self.out_groups = [[] for _ in range(H)]
         for oi in sorted(self.used_out, key=lambda i: -(self.out[i].D + len(self.paths_into(i)))):
@@ -95,24 +95,25 @@ class UVUDetGenerator(UVUDirectGenerator):
         words = max(words_of(g_) for g_ in self.out_groups)
         # fetch the next edge's operands while the current edge is being computed; pays when the
         # per-edge register footprint is small enough to keep several wavefronts per SIMD
-        env = os.environ.get("OEQ_AMD_DET_PREFETCH")          # "0" / "1": tuning override for A/B runs
-        if prefetch_backward is None and env in ("0", "1"):
-            prefetch_backward = (env == "1")
+        if prefetch_backward is None:
+            prefetch_backward = tunables.current.det_prefetch
         self.prefetch_backward = (words <= 80) if prefetch_backward is None else prefetch_backward
-        self.nontemporal = os.environ.get("OEQ_AMD_DET_NT", "1") == "1"   # streaming hint on W / Y / dW / dY
+        # W / Y / dW / dY are touched once: the streaming hint keeps them from evicting the gathered rows
+        # (256 channels, without the hint: forward 2.58 -> 2.73 ms, backward 7.68 -> 8.91 ms)
+        self.nontemporal = True
         # backward operands of the next edge travel global -> LDS without passing through registers
         # (LDS-DMA), which leaves room for a third wavefront per SIMD; see emit_staged_loop
         def stage_words_of(outs):
             return WAVE * (sum(self.dma_stride(w) for i in outs for _, w in self.dma_pieces(self.out[i].D))
                            + sum(p.mv for p in self.paths if p.o.idx in outs) + 1)
         self.stage_words = max(stage_words_of(g_) for g_ in self.out_groups)      # of the largest group
-        env = os.environ.get("OEQ_AMD_DET_LDS")
+        lds = tunables.current.det_lds if lds is None else lds
         stage_waves = (160 * 1024) // (4 * self.stage_words * 4)        # wavefronts per SIMD the stage leaves room for
         # one chunk per node: also at two wavefronts per SIMD (the register pipeline then has one); chunked
         # problems only when three fit (config 5, two: 1 % slower than the register pipeline)
         small = self.NCH == 1 and H == 1
         fits = self.T == "float" and self.P >= self.D2 and (stage_waves >= 3 or (small and stage_waves >= 2))
-        self.lds_backward = fits and env != "0"
+        self.lds_backward = fits and lds is not False
         if self.lds_backward:
             self.waves_per_eu = min(3, stage_waves)
         elif self.prefetch_backward:
@@ -121,7 +122,7 @@ class UVUDetGenerator(UVUDirectGenerator):
         # the forward likewise when the multiplicity fits one chunk: few wavefronts per node, so the
         # registers saved buy a fifth wavefront per SIMD (with several chunks per node it measured 1 % slower)
         fwd_words = self._forward_slabs()[1]
-        self.lds_forward = (self.T == "float" and self.P >= self.D2 and self.NCH == 1 and env != "0"
+        self.lds_forward = (self.T == "float" and self.P >= self.D2 and self.NCH == 1 and lds is not False
                             and 16 * (fwd_words + self.lds_elems) * 4 <= 160 * 1024)
         self.uniform_rows = False          # validity is per lane (edge lists differ between sub-rows)
         self.chunk_in_grid = True
@@ -164,17 +165,12 @@ class UVUDetGenerator(UVUDirectGenerator):
         interleaved sub-lists of the node's edges (edge beg + it*R + sub) and their partial sums are
         combined in a fixed order at the end, which shortens the serial edge loop R-fold."""
         R = self.R
-        if self.NCH > 1 and os.environ.get("OEQ_AMD_DET_CHUNK_MINOR", "0") == "1":
-            # A/B switch: the chunks of a node get consecutive workgroup ids and run at the same time.  Measured
-            # slower (256 channels: forward 2.58 -> 2.75 ms, backward 7.49 -> 9.72 ms): with the launch ordered
-            # chunk by chunk, the wavefronts in flight gather from one chunk's share of X / dZ only, a quarter
-            # of the tensor, which the 256 MB Infinity Cache can hold.
-            E("const u64 lin_ = blockIdx.x + (u64)blockIdx.y * gridDim.x;")
-            E(f"const int c = (int)(lin_ % {self.NCH}); (void)c;")
-            E(f"const u64 bx_ = lin_ / {self.NCH};")
-        else:
-            E("const int c = blockIdx.y; (void)c;")
-            E("const u64 bx_ = blockIdx.x;")
+        # The launch is ordered chunk by chunk (blockIdx.y): the wavefronts in flight then gather from one
+        # chunk's share of X / dZ, a fraction of the tensor that the 256 MB Infinity Cache can hold.  Giving
+        # the chunks of a node consecutive workgroup ids instead measured slower (256 channels: forward
+        # 2.58 -> 2.75 ms, backward 7.49 -> 9.72 ms).
+        E("const int c = blockIdx.y; (void)c;")
+        E("const u64 bx_ = blockIdx.x;")
         E(f"const int u = c * {self.P} + ul;")
         if order:
             E(f"const i64 nd_ = bx_ < node_count ? {order}[bx_] : -1;")

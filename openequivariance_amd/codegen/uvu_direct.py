@@ -22,28 +22,25 @@ vector stores or as coalesced atomics; loads stay register-direct.
 """
 from __future__ import annotations
 
-import os
-
+from .. import tunables
 from ..problem import TPProblem
 from .common import WAVE, Emitter
 from .uvu import Block, Path, UVUGenerator
 
 
 class UVUDirectGenerator(UVUGenerator):
-    ROW_WAVES = 1          # wavefronts that share one row of the batch product (1: one wavefront per row)
-
     def __init__(self, problem: TPProblem, kind: str = "tp", waves_per_eu: int = 0, vector_stores: bool = True):
         super().__init__(problem, kind)
         if (kind == "conv_det" and not getattr(self, "_allow_det", False)) or self.shared:
             raise NotImplementedError("direct schedule: batch product with per-row weights and atomic convolution")
-        self.waves_per_eu = waves_per_eu or int(os.environ.get("OEQ_AMD_WAVES_PER_EU", "0"))
+        self.waves_per_eu = waves_per_eu
         # False: outputs are written with dword-aligned record stores only (for callers whose
         # output tensor is not 16-byte aligned)
         self.vector_stores = vector_stores
-        # words per vector store of the LDS-slot route (16 bytes; OEQ_AMD_TP_STORE_BYTES=8 for A/B runs)
-        self.store_bytes = int(os.environ.get("OEQ_AMD_TP_STORE_BYTES", "16")) if kind == "tp" else 16
-        self.VW = max(1, self.store_bytes // self.itemsize)
-        self.VTYPE = "VT" if self.VW * self.itemsize == 16 else "VT8"
+        # words per 16-byte vector store of the LDS-slot route (8-byte stores measured a tie on the
+        # 128-channel MACE problem, 0.463 against 0.458 ms; 4-byte stores 0.77 ms)
+        self.VW = max(1, 16 // self.itemsize)
+        self.VTYPE = "VT"
         stage = [WAVE * b.D for b in list(self.out) + list(self.in1) if b.D > 1 and b.dim]
         self.lds_elems = max(stage) if stage else 0
         self.ZB = 0
@@ -51,41 +48,27 @@ class UVUDirectGenerator(UVUGenerator):
         # Batch product: every tensor is read or written exactly once.  The backward's loads and stores
         # carry the non-temporal hint (measured on the 128-channel MACE problem, warm and with flushed
         # caches alike: 0.63 -> 0.56 ms); on the forward the hint measured slower (stores: 0.46 -> 0.52 ms
-        # with flushed caches), so it keeps plain accesses.  OEQ_AMD_TP_NT lists the accesses that get the
-        # hint (fl, fs, bl, bs = forward / backward loads / stores) for A/B runs.  Writing the backward's dX
-        # through the LDS slot as full-line vector stores (OEQ_AMD_TP_DX_LDS=1) measured a tie and costs
-        # 37 registers, so dX keeps its record stores.
-        self._nt_modes = set(os.environ.get("OEQ_AMD_TP_NT", "bl,bs").split(",")) if kind == "tp" else set()
+        # with flushed caches), so it keeps plain accesses.  ``tunables.tp_nontemporal`` lists the accesses
+        # that get the hint (fl, fs, bl, bs = forward / backward loads / stores).  Writing the backward's dX
+        # through the LDS slot as full-line vector stores measured a tie (0.626 against 0.632 ms) and costs
+        # 37 registers, so dX keeps its record stores; dealing a row to four wavefronts of one workgroup
+        # measured no gain either (forward 0.456 ms, backward 0.59 ms).
+        self._nt_modes = set(tunables.current.tp_nontemporal.split(",")) if kind == "tp" else set()
         self.nt_load = self.nt_store = False
-        self.dx_via_lds = (kind == "tp") and os.environ.get("OEQ_AMD_TP_DX_LDS", "0") == "1"
         # one row per wavefront: the row index is wave-uniform and an out-of-range wavefront exits
         self.uniform_rows = (self.R == 1)
         self._cur_c = None
-        # Batch product with one row per wavefront: the row's work can be dealt to several wavefronts of one
-        # workgroup (contiguous ranges of the output row each), see split_forward_body
-        want = int(os.environ.get("OEQ_AMD_TP_ROW_WAVES", str(self.ROW_WAVES)))
-        items = self._row_items_all()
-        ok = (kind == "tp" and self.R == 1 and not self.dx_via_lds and not any(p.looped for p in self.paths)
-              and len(items) >= want > 1)
-        self.row_waves = want if ok else 1
 
     def describe(self) -> str:
         return super().describe().replace(f"lds={0}B", "lds=0B") + " direct"
 
     # ------------------------------------------------------------------ pieces
-    def emit_lane_direct(self, E: Emitter, lds: bool = False, waves: int = 1) -> None:
-        if waves > 1:
-            E("const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;")
-        else:
-            E("const int lane = threadIdx.x;")
+    def emit_lane_direct(self, E: Emitter, lds: bool = False) -> None:
+        E("const int lane = threadIdx.x;")
         E(f"const int sub = lane >> {self.LOGP};")
         E(f"const int ul = lane & {self.P - 1};")
         if lds and self.lds_elems:
-            if waves > 1:
-                E(f"__shared__ __attribute__((aligned(16))) T lds_all[{waves * self.lds_elems}];")
-                E(f"T* __restrict__ lds = lds_all + wave * {self.lds_elems};")
-            else:
-                E(f"__shared__ __attribute__((aligned(16))) T lds[{self.lds_elems}];")
+            E(f"__shared__ __attribute__((aligned(16))) T lds[{self.lds_elems}];")
 
     # ---- stores through an LDS slot ---------------------------------------------
     def dense(self, blk: Block) -> int:
@@ -326,7 +309,7 @@ class UVUDirectGenerator(UVUGenerator):
         E = Emitter()
         atomic = (self.kind == "conv_atomic")
         self.nt_load, self.nt_store = "bl" in self._nt_modes, "bs" in self._nt_modes
-        self.emit_lane_direct(E, lds=atomic or self.dx_via_lds)
+        self.emit_lane_direct(E, lds=atomic)
         xrow, zrow, srow = self._rows(E, backward=True)
         E(f"T* __restrict__ Wgr = Wg + {srow} * {self.WN};")
         self.emit_y_load_direct(E)
@@ -368,7 +351,7 @@ class UVUDirectGenerator(UVUGenerator):
                     continue
                 if a.idx in self.used_in1:
                     self.emit_block_store(E, a, [f"dx{a.idx}_{m}" for m in range(a.D)], "Xg", self.D1, xrow,
-                                          self.xrow_of, "atomic" if atomic else "store", via_lds=atomic or self.dx_via_lds)
+                                          self.xrow_of, "atomic" if atomic else "store", via_lds=atomic)
                 elif not atomic:
                     self.emit_record_store(E, ["(T)0"] * a.D, f"Xg + (u64){xrow} * {self.D1} + {a.off} + u * {a.D}",
                                            self.act(a))
@@ -415,168 +398,11 @@ class UVUDirectGenerator(UVUGenerator):
             E("}")
         return E.text()
 
-    # ================================================== one row shared by several wavefronts
-    def _row_items_all(self):
-        """(chunk, output block) pieces of one output row in address order."""
-        return [(c, o) for o in self.out if o.dim for c in range(self.NCH) if c * self.P < o.mul]
-
-    def row_items(self):
-        """The pieces dealt to the row's wavefronts: contiguous ranges of the row, cut where the running
-        cost (record words + weights of the paths into the block) crosses the next equal share."""
-        items = self._row_items_all()
-        cost = [o.D + len(self.paths_into(o.idx)) for _, o in items]
-        total, out, acc, k = sum(cost), [[] for _ in range(self.row_waves)], 0, 0
-        for it, w in zip(items, cost):
-            while k < self.row_waves - 1 and acc + w / 2 > total * (k + 1) / self.row_waves and out[k]:
-                k += 1
-            out[k].append(it)
-            acc += w
-        return out
-
-    def split_forward_body(self) -> str:
-        """Batch forward with the row dealt to ``row_waves`` wavefronts of one workgroup: every wavefront
-        loads the X records and weights its pieces need, computes them and writes its contiguous part of
-        the Z row.  Measured on MI355X with plain copy kernels of the same shape: the memory system
-        sustains more when the rows in flight are fewer and each is moved by several wavefronts at once."""
-        E = Emitter()
-        self.nt_load, self.nt_store = "fl" in self._nt_modes, "fs" in self._nt_modes
-        self.emit_lane_direct(E, lds=True, waves=self.row_waves)
-        xrow, zrow, _ = self._rows(E)
-        self.emit_y_load_direct(E)
-        for w, items in enumerate(self.row_items()):
-            E(f"if (wave == {w}) {{")
-            E.level += 1
-            chunks = sorted({c for c, _ in items})
-            need = {c: ({p.a.idx for cc, o in items if cc == c for p in self.paths_into(o.idx)},
-                        {p.t for cc, o in items if cc == c for p in self.paths_into(o.idx)}) for c in chunks}
-            for c in chunks:
-                self.emit_x_preload(E, c, xrow, only=need[c][0])
-                self.emit_weight_preload(E, c, only=need[c][1])
-            for c, o in items:
-                self._cur_c = self._loop_c = c
-                E("{")
-                E.level += 1
-                E(f"const int c = {c}; (void)c;")
-                E(f"const int u = {c * self.P} + ul;")
-                if o.idx in self.used_out:
-                    self.emit_x_alias(E, c, only={p.a.idx for p in self.paths_into(o.idx)})
-                    self.emit_forward_block(E, o, "Wr")
-                    self.emit_block_store(E, o, [f"z{k}" for k in range(o.D)], "Z", self.D3, zrow, self.zrow_of,
-                                          "store", via_lds=True)
-                else:
-                    self.emit_record_store(E, ["(T)0"] * o.D, f"Z + (u64){zrow} * {self.D3} + {o.off} + u * {o.D}",
-                                           self.act(o))
-                E.level -= 1
-                E("}")
-            E.level -= 1
-            E("}")
-        return E.text()
-
-    def split_backward_body(self) -> str:
-        """Batch backward with the row dealt to ``row_waves`` wavefronts by output blocks (the same pieces as
-        the forward): every wavefront reads its part of the dZ row and the weights of its paths and writes
-        their dW; its contributions to dX and dY go to LDS and are added across the wavefronts in a fixed
-        order after one workgroup barrier, then stored coalesced."""
-        E = Emitter()
-        WPR, P = self.row_waves, self.P
-        self.nt_load, self.nt_store = "bl" in self._nt_modes, "bs" in self._nt_modes
-        self.emit_lane_direct(E, lds=False, waves=WPR)
-        xrow, zrow, srow = self._rows(E, backward=True)
-        E(f"T* __restrict__ Wgr = Wg + {srow} * {self.WN};")
-        E(f"__shared__ T dxp[{WPR * self.D1}];")
-        E(f"__shared__ T dyp[{WPR * self.D2}];")
-        self.emit_y_load_direct(E)
-        contrib = {}
-        for w, items in enumerate(self.row_items()):
-            E(f"if (wave == {w}) {{")
-            E.level += 1
-            mine = [(c, o) for c, o in items if o.idx in self.used_out]
-            ys = sorted({p.b.off + v * p.b.D + j for _, o in mine for p in self.paths_into(o.idx)
-                         for v in range(p.mv) for (_, j) in p.pairs})
-            for f in ys:
-                E(f"T dy{f} = (T)0;")
-            for c in sorted({c for c, _ in mine}):
-                outs = [o for cc, o in mine if cc == c]
-                paths = [p for o in outs for p in self.paths_into(o.idx)]
-                ins = sorted({p.a.idx for p in paths})
-                self._cur_c = self._loop_c = c
-                E("{")
-                E.level += 1
-                E(f"const int c = {c}; (void)c;")
-                E(f"const int u = {c * P} + ul;")
-                self.emit_x_preload(E, c, xrow, only=set(ins))
-                self.emit_weight_preload(E, c, only={p.t for p in paths})
-                for o in outs:
-                    self.emit_record_load(E, [f"G{o.idx}_{k}" for k in range(o.D)],
-                                          f"G + (u64){zrow} * {self.D3} + {o.off} + {self.uclamp(o, c)} * {o.D}",
-                                          self.act(o), zero=True)
-                self.emit_x_alias(E, c, only=set(ins))
-                for i in ins:
-                    for m in range(self.in1[i].D):
-                        E(f"T dx{i}_{m} = (T)0;")
-                for o in outs:
-                    E("{")
-                    E.level += 1
-                    for k in range(o.D):
-                        E(f"const T g{k} = G{o.idx}_{k};")
-
-                    def sink(E, p, v, expr):
-                        if self.nt_store:
-                            E(f"  if ({self.act(p.a)}) oeq_stnt(Wgr + {self.widx(p, 'u', v)}, {expr});")
-                        else:
-                            E(f"  if ({self.act(p.a)}) Wgr[{self.widx(p, 'u', v)}] = {expr};")
-                    self.emit_backward_block(E, o, "Wr", sink)
-                    E.level -= 1
-                    E("}")
-                for i in ins:
-                    a = self.in1[i]
-                    contrib.setdefault((i, c), []).append(w)
-                    E(f"if ({self.act(a)}) {{ T* __restrict__ d_ = dxp + {w * self.D1 + a.off} + u * {a.D}; "
-                      + " ".join(f"d_[{m}] = dx{i}_{m};" for m in range(a.D)) + " }")
-                E.level -= 1
-                E("}")
-            for f in ys:
-                E(f"dy{f} = oeq_wave_sum63(dy{f});")
-            E("if (lane == 63) { " + " ".join(f"dyp[{w * self.D2 + f}] = " + (f"dy{f};" if f in ys else "(T)0;")
-                                                for f in range(self.D2)) + " }")
-            E.level -= 1
-            E("}")
-        E("__syncthreads();")
-        # dX: the pieces (in1 block, chunk) in row order, each the sum of the wavefronts that computed a part of it
-        st = (lambda ptr, v: f"oeq_stnt({ptr}, {v});") if self.nt_store else (lambda ptr, v: f"*({ptr}) = {v};")
-        runs = []
-        for a in self.in1:
-            if a.dim == 0:
-                continue
-            for c in range(self.NCH):
-                cnt = max(0, min(P, a.mul - c * P)) * a.D
-                if cnt == 0:
-                    continue
-                ws_ = tuple(contrib.get((a.idx, c), ()))
-                beg = a.off + c * P * a.D
-                if runs and runs[-1][2] == ws_ and runs[-1][0] + runs[-1][1] == beg:
-                    runs[-1] = (runs[-1][0], runs[-1][1] + cnt, ws_)
-                else:
-                    runs.append((beg, cnt, ws_))
-        E(f"T* __restrict__ Xgr = Xg + (u64){xrow} * {self.D1};")
-        for beg, cnt, ws_ in runs:
-            val = " + ".join(f"dxp[{w * self.D1 + beg} + q]" for w in ws_) if ws_ else "(T)0"
-            E(f"for (int q = threadIdx.x; q < {cnt}; q += {64 * WPR}) {{ " + st(f"Xgr + {beg} + q", val) + " }")
-        E(f"if ((int)threadIdx.x < {self.D2}) {{ " + st(f"Yg + row * {self.D2} + threadIdx.x",
-                                                         " + ".join(f"dyp[{w * self.D2} + threadIdx.x]" for w in range(WPR))) + " }")
-        return E.text()
-
-    def plan(self):
-        fwd, bwd, ws = super().plan()
-        if self.row_waves > 1:
-            fwd[0]["num_threads"] = bwd[0]["num_threads"] = 64 * self.row_waves
-        return fwd, bwd, ws
-
     def tp_forward_body(self) -> str:
-        return self.split_forward_body() if self.row_waves > 1 else self.direct_forward_body()
+        return self.direct_forward_body()
 
     def tp_backward_body(self) -> str:
-        return self.split_backward_body() if self.row_waves > 1 else self.direct_backward_body()
+        return self.direct_backward_body()
 
     def conv_atomic_forward_body(self) -> str:
         return self.direct_forward_body()

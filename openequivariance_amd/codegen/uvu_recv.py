@@ -24,17 +24,17 @@ tiles: the dZ row of a receiver whose edges span two tiles is then re-read from 
 """
 from __future__ import annotations
 
-import os
-
 from ..problem import TPProblem
 from .common import Emitter
 from .uvu_det import UVUDetGenerator
 
 
 class UVURecvGenerator(UVUDetGenerator):
-    MIN_TILE_ITERS = int(os.environ.get("OEQ_AMD_RECV_MIN_ITERS", "8"))       # edge-loop iterations of the smallest tile
-    MAX_TILES = int(os.environ.get("OEQ_AMD_RECV_MAX_TILES", "16384"))       # tiles per chunk of the largest launches (the tile then grows with the edge count)
-    DX_UNROLL = int(os.environ.get("OEQ_AMD_RECV_DX_UNROLL", "4"))           # spill rows in flight per lane group in pass 2
+    # Tile counts from 4096 to one tile per 16 edges and 2 / 4 / 8 spill rows in flight in pass 2 moved pass 1 by
+    # less than 4 % (256 channels: 6.39 - 6.71 ms)
+    MIN_TILE_ITERS = 8       # edge-loop iterations of the smallest tile
+    MAX_TILES = 16384        # tiles per chunk of the largest launches (the tile then grows with the edge count)
+    DX_UNROLL = 4            # spill rows in flight per lane group in pass 2
 
     def __init__(self, problem: TPProblem, vector_stores: bool = True, idx_ctype: str = "i64", prefetch=None):
         # pass 1 is one launch: the per-edge dX rows cannot be split over launches of output-block groups
@@ -51,10 +51,8 @@ class UVURecvGenerator(UVUDetGenerator):
         per_edge = self.NW + sum(p.mv for p in self.paths) + len(self.used_y)
         # One register set measured faster than two on every shape tried (config 3: 0.182 vs 0.202 ms,
         # config 5: 7.93 vs 8.01 ms, the 128-channel MACE problem: 2.14 vs 5.05 ms, where two sets leave one
-        # wavefront per SIMD); OEQ_AMD_RECV_PREFETCH=1 turns the second set on for A/B runs.
-        self.prefetch_edges = os.environ.get("OEQ_AMD_RECV_PREFETCH", "0") == "1"
-        if prefetch is not None:
-            self.prefetch_edges = prefetch
+        # wavefront per SIMD); ``prefetch=True`` turns the second set on.
+        self.prefetch_edges = bool(prefetch)
         # large per-edge footprints: hold the allocation to two wavefronts per SIMD (a handful of spilled
         # words) instead of one
         self.waves_hint = 2 if held + per_edge > 100 else 0
@@ -90,7 +88,7 @@ class UVURecvGenerator(UVUDetGenerator):
         return fwd, bwd, ws
 
     def backward_kernel_sources(self):
-        w = int(os.environ.get("OEQ_AMD_RECV_WAVES", str(self.waves_hint)))
+        w = self.waves_hint
         attr = f" __attribute__((amdgpu_waves_per_eu({w}, {w})))" if w else ""
         return [dict(name="backward", threads=64, attr=attr, body=self._edges_body()),
                 dict(name="backward_dx", threads=64, attr="", body=self._dx_body())]

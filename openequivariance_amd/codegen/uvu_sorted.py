@@ -23,8 +23,7 @@ prepared by one forward and one backward call serves later calls on the same gra
 """
 from __future__ import annotations
 
-import os
-
+from .. import tunables
 from ..problem import TPProblem
 from .common import jinja_env
 from .uvu_det import UVUDetGenerator
@@ -47,9 +46,8 @@ class UVUSortedGenerator:
         self.problem = problem
         self.fwd = UVUDetGenerator(problem, forward_perm=True, vector_stores=vector_stores, idx_ctype=idx_ctype)
         if grouped_backward is None:
-            env = os.environ.get("OEQ_AMD_CONV_BACKWARD")            # "grouped" / "atomic": A/B runs
-            grouped_backward = (env == "grouped") if env in ("grouped", "atomic") \
-                else self.fwd.D1 >= self.ATOMIC_BACKWARD_MAX_D1
+            forced = tunables.current.conv_backward               # "grouped" / "atomic": A/B runs
+            grouped_backward = (forced == "grouped") if forced else self.fwd.D1 >= self.ATOMIC_BACKWARD_MAX_D1
         self.grouped_backward = grouped_backward
         if grouped_backward:
             self.bwd = UVUDetGenerator(problem, backward_perm=True, vector_stores=vector_stores, idx_ctype=idx_ctype)

@@ -33,8 +33,6 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Dict, List, Tuple
 
-import os
-
 import numpy as np
 
 from ..problem import TPProblem
@@ -92,13 +90,10 @@ class WPath:
 
 class UVWGenerator:
     DW_WORKGROUPS = 256          # persistent dW workgroups: one per compute unit of an MI355X
-    FWD_ACC_LIMIT = 80           # accumulator registers of one forward work item
-    # forward with the X tile in LDS, one workgroup per tile: "0", "1" or "auto" (when the tile fits the bound
-    # below).  Measured slower than one wavefront per work item (fp32 394 vs 359 us, fp64 747 vs 620 us on
-    # 64x0e+64x1o+64x2e: the wavefronts of a tile differ 7 : 4 : 1 in work and hold the tile's LDS until the
-    # longest is done), so it is off.
-    FWD_LDS_DEFAULT = "0"
-    FWD_LDS_MAX_BYTES = 40 * 1024
+    # Accumulator registers of one forward work item; an output block needing more is cut into ranges of its
+    # w tiles.  (48 instead of 80, for a third wavefront per SIMD, measured slower on 64x0e+64x1o+64x2e: fp32
+    # 0.329 -> 0.376 ms, fp64 0.566 -> 0.694 ms - the CG part of a tile is then computed once per range.)
+    FWD_ACC_LIMIT = 80
 
     def __init__(self, problem: TPProblem):
         self.problem = problem
@@ -108,20 +103,14 @@ class UVWGenerator:
         self.shared = bool(problem.shared_weights)
         if not self.shared and not getattr(self, "_allow_batched", False):
             raise NotImplementedError("this generator handles shared weights; see uvw_batched.py for per-row weights")
-        import os
-        # forward K loop: steps fetched per batch of loads, and unroll factor of the batch loop
-        # (measured on MI355X: fp32 4 / 1, fp64 1 / 3)
-        dflt = ("4", "1") if self.T == "float" else ("1", "3")
-        self.fwd_group = int(os.environ.get("OEQ_AMD_UVW_GROUP", dflt[0]))
-        self.fwd_unroll = int(os.environ.get("OEQ_AMD_UVW_UNROLL", dflt[1]))
-        # backward dX/dY: register sets for the packed weight fragments (2 = fetched one item ahead)
-        self.bwd_a_sets = int(os.environ.get("OEQ_AMD_UVW_ASETS", "1"))
-        self._bwd_lds_env = os.environ.get("OEQ_AMD_UVW_BWD_LDS", "1") == "1"
-        self.fwd_xcd_map = os.environ.get("OEQ_AMD_UVW_FWD_XCD", "1") == "1"
-        # forward: contract the CG tensor with the row's Y once per path and apply the small matrix per channel
-        self.fwd_row_matrix = os.environ.get("OEQ_AMD_UVW_FWD_MATRIX", "1") == "1"
-        # backward dW: fetch the operands of the next step while the current one runs (two register sets)
-        self.dw_prefetch = os.environ.get("OEQ_AMD_UVW_DW_PREFETCH", "1" if self.T == "float" else "0") == "1"
+        # forward K loop: steps fetched per batch of loads, and unroll factor of the batch loop (measured on
+        # MI355X: fp32 4 / 1, fp64 1 / 3; a loop written out on alternating register sets, so that nothing is
+        # copied between sets, has 0.9 instead of 2.1 vector-ALU instructions per MFMA and measured 0.341
+        # against 0.331 ms; larger groups for the cheap work items 0.361 - 0.422 against 0.359 ms)
+        self.fwd_group, self.fwd_unroll = (4, 1) if self.T == "float" else (1, 3)
+        # backward dW: fetch the operands of the next step while the current one runs (two register sets);
+        # in fp64 the second set crosses the 512-register limit even per pass (1.31 against 1.22 ms)
+        self.dw_prefetch = self.T == "float"
         self.in1, self.in2, self.out = _blocks(problem.irreps_in1), _blocks(problem.irreps_in2), _blocks(problem.irreps_out)
         self.D1, self.D2, self.D3 = problem.irreps_in1.dim, problem.irreps_in2.dim, problem.irreps_out.dim
         self.WN = problem.weight_numel
@@ -154,7 +143,7 @@ class UVWGenerator:
         # whose accumulator tile (D * tiles * 4 registers) exceeds FWD_ACC_LIMIT is cut into w ranges, each
         # a work item of its own: fewer accumulators per wavefront buy a third wavefront per SIMD, which
         # hides one wavefront's vector-ALU phases behind another's matrix-core phases
-        limit = int(os.environ.get("OEQ_AMD_UVW_FWD_ACC", str(self.FWD_ACC_LIMIT)))
+        limit = self.FWD_ACC_LIMIT
         self.fwd_order = []
         for o in sorted([o for o in self.out if o.dim > 0], key=lambda o: -cost(o)):
             nt_all = _ceil(o.mul, 16)
@@ -167,22 +156,10 @@ class UVWGenerator:
                 self.fwd_order.append((o, lo, min(nt_all, lo + step)))
         seg_cost = lambda it: cost(it[0]) * (it[2] - it[1]) / _ceil(it[0].mul, 16)
         self.fwd_order.sort(key=lambda it: -seg_cost(it))
-        # Work items of a tile: one segment each.  OEQ_AMD_UVW_FWD_ITEMS packs the segments (longest first, into
-        # the lightest item) into that many items per tile (-1: as many as the total work holds copies of the
-        # largest segment), a wavefront then runs the segments of its item one after the other.  Measured on
-        # 64x0e+64x1o+64x2e, [l=2], [l=1, l=0] (work 20 : 15) against three items (20 : 12 : 3): fp32 353 vs
-        # 350 us, fp64 670 vs 604 us, so the segments stay separate.
-        costs = [seg_cost(it) for it in self.fwd_order]
-        nitems = int(os.environ.get("OEQ_AMD_UVW_FWD_ITEMS", "0"))
-        if nitems < 0:
-            nitems = max(1, -(-int(sum(costs)) // max(1, int(max(costs))))) if max(costs) > 0 else 1
-        if nitems == 0 or nitems >= len(self.fwd_order):
-            self.fwd_items = [[i] for i in range(len(self.fwd_order))]
-        else:
-            bins = [[] for _ in range(nitems)]
-            for i in range(len(self.fwd_order)):
-                min(bins, key=lambda b: sum(costs[j] for j in b)).append(i)
-            self.fwd_items = sorted([b for b in bins if b], key=lambda b: -sum(costs[j] for j in b))
+        # Work items of a tile: one segment each.  (Packing the three segments of 64x0e+64x1o+64x2e into two
+        # items of similar length, work 20 : 15 instead of 20 : 12 : 3, measured fp32 353 against 350 us and
+        # fp64 670 against 604 us.)
+        self.fwd_items = [[i] for i in range(len(self.fwd_order))]
         # dW kernel: output blocks split into two groups of similar MFMA work
         # (f64 accumulators are twice as wide: one group, four wavefronts, the whole register file)
         work = {o: sum(p.o.D * p.NTW * p.NTU for p in self.paths if p.o.idx == o) for o in self.used_out}
@@ -195,13 +172,7 @@ class UVWGenerator:
         # backward dX/dY: the 16-row dZ tile is staged in LDS when it fits (row stride padded against bank
         # conflicts of the B-operand reads: lanes c = 0..15 read 16 different rows at the same column)
         self.bwd_rs = self._pick_row_stride()
-        self.bwd_lds = self._bwd_lds_env and 16 * self.bwd_rs * self.itemsize <= 80 * 1024    # gfx950: 160 KB per CU
-        # forward: the 16-row X tile staged in LDS once per workgroup, one wavefront per work item
-        self.fwd_xrs = self._pick_x_row_stride()
-        mode = os.environ.get("OEQ_AMD_UVW_FWD_LDS", self.FWD_LDS_DEFAULT)
-        fits = 16 * self.fwd_xrs * self.itemsize <= self.FWD_LDS_MAX_BYTES
-        self.fwd_lds = (mode == "1") or (mode == "auto" and fits)
-        self.fwd_waves = min(len(self.fwd_items), 8) if self.fwd_lds else 1
+        self.bwd_lds = 16 * self.bwd_rs * self.itemsize <= 80 * 1024    # gfx950: 160 KB per CU
         # packed weight copies in the workspace
         pos = 0
         for p in self.paths:
@@ -219,48 +190,13 @@ class UVWGenerator:
         self.ws_elems = self.PART_OFF + self.DW_WORKGROUPS * self.WN
 
     # ------------------------------------------------------------------ helpers
-    def fwd_group_of(self, o: Block) -> int:
-        """K steps fetched per batch of loads in the forward work item of output block ``o``: the fewer matrix
-        instructions a step has (2l+1 per w tile), the more steps one batch must cover for the next batch's
-        operands to arrive in time."""
-        per_l = os.environ.get("OEQ_AMD_UVW_GROUPS", "")
-        if per_l:
-            tab = [int(v) for v in per_l.split(",")]
-            return tab[min(o.l, len(tab) - 1)]
-        return self.fwd_group
-
-    def forward_attr(self) -> str:
-        """Occupancy target of the forward kernel (wavefronts per SIMD), when one is set."""
-        w = int(os.environ.get("OEQ_AMD_UVW_FWD_OCC", "0"))
-        return f" __attribute__((amdgpu_waves_per_eu({w}, {w})))" if w else ""
-
     def backward_attr(self) -> str:
         """Occupancy target of the dX/dY kernel: as many workgroups per CU (one wavefront per SIMD
         each) as the LDS tile allows; the register allocator then stays within that budget."""
-        if not self.bwd_lds or os.environ.get("OEQ_AMD_UVW_BWD_OCC", "1") != "1":
+        if not self.bwd_lds:
             return ""
         per_cu = max(1, min(4, (160 * 1024) // (16 * self.bwd_rs * self.itemsize + 4 * 16 * max(1, self.D2) * self.itemsize)))
         return f" __attribute__((amdgpu_waves_per_eu({per_cu}, {per_cu})))" if per_cu >= 3 else ""
-
-    def _pick_x_row_stride(self) -> int:
-        """Row stride (elements) of the X tile in LDS: a multiple of the 16-byte vector the tile is written
-        with, padded so that the 16 rows x 2 lane groups of one LDS pass spread best over the 32 banks."""
-        words, vw = self.itemsize // 4, 16 // self.itemsize
-        base = _ceil(self.D1, vw) * vw
-        best = None
-        for pad in range(0, 33, vw):
-            rs = base + pad
-            worst = 0
-            for d in {a.D for a in self.in1 if a.dim}:
-                hits = {}
-                for c in range(16):
-                    for g in range(2):
-                        bank = ((c * rs + g * 4 * d) * words) % 32
-                        hits[bank] = hits.get(bank, 0) + 1
-                worst = max(worst, max(hits.values()))
-            if best is None or worst < best[0]:
-                best = (worst, rs)
-        return best[1]
 
     def _pick_row_stride(self) -> int:
         """Row stride (elements) of the dZ tile in LDS: the smallest padding for which the 32 lanes of
@@ -397,10 +333,8 @@ class UVWGenerator:
     def forward_body(self) -> str:
         E = Emitter()
         NO = len(self.fwd_items)
-        if self.fwd_lds:
-            return self._forward_items(E, self._forward_lds_head(E))
         E("const int lane = threadIdx.x, c = lane & 15, g = lane >> 4;")
-        if self.fwd_xcd_map:
+        if True:          # (kept as a block: the mapping below is the only one)
             # Work item = (batch tile, output block).  Workgroups are handed to the 8 XCDs round robin by
             # their linear id, and every XCD has an L2 of its own: the items of one tile get ids 8 apart,
             # i.e. consecutive turns of the same XCD, so that the X rows fetched for the first output
@@ -409,14 +343,11 @@ class UVWGenerator:
             # The last fifth of the tiles is laid out item-major instead (all their most expensive items, then
             # the next ...): the launch then ends on the cheap items, which shortens its ragged end
             # (measured: forward 356 -> 346 us in fp32, 616 -> 598 us in fp64; a third or a half: no better).
-            tail = int(os.environ.get("OEQ_AMD_UVW_FWD_TAIL", "5"))
-            head8 = f"((ntiles - ntiles / {tail}) >> 3)" if tail else "(ntiles >> 3)"
+            head8 = "((ntiles - ntiles / 5) >> 3)"
             E(f"const u64 head = {head8} << 3, full = head * {NO};")
             E("u64 tile; int slot;")
             E(f"if (lin < full) {{ const u64 j = lin >> 3; slot = (int)(j % {NO}); tile = (j / {NO}) * 8 + (lin & 7); }}")
             E("else { const u64 rem = ntiles - head, l2 = lin - full; slot = (int)(l2 / rem); tile = head + l2 % rem; }")
-        else:
-            E("const u64 tile = blockIdx.x; const int slot = blockIdx.y;")
         E("const u64 row0 = tile * 16;")
         E("if (row0 >= n) return;")
         E("const u64 rowA = min(row0 + (u64)c, n - 1);       // rows past the end repeat the last row, never stored")
@@ -428,48 +359,6 @@ class UVWGenerator:
         # to the least expensive, so the dispatcher fills the tail of the launch with the cheap ones
         # (whole tiles per wavefront leave a third of the machine idle while the last ones finish).
         return self._forward_items(E, lambda slot: f"slot == {slot}")
-
-    def _forward_lds_head(self, E: Emitter):
-        """Workgroup = one batch tile, one wavefront per work item.  The 16 rows of X are contiguous in
-        memory: the workgroup copies them into LDS with 16-byte vectors that are all requested before the
-        first is written, and the K loops read their X records from there - X crosses the memory system
-        once, with one exposed round trip per tile instead of one per path and work item.  Returns the
-        condition that selects a work item."""
-        NWV, RS, VW = self.fwd_waves, self.fwd_xrs, self.VW
-        NTH = 64 * NWV
-        E("const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, c = lane & 15, g = lane >> 4;")
-        E("const u64 row0 = (u64)blockIdx.x * 16;")
-        E("if (row0 >= n) return;")
-        E("const u64 rowA = min(row0 + (u64)c, n - 1);       // rows past the end repeat the last row, never stored")
-        E("const T* __restrict__ wsT = (const T*)ws;")
-        E(f"__shared__ T xl[16 * {RS}];")
-        for f in self.used_y:
-            E(f"const T y{f} = Y[rowA * {self.D2} + {f}];")
-        if self.D1 % VW == 0:
-            NV, RV = 16 * self.D1 // VW, self.D1 // VW
-            NQ = _ceil(NV, NTH)
-            E("if ((((unsigned long long)X) & 15ull) == 0) {")
-            E.level += 1
-            E(f"VT xv[{NQ}];")
-            for q in range(NQ):
-                idx = f"(int)threadIdx.x + {NTH * q}"
-                guard = "" if NTH * (q + 1) <= NV else f"if ({idx} < {NV}) "
-                E(f"{guard}{{ const int r_ = ({idx}) / {RV}, v_ = ({idx}) - r_ * {RV}; "
-                  f"xv[{q}] = *(const VT*)(X + min(row0 + (u64)r_, n - 1) * {self.D1} + v_ * {VW}); }}")
-            for q in range(NQ):
-                idx = f"(int)threadIdx.x + {NTH * q}"
-                guard = "" if NTH * (q + 1) <= NV else f"if ({idx} < {NV}) "
-                E(f"{guard}{{ const int r_ = ({idx}) / {RV}, v_ = ({idx}) - r_ * {RV}; T* __restrict__ d_ = xl + r_ * {RS} + v_ * {VW}; "
-                  + " ".join(f"d_[{i}] = xv[{q}][{i}];" for i in range(VW)) + " }")
-            E.level -= 1
-            E("} else")
-        E(f"for (int q = threadIdx.x; q < 16 * {self.D1}; q += {NTH}) {{")
-        E(f"    const int r_ = q / {self.D1}, col_ = q - r_ * {self.D1};")
-        E(f"    xl[r_ * {RS} + col_] = X[min(row0 + (u64)r_, n - 1) * {self.D1} + col_];")
-        E("}")
-        E("__syncthreads();")
-        E(f"const T* __restrict__ Xr = xl + c * {RS};")
-        return lambda slot: f"wave == {slot % NWV}"
 
     def _forward_items(self, E: Emitter, select) -> str:
         for slot, item in enumerate(self.fwd_items):
@@ -504,15 +393,14 @@ class UVWGenerator:
                 # matrix core.  What bounds this kernel is the L2 -> L1 stream of operands (every
                 # wavefront re-reads the packed weights), so the bytes in flight per wavefront matter
                 # more than anything else here.
-                GS = self.fwd_group_of(o)
+                GS = self.fwd_group
                 NG = _ceil(p.SU, GS)
-                pingpong = (self.fwd_unroll == 0)
-                sets = ("a", "b") if pingpong else ("n",)
+                sets = ("n",)
                 regs = [f"{q}x{j}_{i}" for q in sets for j in range(GS) for i in range(p.a.D)] \
                     + [f"{q}b{j}_{nt}" for q in sets for j in range(GS) for nt in NTS]
                 E("T " + ", ".join(regs) + ";")
-                if self.fwd_row_matrix:
-                    self.emit_cg_matrix(E, p, "y", "m")
+                # the CG tensor is contracted with the row's Y once per path; the small matrix is applied per channel
+                self.emit_cg_matrix(E, p, "y", "m")
 
                 def load(E, gexp, q="n"):
                     for j in range(GS):
@@ -532,10 +420,7 @@ class UVWGenerator:
                         E("{")
                         E.level += 1
                         E("const T " + ", ".join(f"x{i} = {q}x{j}_{i}" for i in range(p.a.D)) + ";")
-                        if self.fwd_row_matrix:
-                            self.emit_cg_apply(E, p, "x", "m", "t")
-                        else:
-                            self.emit_cg_forward(E, p, "x", "y", "t")
+                        self.emit_cg_apply(E, p, "x", "m", "t")
                         if p.mu % 16 != 0 or NG * GS != p.SU:
                             E(f"if (16 * ((({sgexp}) * {GS} + {j}) >> 2) + 4 * g + ((({sgexp}) * {GS} + {j}) & 3) >= {p.mu}) {{ " + " ".join(f"t{k} = (T)0;" for k in range(o.D)) + " }")
                         for k in range(o.D):
@@ -543,29 +428,19 @@ class UVWGenerator:
                                 E(f"acc{k}_{nt} = oeq_mfma(t{k}, {q}b{j}_{nt}, acc{k}_{nt});")
                         E.level -= 1
                         E("}")
-                if pingpong:
-                    # the groups are written out one after the other on alternating register sets: the operands
-                    # of the next group are requested into the other set, nothing is copied between sets
-                    load(E, "0", "a")
-                    for sg in range(NG):
-                        cur, nxt = ("a", "b") if sg % 2 == 0 else ("b", "a")
-                        if sg + 1 < NG:
-                            load(E, str(sg + 1), nxt)
-                        steps(E, str(sg), cur)
-                else:
-                    load(E, "0")
-                    E(f"#pragma unroll {self.fwd_unroll}")
-                    E(f"for (int sg = 0; sg < {NG}; ++sg) {{")
-                    E.level += 1
-                    E("const T " + ", ".join(f"c{r} = {r}" for r in regs) + ";")
-                    E(f"if (sg + 1 < {NG}) {{")
-                    E.level += 1
-                    load(E, "sg + 1")
-                    E.level -= 1
-                    E("}")
-                    steps(E, "sg", "cn")
-                    E.level -= 1
-                    E("}")
+                load(E, "0")
+                E(f"#pragma unroll {self.fwd_unroll}")
+                E(f"for (int sg = 0; sg < {NG}; ++sg) {{")
+                E.level += 1
+                E("const T " + ", ".join(f"c{r} = {r}" for r in regs) + ";")
+                E(f"if (sg + 1 < {NG}) {{")
+                E.level += 1
+                load(E, "sg + 1")
+                E.level -= 1
+                E("}")
+                steps(E, "sg", "cn")
+                E.level -= 1
+                E("}")
                 E.level -= 1
                 E("}")
             # lane holds, for each of its 4 rows, w = NT*c + nt (nt < NT) and all k: a contiguous run
@@ -669,7 +544,7 @@ class UVWGenerator:
         else:
             items = [(oi, p, q) for oi in self.used_out for p in self.paths_into(oi) for q in range(_ceil(p.NTU, 4))]
         max_sw = max(_ceil(self.out[oi].mul, 4) for oi in self.used_out)
-        NSETS = self.bwd_a_sets
+        NSETS = 1          # register sets of packed weight fragments (a second set, fetched one item ahead, measured no gain)
         E("T " + ", ".join(f"af{b_}_{s_}" for b_ in range(NSETS) for s_ in range(max_sw)) + ";")
 
         def load_a(E, j):
@@ -784,28 +659,39 @@ class UVWGenerator:
     DW_ACC_BUDGET = {4: 352, 8: 192}
 
     def dw_passes(self):
-        """(wavefront group, paths) of the passes of the dW kernel.  The accumulators of all paths of a
-        pass are live at once (4 registers per 16 x 16 tile, 8 in fp64); problems with many paths - every
-        copy of a second operand with mul > 1 is a path of its own - are cut into passes of at most
-        DW_ACC_BUDGET accumulator registers, each walking the batch again, so that the register file is
-        never oversubscribed (a kernel spilling hundreds of accumulators is slow, and its fp64 results
-        were not exact on the device)."""
+        """(wavefront group, [(path, first w tile, end w tile), ...]) of the passes of the dW kernel.  The
+        accumulators of all segments of a pass are live at once (4 registers per 16 x 16 tile, 8 in fp64);
+        problems with many paths - every copy of a second operand with mul > 1 is a path of its own - are
+        cut into passes of at most DW_ACC_BUDGET accumulator registers, each walking the batch again, and
+        a single path that exceeds the budget is cut by ranges of its 16-wide w tiles, so that the register
+        file is never oversubscribed (a kernel spilling hundreds of accumulators is slow, and its fp64
+        results were not exact on the device)."""
         per_tile = 4 * (self.itemsize // 4)
-        budget = int(os.environ.get("OEQ_AMD_UVW_DW_ACC", str(self.DW_ACC_BUDGET[self.itemsize])))
+        budget = self.DW_ACC_BUDGET[self.itemsize]
         passes = []
         for grp in range(self.dw_groups):
-            mine = [p for p in self.paths if self.dw_group[p.o.idx] == grp]
-            need = {p.t: _ceil(p.NTU, 4) * p.NTW * per_tile for p in mine}
-            total = sum(need.values())
+            segs = []
+            for p in (p for p in self.paths if self.dw_group[p.o.idx] == grp):
+                per_w = _ceil(p.NTU, 4) * per_tile                 # accumulator registers of one w tile
+                if per_w > budget:
+                    raise NotImplementedError(
+                        f"uvw dW: {p.mu} channels of the first operand need {per_w} accumulator registers per "
+                        f"16-wide tile of the output, more than the {budget} one pass may hold")
+                step = min(p.NTW, budget // per_w)
+                pieces = _ceil(p.NTW, step)
+                step = _ceil(p.NTW, pieces)                        # pieces of about equal width
+                segs += [(p, lo, min(p.NTW, lo + step)) for lo in range(0, p.NTW, step)]
+            need = [_ceil(p.NTU, 4) * (hi - lo) * per_tile for p, lo, hi in segs]
+            total = sum(need)
             count = max(1, _ceil(total, budget))
             target = total / count                   # passes of about equal accumulator count
             cur, used = [], 0
-            for p in mine:
-                if cur and (used + need[p.t] > budget or used >= target):
+            for seg, nd in zip(segs, need):
+                if cur and (used + nd > budget or used >= target):
                     passes.append((grp, cur))
                     cur, used = [], 0
-                cur.append(p)
-                used += need[p.t]
+                cur.append(seg)
+                used += nd
             if cur:
                 passes.append((grp, cur))
         return passes
@@ -819,17 +705,20 @@ class UVWGenerator:
         E("const int lane = threadIdx.x & 63, wave = (threadIdx.x >> 6) & 3, grp = threadIdx.x >> 8, c = lane & 15, g = lane >> 4;")
         E("const u64 ntiles = (n + 15) / 16;")
         E(f"T* __restrict__ part = (T*)ws + {self.PART_OFF} + (u64)blockIdx.x * {self.WN};")
-        for grp, paths in self.dw_passes():
-            # a pass: these paths' accumulators are the only ones live while the batch is walked once
+        for grp, segs in self.dw_passes():
+            # a pass: these segments' accumulators are the only ones live while the batch is walked once
+            paths = [p for p, _, _ in segs]
             outs = sorted({p.o.idx for p in paths})
             ins = sorted({p.a.idx for p in paths})
             ys = sorted({p.b.off + j for p in paths for (_, j) in p.pairs})
-            into = lambda oi, paths=paths: [p for p in paths if p.o.idx == oi]
+            into = lambda oi, segs=segs: [sg for sg in segs if sg[0].o.idx == oi]
+            # w tiles of an output block whose dZ records this pass reads
+            tiles_of = {oi: sorted({nt for p, lo, hi in segs if p.o.idx == oi for nt in range(lo, hi)}) for oi in outs}
             E(f"if (grp == {grp}) {{")
             E.level += 1
-            for p in paths:
+            for p, lo, hi in segs:
                 for q in range(_ceil(p.NTU, 4)):
-                    for nt in range(p.NTW):
+                    for nt in range(lo, hi):
                         E(f"V4 acc{p.t}_{q}_{nt} = {{0, 0, 0, 0}};")
             if self.dw_prefetch:
                 # One step = 4 batch rows (the K of one MFMA) of one tile.  The steps of all tiles of this
@@ -842,9 +731,9 @@ class UVWGenerator:
                     names += [f"x{ai}_{q}_{i}" for q in range(_ceil(_ceil(a_.mul, 16), 4)) for i in range(a_.D)]
                 for oi in outs:
                     o = self.out[oi]
-                    names += [f"gz{oi}_{nt}_{k}" for nt in range(_ceil(o.mul, 16)) for k in range(o.D)]
+                    names += [f"gz{oi}_{nt}_{k}" for nt in tiles_of[oi] for k in range(o.D)]
 
-                def load(E, it, h, ys=ys, ins=ins, outs=outs):
+                def load(E, it, h, ys=ys, ins=ins, outs=outs, tiles_of=tiles_of):
                     E("{")
                     E.level += 1
                     E(f"const u64 b = (blockIdx.x + (u64)(({it}) >> 2) * gridDim.x) * 16 + 4 * (({it}) & 3) + g;   // batch row of this lane for both operands")
@@ -866,7 +755,7 @@ class UVWGenerator:
                                 E(f"if ({uexp} >= {a_.mul}) {{ " + " ".join(f"S{h}x{ai}_{q}_{i} = (T)0;" for i in range(a_.D)) + " }")
                     for oi in outs:
                         o = self.out[oi]
-                        for nt in range(_ceil(o.mul, 16)):
+                        for nt in tiles_of[oi]:
                             wexp = f"{16 * nt} + c"
                             wcl = wexp if o.mul % 16 == 0 else f"min({wexp}, {o.mul - 1})"
                             E(f"{{ const T* __restrict__ gp = Gr + {o.off} + ({wcl}) * {o.D}; "
@@ -877,13 +766,12 @@ class UVWGenerator:
                 def compute(E, outs=outs, into=into):
                     for oi in outs:
                         o = self.out[oi]
-                        NT = _ceil(o.mul, 16)
-                        for p in into(oi):
+                        for p, lo, hi in into(oi):
                             for q in range(_ceil(p.NTU, 4)):
-                                E(f"if (wave + {4 * q} < {p.NTU}) {{  // path {p.t}")
+                                E(f"if (wave + {4 * q} < {p.NTU}) {{  // path {p.t}, w tiles {lo} .. {hi - 1}")
                                 E.level += 1
                                 self.emit_cg_forward(E, p, f"x{p.a.idx}_{q}_", "y", "t")
-                                for nt in range(NT):
+                                for nt in range(lo, hi):
                                     for k in range(o.D):
                                         E(f"acc{p.t}_{q}_{nt} = oeq_mfma(t{k}, gz{oi}_{nt}_{k}, acc{p.t}_{q}_{nt});")
                                 E.level -= 1
@@ -956,20 +844,19 @@ class UVWGenerator:
                             E(f"if ({uexp} >= {a_.mul}) {{ " + " ".join(f"x{ai}_{q}_{i} = (T)0;" for i in range(a_.D)) + " }")
                 for oi in outs:
                     o = self.out[oi]
-                    NT = _ceil(o.mul, 16)
                     E(f"{{ // output block {oi}: dZ records, w = 16 nt + c")
                     E.level += 1
-                    for nt in range(NT):
+                    for nt in tiles_of[oi]:
                         wexp = f"{16 * nt} + c"
                         wcl = wexp if o.mul % 16 == 0 else f"min({wexp}, {o.mul - 1})"
                         E(f"const T* __restrict__ gp{nt} = Gr + {o.off} + ({wcl}) * {o.D};")
                         E("const T " + ", ".join(f"gz{nt}_{k} = gp{nt}[{k}]" for k in range(o.D)) + ";")
-                    for p in into(oi):
+                    for p, lo, hi in into(oi):
                         for q in range(_ceil(p.NTU, 4)):
-                            E(f"if (wave + {4 * q} < {p.NTU}) {{  // path {p.t}")
+                            E(f"if (wave + {4 * q} < {p.NTU}) {{  // path {p.t}, w tiles {lo} .. {hi - 1}")
                             E.level += 1
                             self.emit_cg_forward(E, p, f"x{p.a.idx}_{q}_", "y", "t")
-                            for nt in range(NT):
+                            for nt in range(lo, hi):
                                 for k in range(o.D):
                                     E(f"acc{p.t}_{q}_{nt} = oeq_mfma(t{k}, gz{nt}_{k}, acc{p.t}_{q}_{nt});")
                             E.level -= 1
@@ -981,10 +868,10 @@ class UVWGenerator:
                 E.level -= 1
                 E("}")
             # ---- partial sums of this workgroup, laid out [t][u][w]
-            for p in paths:
+            for p, lo, hi in segs:
                 for q in range(_ceil(p.NTU, 4)):
                     E(f"if (wave + {4 * q} < {p.NTU}) {{")
-                    for nt in range(p.NTW):
+                    for nt in range(lo, hi):
                         for r in range(4):
                             E(f"    {{ const int u = 16 * (wave + {4 * q}) + {self.row(r)}; const int w = {16 * nt} + c;")
                             E(f"      if (u < {p.mu} && w < {p.mw}) part[{p.poff} + u * {p.mw} + w] = acc{p.t}_{q}_{nt}[{r}]; }}")
@@ -1020,8 +907,7 @@ class UVWGenerator:
     def plan(self):
         FIXED, ROW = 0, 1
         fwd = [dict(kernel="prep_forward", num_threads=256, grid_kind=FIXED, num_blocks=self.prep_blocks),
-               dict(kernel="forward", num_threads=64 * self.fwd_waves, grid_kind=ROW, work_per_block=16,
-                    grid_y=1 if self.fwd_lds else len(self.fwd_items))]
+               dict(kernel="forward", num_threads=64, grid_kind=ROW, work_per_block=16, grid_y=len(self.fwd_items))]
         bwd = [dict(kernel="prep_backward", num_threads=256, grid_kind=FIXED, num_blocks=self.prep_blocks),
                dict(kernel="backward", num_threads=256, grid_kind=ROW, work_per_block=16),
                dict(kernel="backward_dw", num_threads=256 * self.dw_groups, grid_kind=FIXED,

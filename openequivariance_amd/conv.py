@@ -15,13 +15,13 @@ assumption about the graph.
 """
 from __future__ import annotations
 
-import os
 import typing
 
 import numpy as np
 import torch
 
 from . import runtime as rt
+from . import tunables
 from .autograd_glue import double_backward_terms
 from .codegen.uvu_det import UVUDetGenerator
 from .codegen.uvu_direct import UVUDirectGenerator
@@ -91,16 +91,28 @@ def sort_by_receiver(rows: "torch.Tensor", cols: "torch.Tensor", node_count: typ
     return rows_s, cols_s, receiver_perm, transpose_perm
 
 
+# d3 / d1 from which the deterministic backward walks the edges in receiver order (see select_conv_generator)
+RECV_ORDER_MIN_RATIO = 7
+
+
 def select_conv_generator(config: TPProblem, deterministic: bool, vector_stores: bool = True, idx_dtype=np.int64):
     """Kernel generator of the fused convolution: one node per wavefront with fixed summation order
     when deterministic; otherwise a forward that groups the edges by receiver on the fly and a
     backward with coalesced atomics."""
     idx_ctype = "i64" if np.dtype(idx_dtype) == np.dtype(np.int64) else "int"
     if deterministic:
-        if os.environ.get("OEQ_AMD_DET_BACKWARD", "send") == "recv":
+        order = tunables.current.det_backward
+        if order is None:
+            # Static rule (no clock: which kernel runs must not depend on timing if results are to repeat
+            # bit for bit).  The sender order gathers a dZ row (d3 words) per edge, the receiver order an X
+            # row and spills a dX row (3 d1 words, half of them writes).  Measured backward, sender against
+            # receiver order: d3 / d1 = 3.9 (32 channels) 0.155 / 0.187 ms, 4.8 (256 channels) 7.48 / 7.78 ms,
+            # 7.9 (the 128-channel MACE problem) 2.15 / 2.07 ms.
+            order = "recv" if config.irreps_out.dim >= RECV_ORDER_MIN_RATIO * config.irreps_in1.dim else "send"
+        if order == "recv":
             return UVURecvGenerator(config, vector_stores=vector_stores, idx_ctype=idx_ctype)
         return UVUDetGenerator(config, vector_stores=vector_stores, idx_ctype=idx_ctype)
-    if os.environ.get("OEQ_AMD_CONV_FORWARD", "sorted") == "atomic":     # A/B measurements only
+    if tunables.current.conv_forward == "atomic":     # A/B measurements only
         g = UVUDirectGenerator(config, "conv_atomic", vector_stores=vector_stores)
         g.idx_ctype = idx_ctype
         return g
@@ -124,7 +136,13 @@ class TensorProductConv:
     next_conv_id = 0
 
     def __init__(self, config: TPProblem, torch_op: bool = False, deterministic: bool = False,
-                 idx_dtype=np.int64):
+                 idx_dtype=np.int64, graph_cache: typing.Optional[bool] = None):
+        """``graph_cache=True`` (default: ``tunables.graph_cache``, off) lets the torch operators skip the
+        graph preparation when a call names the same index tensors as the previous one (same addresses,
+        same in-place version counters, same sizes).  The key cannot see writes that bypass torch's version
+        counter - memory wrapped with from_blob / DLPack, kernels of other libraries writing into a
+        preallocated neighbour list, a HIP graph replay rewriting a static index buffer - so it is for
+        callers who know that their index tensors change only through torch."""
         assert isinstance(config, TPProblem)
         self.config = config
         self.L1, self.L2, self.L3 = config.irreps_in1, config.irreps_in2, config.irreps_out
@@ -158,7 +176,7 @@ class TensorProductConv:
         # sender first depends on the row length AND on the graph (atomics per edge against the gathers of
         # the segmented kernel); the generator's rule of thumb is only the starting point.  The torch
         # operator times both on the first backward call of each size class and keeps the faster one
-        # (OEQ_AMD_CONV_BACKWARD=atomic|grouped or OEQ_AMD_AUTOTUNE=0 switch the measurement off).  The
+        # (``tunables.conv_backward`` = atomic | grouped or ``tunables.autotune`` = False switch the measurement off).  The
         # deterministic operator never chooses by timing: which kernel runs must not depend on a stopwatch
         # if results are to repeat bit for bit from one process to the next.
         self._bwd_variants = {}
@@ -166,9 +184,9 @@ class TensorProductConv:
         if isinstance(self.generator, UVUSortedGenerator):
             self._bwd_default = "grouped" if self.generator.grouped_backward else "atomic"
             self._bwd_variants[self._bwd_default] = (self.internal, self.backward_overwrites)
-        self.autotune = (bool(self._bwd_variants) and os.environ.get("OEQ_AMD_AUTOTUNE", "1") != "0"
-                         and os.environ.get("OEQ_AMD_CONV_BACKWARD") not in ("atomic", "grouped"))
-        self.graph_cache = os.environ.get("OEQ_AMD_GRAPH_CACHE", "1") != "0"
+        self.autotune = (bool(self._bwd_variants) and tunables.current.autotune
+                         and tunables.current.conv_backward is None)
+        self.graph_cache = tunables.current.graph_cache if graph_cache is None else bool(graph_cache)
         self._internal_unaligned = None
         self._reorder = WeightReorder(config)
         self.reorder_weights_e3nn_to_oeq = self._reorder.e3nn_to_oeq

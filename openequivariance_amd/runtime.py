@@ -14,9 +14,11 @@ import pathlib
 import threading
 from typing import List, Optional, Sequence
 
+from . import tunables
+
 PKG_DIR = pathlib.Path(__file__).resolve().parent
 LIB_PATH = PKG_DIR / "csrc" / "liboeq_hip.so"
-CACHE_DIR = pathlib.Path(os.environ.get("OEQ_AMD_CACHE", PKG_DIR / "_kcache"))
+CACHE_DIR = tunables.current.cache_dir
 TARGET_ARCH = "gfx950"
 
 GRID_FIXED, GRID_PER_ROW, GRID_PER_NODE = 0, 1, 2

@@ -88,6 +88,32 @@ def backward(prob: Problem, X, Y, W, G):
     return dX, dY, dW
 
 
+def shared_weight_gradient(prob: Problem, X, Y, G, chunk: int = 8192):
+    """dW of <G, Z> for shared weights (e3nn order), accumulated in float64 over chunks of rows: the
+    same contraction as ``backward`` split in two steps, ``T = C x y`` then ``dW = T . G`` over
+    (row, k), so that a batch of 10^5 rows costs seconds and bounded memory.  Pinned against
+    ``backward`` in tests/test_oracle.py."""
+    assert prob.shared_weights
+    X, Y, G = (np.asarray(a) for a in (X, Y, G))
+    dW = np.zeros(prob.weight_numel)
+    for b0 in range(0, X.shape[0], chunk):
+        Xc, Yc, Gc = (np.asarray(a[b0:b0 + chunk], dtype=np.float64) for a in (X, Y, G))
+        B = Xc.shape[0]
+        for p in prob.paths:
+            (m1, l1, o1), (m2, l2, o2), (mo, l3, o3) = _blocks(prob, p)
+            C = wigner_3j(l1, l2, l3) * p["coeff"]
+            x = Xc[:, o1:o1 + m1 * (2 * l1 + 1)].reshape(B, m1, 2 * l1 + 1)
+            y = Yc[:, o2:o2 + m2 * (2 * l2 + 1)].reshape(B, m2, 2 * l2 + 1)
+            g = Gc[:, o3:o3 + mo * (2 * l3 + 1)].reshape(B, mo, 2 * l3 + 1)
+            T = np.einsum("ijk,zui,zvj->zuvk", C, x, y, optimize=True)
+            if p["mode"] == "uvu":
+                dw = np.einsum("zuvk,zuk->uv", T, g, optimize=True)
+            else:
+                dw = np.tensordot(T, g, axes=([0, 3], [0, 2]))            # [u, v, w]
+            dW[p["woff"]: p["woff"] + prod(p["shape"])] += dw.reshape(-1)
+    return dW
+
+
 # ---------------------------------------------------------------------------
 # fused convolution: Z[n] = sum over edges e with rows[e] == n of TP(X[cols[e]], Y[e], W[e])
 # ---------------------------------------------------------------------------

@@ -39,20 +39,6 @@ def test_direct_tp_ragged_two_chunks():
     _tp(UVUDirectGenerator, ("5x0e+3x1o+70x2e", "1x0e+1x1o+1x2e", "5x0e+3x1o+70x2e+7x3o"), 3, 2)
 
 
-@pytest.mark.parametrize("irreps,waves", [(("64x0e+64x1o+64x2e", "1x0e+1x1o+1x2e", "64x0e+64x1o+64x2e+64x1e"), 4),
-                                          (("70x0e+100x1o", "1x0e+1x1o+1x2e", "70x0e+70x1o+100x1o+100x2e"), 3),
-                                          (("128x0e+128x1o", "1x0e+1x1o", "128x0e+128x1o+128x1o+128x0e"), 2)])
-def test_direct_tp_row_dealt_to_several_wavefronts(irreps, waves, monkeypatch):
-    """One row per workgroup of 2-4 wavefronts: contiguous parts of the Z / dZ row each, dX and dY combined
-    through LDS in a fixed order (full and ragged chunks, one and two chunks, blocks nobody writes)."""
-    monkeypatch.setenv("OEQ_AMD_TP_ROW_WAVES", str(waves))
-    prob, _ = common.channelwise(irreps)
-    g = UVUDirectGenerator(prob, "tp")
-    assert g.row_waves == waves and all(g.row_items())
-    assert g.plan()[0][0]["num_threads"] == 64 * waves
-    _tp(UVUDirectGenerator, irreps, 3, 5)
-
-
 def test_direct_tp_record_stores_only():
     _tp(UVUDirectGenerator, common.NEQUIP, 3, 3, vector_stores=False)
 
@@ -99,13 +85,12 @@ def test_conv(variant):
 
 
 @pytest.mark.parametrize("staged", [True, False])
-def test_conv_det_long_edge_lists(staged, monkeypatch):
+def test_conv_det_long_edge_lists(staged):
     """Edge lists of about 13 edges per node (6-7 iterations of two sub-lists) reach the steady state of
     the edge pipeline, with the next edge's operands staged through LDS and with register prefetch; the
     last node has no edges."""
-    monkeypatch.setenv("OEQ_AMD_DET_LDS", "1" if staged else "0")
     prob, oprob = common.channelwise(common.NEQUIP)
-    g = UVUDetGenerator(prob)
+    g = UVUDetGenerator(prob, lds=staged)
     assert g.lds_backward == staged and g.lds_forward == staged
     nodes, nnz = 4, 40
     rows, cols = common.random_graph(nodes - 1, nnz, 11)          # node 3 has no edges
@@ -222,6 +207,27 @@ def test_uvw_matrix_core_kernels(dtype, monkeypatch):
     assert rel_err(ow.oeq_to_e3nn(oprob, out["Wg"]), dW) < tol
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_uvw_dw_single_path_beyond_the_accumulator_budget(dtype, monkeypatch):
+    """One path whose accumulators alone exceed what a dW pass may hold is cut by ranges of its w tiles: with
+    the budget lowered to two tiles' worth, 70 x 40 channels take three passes for the first path."""
+    monkeypatch.setattr(UVWGenerator, "DW_WORKGROUPS", 2)
+    per_tile = 4 if dtype == np.float32 else 8
+    monkeypatch.setattr(UVWGenerator, "DW_ACC_BUDGET", {4: 4 * per_tile, 8: 4 * per_tile})     # ceil(5 / 4) = 2 u groups x 2 w tiles
+    a = ("70x0e+5x1o", "1x0e+1x1o", "40x0e+9x1o")
+    prob, oprob = common.fully_connected(a, shared=True, dtype=dtype)
+    g = UVWGenerator(prob)
+    passes = g.dw_passes()
+    assert max(sum(-(-p.NTU // 4) * (hi - lo) * per_tile for p, lo, hi in segs) for _, segs in passes) <= 4 * per_tile
+    assert sum(1 for _, segs in passes for p, lo, hi in segs if p.t == 0) >= 2
+    X, Y, We, G = common.tp_inputs(prob, 19, 13, dtype, w_scale=0.3)
+    W = ow.e3nn_to_oeq(oprob, We)
+    _, bwd, ws = g.plan()
+    out = emu.run_tp(g, bwd, X, Y, W, G, ws_bytes=ws())
+    tol = TOL if dtype == np.float32 else 1e-13
+    assert rel_err(ow.oeq_to_e3nn(oprob, out["Wg"]), otp.backward(oprob, X, Y, We, G)[2]) < tol
+
+
 def test_uvw_forward_work_item_mapping_over_many_tiles():
     """19 batch tiles: 16 of them in groups of 8 with the items of a tile 8 workgroup ids apart, the last three
     item-major; every (tile, item) pair must be visited exactly once."""
@@ -232,24 +238,6 @@ def test_uvw_forward_work_item_mapping_over_many_tiles():
     fwd, _, ws = g.plan()
     out = emu.run_tp(g, fwd, X, Y, ow.e3nn_to_oeq(oprob, We), ws_bytes=ws())
     assert rel_err(out["Z"], otp.forward(oprob, X, Y, We)) < TOL
-
-
-@pytest.mark.parametrize("dtype,a,n", [(np.float32, ("5x0e+21x1o", "1x0e+1x1o+1x2e", "18x0e+7x1o+3x2e"), 21),
-                                       (np.float64, ("16x0e+16x1o+4x2e", "1x0e+1x1o", "16x0e+20x1o"), 16),
-                                       (np.float32, ("3x0e+2x1o+1x2e", "1x0e+1x1o", "4x0e+4x1o+4x1e+4x2e+2x2o"), 35)])
-def test_uvw_forward_with_the_x_tile_in_lds(dtype, a, n, monkeypatch):
-    """One workgroup per batch tile, one wavefront per output block, X read through LDS (vector fill when the
-    row length allows it, element-wise otherwise; last tile partial)."""
-    monkeypatch.setenv("OEQ_AMD_UVW_FWD_LDS", "1")
-    prob, oprob = common.fully_connected(a, shared=True, dtype=dtype)
-    g = UVWGenerator(prob)
-    assert g.fwd_lds and g.fwd_waves == len(g.fwd_items)
-    X, Y, We, _ = common.tp_inputs(prob, n, 11, dtype, w_scale=0.3)
-    W = ow.e3nn_to_oeq(oprob, We)
-    fwd, _, ws = g.plan()
-    assert fwd[1]["num_threads"] == 64 * g.fwd_waves and fwd[1]["grid_y"] == 1
-    out = emu.run_tp(g, fwd, X, Y, W, ws_bytes=ws())
-    assert rel_err(out["Z"], otp.forward(oprob, X, Y, We)) < (TOL if dtype == np.float32 else 1e-13)
 
 
 @pytest.mark.parametrize("shared", [False, True])

@@ -83,11 +83,25 @@ def test_conv_outputs_of_either_parity(cuda, which, deterministic):
         _run(prob, oprob, 30, 400, 38, deterministic, sh_lmax=3)
 
 
-@pytest.mark.parametrize("deterministic", [False, True])
-def test_mace_conv_backward_split_over_output_blocks(cuda, deterministic):
-    """The MACE problem as a convolution: 104 registers of operands per edge, so the backward runs as two
-    launches over two groups of output blocks (the second adds to dX; dY through per-group partials)."""
+def test_mace_conv_deterministic_backward_defaults_to_receiver_order(cuda):
+    """A dZ row of the MACE problem is 7.9 times as long as an X row: the static rule picks the two-pass
+    receiver-order backward (config 3 and 5, ratios 3.9 and 4.8, keep the sender order)."""
+    from openequivariance_amd.codegen.uvu_recv import UVURecvGenerator
     from openequivariance_amd.conv import select_conv_generator
+    assert isinstance(select_conv_generator(common.channelwise(common.MACE)[0], True), UVURecvGenerator)
+    for irreps in (common.NEQUIP, common.LARGE):
+        assert not isinstance(select_conv_generator(common.channelwise(irreps)[0], True), UVURecvGenerator)
+    prob, oprob = common.channelwise(common.MACE)
+    _run(prob, oprob, 60, 900, 40, True, sh_lmax=3)
+
+
+@pytest.mark.parametrize("deterministic", [False, True])
+def test_mace_conv_backward_split_over_output_blocks(cuda, deterministic, monkeypatch):
+    """The MACE problem as a convolution in sender order: 104 registers of operands per edge, so the backward
+    runs as two launches over two groups of output blocks (the second adds to dX; dY through per-group partials)."""
+    from openequivariance_amd import tunables
+    from openequivariance_amd.conv import select_conv_generator
+    monkeypatch.setattr(tunables.current, "det_backward", "send")
     prob, oprob = common.channelwise(common.MACE)
     gen = select_conv_generator(prob, True)
     assert gen.H == 2 and sorted(sum(gen.out_groups, [])) == gen.used_out
@@ -96,11 +110,12 @@ def test_mace_conv_backward_split_over_output_blocks(cuda, deterministic):
 
 @pytest.mark.parametrize("which", ["nequip", "large", "mace", "ragged"])
 def test_receiver_order_backward(cuda, which, monkeypatch):
-    """The two-pass backward of the deterministic variant (OEQ_AMD_DET_BACKWARD=recv): parity, and
-    bit-equal repeats."""
+    """The two-pass backward of the deterministic variant (forced for every shape here; by itself it is
+    chosen for rows of dZ at least seven times as long as rows of X): parity, and bit-equal repeats."""
     import torch
+    from openequivariance_amd import tunables
     from openequivariance_amd.codegen.uvu_recv import UVURecvGenerator
-    monkeypatch.setenv("OEQ_AMD_DET_BACKWARD", "recv")
+    monkeypatch.setattr(tunables.current, "det_backward", "recv")
     irreps = {"nequip": common.NEQUIP, "large": common.LARGE, "mace": common.MACE,
               "ragged": ("5x0e+3x1o+70x2e", "1x0e+1x1o+1x2e", "5x0e+3x1o+70x2e+7x3o")}[which]
     prob, oprob = common.channelwise(irreps)

@@ -118,11 +118,11 @@ def test_edges_naming_no_node_contribute_nothing(cuda, variant, irreps, monkeypa
     import torch
     import openequivariance_amd as oeq
     from oracle import tp as otp
-    monkeypatch.setenv("OEQ_AMD_AUTOTUNE", "0")
-    if variant == "det_recv":
-        monkeypatch.setenv("OEQ_AMD_DET_BACKWARD", "recv")
+    from openequivariance_amd import tunables
+    monkeypatch.setattr(tunables.current, "autotune", False)
+    monkeypatch.setattr(tunables.current, "det_backward", "recv" if variant == "det_recv" else "send")
     if variant.startswith("unsorted"):
-        monkeypatch.setenv("OEQ_AMD_CONV_BACKWARD", variant.split("_")[1])
+        monkeypatch.setattr(tunables.current, "conv_backward", variant.split("_")[1])
     deterministic = variant.startswith("det")
     prob, oprob = common.channelwise(irreps)
     nodes, nnz = 40, 900

@@ -1,7 +1,8 @@
-"""The convolution reuses the graph preparation (CSR pointers, position lists, node order) that a
-call leaves in its workspace while the index tensors are unchanged, and rebuilds it when they change:
-in place (version counter), by new tensors, or by sizes.  Also: int32 index tensors, per-stream
-workspaces, and the raw entry points' ``prepared`` flag."""
+"""With ``graph_cache=True`` the convolution reuses the graph preparation (CSR pointers, position lists,
+node order) that a call leaves in its workspace while the index tensors are unchanged, and rebuilds it
+when they change: in place (version counter), by new tensors, or by sizes.  By default it prepares the
+graph on every call, so writes that torch's version counter cannot see are always picked up.  Also: int32
+index tensors, per-stream workspaces, and the raw entry points' ``prepared`` flag."""
 import numpy as np
 import pytest
 
@@ -45,7 +46,7 @@ def test_preparation_is_reused_and_rebuilt(cuda, deterministic, irreps):
     import torch
     import openequivariance_amd as oeq
     prob, oprob = common.channelwise(irreps)
-    conv = oeq.TensorProductConv(prob, torch_op=True, deterministic=deterministic)
+    conv = oeq.TensorProductConv(prob, torch_op=True, deterministic=deterministic, graph_cache=True)
     nodes, nnz = 60, 900
     host, graph, t, index, g = _inputs(prob, nodes, nnz, 5, deterministic, cuda)
     rec = lambda: conv._workspace_record(nnz, nodes)
@@ -73,15 +74,30 @@ def test_preparation_is_reused_and_rebuilt(cuda, deterministic, irreps):
     _check(oprob, host, graph2, conv, t, index, g)
 
 
-def test_cache_can_be_switched_off(cuda, monkeypatch):
+@pytest.mark.parametrize("deterministic", [True, False])
+def test_cache_is_off_by_default_and_sees_writes_behind_torchs_back(cuda, deterministic):
+    """The default operator prepares the graph on every call.  The index tensors are rewritten through an
+    alias that does not bump their version counter (a view made by from_dlpack of the same memory: the
+    hazard of neighbour lists written by another library): results must follow the new contents.  The same
+    alias goes unnoticed by an operator built with graph_cache=True, which is why that is opt-in."""
+    import torch
     import openequivariance_amd as oeq
-    monkeypatch.setenv("OEQ_AMD_GRAPH_CACHE", "0")
+    from openequivariance_amd import tunables
+    assert tunables.current.graph_cache is False
     prob, oprob = common.channelwise(common.NEQUIP)
-    conv = oeq.TensorProductConv(prob, torch_op=True, deterministic=True)
-    host, graph, t, index, g = _inputs(prob, 40, 500, 8, True, cuda)
+    conv = oeq.TensorProductConv(prob, torch_op=True, deterministic=deterministic)
+    assert conv.graph_cache is False
+    nodes, nnz = 40, 500
+    host, graph, t, index, g = _inputs(prob, nodes, nnz, 8, deterministic, cuda)
     _check(oprob, host, graph, conv, t, index, g)
-    _check(oprob, host, graph, conv, t, index, g)
-    assert conv._workspace_record(500, 40).fwd_key is None
+    assert conv._workspace_record(nnz, nodes).fwd_key is None
+    _, graph2, _, index2, _ = _inputs(prob, nodes, nnz, 9, deterministic, cuda)
+    versions = [i._version for i in index]
+    for dst, src in zip(index, index2):
+        torch.utils.dlpack.from_dlpack(torch.utils.dlpack.to_dlpack(dst)).copy_(src)
+    torch.cuda.synchronize()
+    assert [i._version for i in index] == versions, "the alias must not bump the version counters"
+    _check(oprob, host, graph2, conv, t, index, g)           # fresh results from the rewritten edge list
 
 
 @pytest.mark.parametrize("deterministic", [True, False])
@@ -158,8 +174,9 @@ def test_unsorted_backward_variant_is_chosen_by_measurement(cuda, monkeypatch):
     """The first backward call of a size class times the atomic and the grouped backward on the caller's
     tensors and keeps the faster; both give the oracle's gradients; overrides switch the timing off."""
     import openequivariance_amd as oeq
-    monkeypatch.delenv("OEQ_AMD_CONV_BACKWARD", raising=False)
-    monkeypatch.delenv("OEQ_AMD_AUTOTUNE", raising=False)
+    from openequivariance_amd import tunables
+    monkeypatch.setattr(tunables.current, "conv_backward", None)
+    monkeypatch.setattr(tunables.current, "autotune", True)
     prob, oprob = common.channelwise(common.NEQUIP)
     conv = oeq.TensorProductConv(prob, torch_op=True, deterministic=False)
     assert conv.autotune and conv._bwd_default == "grouped"
@@ -174,6 +191,6 @@ def test_unsorted_backward_variant_is_chosen_by_measurement(cuda, monkeypatch):
     for name in ("atomic", "grouped"):                       # either variant, forced, against the oracle
         conv._bwd_choice = {k: name for k in conv._bwd_choice}
         _check(oprob, host, graph, conv, t, index, g)
-    monkeypatch.setenv("OEQ_AMD_AUTOTUNE", "0")
+    monkeypatch.setattr(tunables.current, "autotune", False)
     assert not oeq.TensorProductConv(prob, torch_op=True, deterministic=False).autotune
     assert not oeq.TensorProductConv(prob, torch_op=True, deterministic=True).autotune

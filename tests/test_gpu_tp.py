@@ -57,16 +57,6 @@ def test_mace_uvu(cuda, n):
     _run(prob, oprob, n, 2, np.float32, sh_lmax=3)
 
 
-@pytest.mark.parametrize("waves,dtype", [(4, np.float32), (2, np.float64)])
-def test_mace_uvu_row_dealt_to_several_wavefronts(cuda, waves, dtype, monkeypatch):
-    """The variant with 2 / 4 wavefronts per row (contiguous parts of the Z / dZ row each, dX and dY combined
-    through LDS); off by default, kept measurable."""
-    monkeypatch.setenv("OEQ_AMD_TP_ROW_WAVES", str(waves))
-    prob, oprob = common.channelwise(common.MACE, dtype=dtype)
-    tp = _run(prob, oprob, 70, 21, dtype, sh_lmax=3)
-    assert tp.generator.row_waves == waves
-
-
 def test_nequip_uvu_two_rows_per_wave(cuda):
     """mul 32: two rows share a wavefront; odd batch leaves a half-empty tile."""
     prob, oprob = common.channelwise(common.NEQUIP)

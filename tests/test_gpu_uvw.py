@@ -84,6 +84,33 @@ def test_dw_bit_reproducible_and_full_batch(cuda):
     assert rel_err(z.detach()[sl].cpu().numpy(), otp.forward(oprob, X[sl], Y[sl], We_)) <= FP32_TOL
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_full_batch_dw_element_wise(cuda, dtype):
+    """dW of the full config-4 batch (100 000 rows) element by element against the oracle's dW accumulated in
+    fp64 over chunks of rows on the CPU, plus the last rows of Z, dX and dY against the oracle."""
+    import torch
+    import openequivariance_amd as oeq
+    tol = FP32_TOL if dtype == np.float32 else FP64_TOL
+    prob, oprob = common.fully_connected(common.DENSE, shared=True, dtype=dtype)
+    n = 100000
+    X, Y, We, G = common.tp_inputs(prob, n, 12349, dtype, 2, w_scale=0.125)
+    tp = oeq.TensorProduct(prob, torch_op=True)
+    W = ow.e3nn_to_oeq(oprob, We)
+    x, y, w = (torch.tensor(a, device=cuda, requires_grad=True) for a in (X, Y, W))
+    z = tp(x, y, w)
+    z.backward(torch.tensor(G, device=cuda))
+    torch.cuda.synchronize()
+    dWr = otp.shared_weight_gradient(oprob, X, Y, G)
+    errs = dict(dW=rel_err(ow.oeq_to_e3nn(oprob, w.grad.cpu().numpy()), dWr))
+    sl = slice(n - 24, n)
+    dXr, dYr, _ = otp.backward(oprob, X[sl], Y[sl], We, G[sl])
+    errs.update(Z=rel_err(z.detach()[sl].cpu().numpy(), otp.forward(oprob, X[sl], Y[sl], We)),
+                dX=rel_err(x.grad[sl].cpu().numpy(), dXr), dY=rel_err(y.grad[sl].cpu().numpy(), dYr))
+    print(f"n={n} {np.dtype(dtype).name} {errs}", flush=True)
+    for k, v in errs.items():
+        assert v <= tol, f"{k}: relative error {v:.3e} > {tol}"
+
+
 def test_uvw_tensors_beyond_two_giga_elements(cuda):
     """3.8 M rows of the config-4 problem: X, Z and their gradients have more than 2^31 elements each.
     Sampled rows (start, around element 2^31, end) of Z, dX, dY against the oracle; dW, which sums over
@@ -143,8 +170,6 @@ def test_uvw_several_copies_of_the_second_operand(cuda, name, shared, dtype):
     loop_unroll_tp.cuh:48-60 walks v)."""
     import torch
     import openequivariance_amd as oeq
-    if name.startswith("ragged") and dtype == np.float64 and not shared:
-        pytest.skip("same code path as fp32, 38 per-row weight matrices of 8-byte words")
     tol = FP32_TOL if dtype == np.float32 else FP64_TOL
     prob, oprob = common.fully_connected(UVW_MUL2[name], shared=shared, dtype=dtype)
     n = 37

@@ -109,7 +109,8 @@ def test_staged_conv_selection(monkeypatch):
     whose stage leaves room for three wavefronts per SIMD; other problems keep the register pipeline."""
     from openequivariance_amd.codegen.uvu_det import UVUDetGenerator
     from openequivariance_amd.problem import ChannelwiseTPP
-    monkeypatch.delenv("OEQ_AMD_DET_LDS", raising=False)
+    from openequivariance_amd import tunables
+    monkeypatch.setattr(tunables.current, "det_lds", None)
     small = UVUDetGenerator(ChannelwiseTPP("32x0e+32x1o+32x2e", "1x0e+1x1o+1x2e", "32x0e+32x1o+32x2e"))
     assert small.lds_forward and small.lds_backward and 12 * small.stage_words * 4 <= 160 * 1024
     large = UVUDetGenerator(ChannelwiseTPP("256x0e+256x1o+256x2e", "1x0e+1x1o+1x2e+1x3o", "256x0e+256x1o+256x2e"))
@@ -126,7 +127,8 @@ def test_unsorted_conv_backward_selection(monkeypatch):
     128 values per edge on."""
     from openequivariance_amd.codegen.uvu_sorted import UVUSortedGenerator
     from openequivariance_amd.problem import ChannelwiseTPP
-    monkeypatch.delenv("OEQ_AMD_CONV_BACKWARD", raising=False)
+    from openequivariance_amd import tunables
+    monkeypatch.setattr(tunables.current, "conv_backward", None)
     small = UVUSortedGenerator(ChannelwiseTPP("8x0e+8x1o+8x2e", "1x0e+1x1o+1x2e", "8x0e+8x1o+8x2e"))
     assert UVUSortedGenerator(ChannelwiseTPP("32x0e+32x1o+32x2e", "1x0e+1x1o+1x2e", "32x0e+32x1o+32x2e")).grouped_backward
     large = UVUSortedGenerator(ChannelwiseTPP("256x0e+256x1o+256x2e", "1x0e+1x1o+1x2e+1x3o", "256x0e+256x1o+256x2e"))

@@ -97,6 +97,28 @@ def test_backward_against_torch_autograd_and_adjoint_identity(name):
         assert float((a * g).sum()) == pytest.approx(gz, rel=1e-11)
 
 
+@pytest.mark.parametrize("name", ["uvw_shared", "uvu_shared_v2", "dense"])
+def test_shared_weight_gradient_against_backward_and_finite_differences(name):
+    """The chunked dW-only routine (used where the full backward is too slow) against ``backward`` on a
+    batch that spans several chunks with a ragged last one, and against a central finite difference."""
+    prob = {"uvw_shared": PROBLEMS["uvw_shared"],
+            "uvu_shared_v2": lambda: spec.Problem("3x0e+3x1o", "2x0e+2x1o", "3x0e+3x1o",
+                                                  [(0, 0, 0, "uvu", True), (1, 1, 0, "uvu", True), (1, 0, 1, "uvu", True)],
+                                                  shared_weights=True),
+            "dense": lambda: spec.fully_connected(*common.DENSE, shared_weights=True)}[name]()
+    X, Y, W, G = _inputs(prob, 23, 5)
+    dW = otp.shared_weight_gradient(prob, X, Y, G, chunk=7)
+    np.testing.assert_allclose(dW, otp.backward(prob, X, Y, W, G)[2], rtol=1e-12, atol=1e-12)
+    rng = np.random.default_rng(6)
+    h = 1e-6
+    for _ in range(4):
+        q = int(rng.integers(0, prob.weight_numel))
+        plus, minus = W.copy(), W.copy()
+        plus[q] += h; minus[q] -= h
+        fd = float(((otp.forward(prob, X, Y, plus) - otp.forward(prob, X, Y, minus)) * G).sum()) / (2 * h)
+        assert dW[q] == pytest.approx(fd, rel=1e-6, abs=1e-7)
+
+
 def test_equivariance_under_rotation_and_inversion():
     """Z(D1 x, D2 y) = D3 Z(x, y) with Wigner matrices generated from the coupling tensors' own
     invariance generators (rotation) and parity signs (inversion)."""
