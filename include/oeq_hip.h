@@ -61,13 +61,22 @@ int  oeq_hiprtc_version(int* major, int* minor);
 /* -------------------------------------------------------------- launch plan */
 /* One kernel launch of an operator.  Replaces KernelLaunchConfig
  * (extension/util/backend_hip.hpp:123-133) and adds how the grid follows the work size. */
-enum { OEQ_GRID_FIXED = 0, OEQ_GRID_PER_ROW = 1, OEQ_GRID_PER_NODE = 2 };
+/* OEQ_GRID_PER_NODE_AND_PIECE: one workgroup per `work_per_block` nodes followed by two per tile of
+ * T = max(OEQ_PIECE_MIN_EDGES, num_blocks * ceil(nnz / node_count)) consecutive positions of the edge
+ * list; `num_blocks` holds the long-node factor instead of a bound (0: no piece workgroups).  The
+ * extra workgroups walk the pieces of nodes whose edge list is longer than T, so that a hub does not
+ * serialise one wavefront (the reference deals the edge list to its warps in equal shares and repairs
+ * the seams: templates/loop_unroll_conv_det.cuh:33-133). */
+enum { OEQ_GRID_FIXED = 0, OEQ_GRID_PER_ROW = 1, OEQ_GRID_PER_NODE = 2, OEQ_GRID_PER_NODE_AND_PIECE = 3 };
+#define OEQ_PIECE_MIN_EDGES 32u
 /* What a step dereferences and what it is for.  A call whose plan holds a step with
  * OEQ_STEP_NEEDS_WORKSPACE (OEQ_STEP_NEEDS_TPERM) is rejected, before anything is launched, when the
  * workspace (transpose permutation) pointer is NULL.  OEQ_STEP_GRAPH_PREP marks the steps that only
  * derive graph structure (CSR pointers, position lists, node order) from rows / cols /
- * transpose_perm into the workspace: the *_prepared entry points skip them. */
-enum { OEQ_STEP_NEEDS_WORKSPACE = 1, OEQ_STEP_NEEDS_TPERM = 2, OEQ_STEP_GRAPH_PREP = 4 };
+ * transpose_perm into the workspace: a call with OEQ_CALL_PREPARED skips them.  OEQ_STEP_COUNTER_CLEAR
+ * marks a step that only zeroes counters in the workspace which the operator's later steps leave
+ * zeroed again: a call with OEQ_CALL_COUNTERS_ZERO skips it. */
+enum { OEQ_STEP_NEEDS_WORKSPACE = 1, OEQ_STEP_NEEDS_TPERM = 2, OEQ_STEP_GRAPH_PREP = 4, OEQ_STEP_COUNTER_CLEAR = 8 };
 typedef struct {
     char     kernel[64];        /* extern "C" symbol in the code object */
     uint32_t num_threads;       /* workgroup size */
@@ -127,27 +136,43 @@ int  oeq_conv_backward(oeq_conv* conv, const void* L1_in, void* L1_grad, const v
                        const void* rows, const void* cols, uint64_t nnz, uint64_t node_count,
                        void* workspace, const void* transpose_perm, void* stream);
 
-/* The same two calls for a workspace that already holds this graph's preparation: the steps flagged
- * OEQ_STEP_GRAPH_PREP are skipped.  Valid only if the last oeq_conv_forward (for _forward_prepared) /
- * oeq_conv_backward (for _backward_prepared) that used this workspace ran with the same rows, cols,
- * transpose_perm contents, nnz and node_count, and nothing else has written the workspace's
- * preparation areas since (forward and backward keep theirs in disjoint parts of the workspace).  A
- * model calls one graph for the forward, the backward and the seven launches of the double backward
- * of every layer; the reference allocates its workspace once and rebuilds nothing either
- * (implementations/convolution/ConvolutionBase.py:93-100). */
-int  oeq_conv_forward_prepared(oeq_conv* conv, const void* L1_in, const void* L2_in, const void* weights,
-                               void* L3_out, const void* rows, const void* cols, uint64_t nnz,
-                               uint64_t node_count, void* workspace, const void* transpose_perm, void* stream);
-int  oeq_conv_backward_prepared(oeq_conv* conv, const void* L1_in, void* L1_grad, const void* L2_in,
-                                void* L2_grad, const void* weights, void* weights_grad, const void* L3_grad,
-                                const void* rows, const void* cols, uint64_t nnz, uint64_t node_count,
-                                void* workspace, const void* transpose_perm, void* stream);
+/* The same two calls with what the caller knows about the workspace (OEQ_CALL_* flags, or 0).
+ * OEQ_CALL_PREPARED: the workspace already holds this graph's preparation; the steps flagged
+ * OEQ_STEP_GRAPH_PREP are skipped.  Valid only if the last forward (for _forward_ex) / backward (for
+ * _backward_ex) call that used this workspace ran with the same rows, cols, transpose_perm contents,
+ * nnz and node_count, and nothing else has written the workspace's preparation areas since (forward
+ * and backward keep theirs in disjoint parts of the workspace).  A model calls one graph for the
+ * forward, the backward and the seven launches of the double backward of every layer; the reference
+ * allocates its workspace once and rebuilds nothing either
+ * (implementations/convolution/ConvolutionBase.py:93-100).
+ * OEQ_CALL_COUNTERS_ZERO: the counters that the operator keeps in the workspace are zero: the workspace
+ * was zero-filled, or the last call that used it was a completed call of this operator with the same
+ * node_count, and nothing else has written it since.  The steps flagged OEQ_STEP_COUNTER_CLEAR are
+ * skipped (every call leaves its counters zeroed). */
+enum { OEQ_CALL_PREPARED = 1, OEQ_CALL_COUNTERS_ZERO = 2 };
+int  oeq_conv_forward_ex(oeq_conv* conv, const void* L1_in, const void* L2_in, const void* weights,
+                         void* L3_out, const void* rows, const void* cols, uint64_t nnz,
+                         uint64_t node_count, void* workspace, const void* transpose_perm, void* stream,
+                         uint32_t call_flags);
+int  oeq_conv_backward_ex(oeq_conv* conv, const void* L1_in, void* L1_grad, const void* L2_in,
+                          void* L2_grad, const void* weights, void* weights_grad, const void* L3_grad,
+                          const void* rows, const void* cols, uint64_t nnz, uint64_t node_count,
+                          void* workspace, const void* transpose_perm, void* stream, uint32_t call_flags);
+
+/* Workspace bytes the forward steps use when every node is walked by one wavefront (no pieces):
+ * fixed_bytes + bytes_per_node * node_count + bytes_per_edge * nnz.  The host sets it from the plan it
+ * built the operator with; oeq_conv_forward_noalloc checks graphs against it.  (The reference sizes
+ * its workspace on the Python side as well: implementations/convolution/LoopUnrollConv.py:61-72.) */
+int  oeq_conv_set_forward_workspace(oeq_conv* conv, uint64_t fixed_bytes, uint64_t bytes_per_node,
+                                    uint64_t bytes_per_edge);
 
 /* oeq_conv_forward for callers that cannot allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
  * The workspace is a static device array of OEQ_NOALLOC_SCRATCH_BYTES inside the library (one copy
  * per GPU, held until the process ends); the call allocates and frees nothing.  The forward kernels
- * use 8 * (2 * (node_count + 1) + nnz) bytes of it; larger graphs are rejected with an error.  All
+ * use what oeq_conv_set_forward_workspace declared (every node is walked by one wavefront here: the
+ * pieces of long nodes would need partial rows beyond a static array); larger graphs are rejected
+ * with an error.  All
  * calls on one GPU share the array: calls that overlap in time on one GPU (different streams or
  * threads) race on it, and a captured graph holding such a call must not replay concurrently with
  * another.  Inputs and outputs are the caller's, as in oeq_conv_forward. */

@@ -37,10 +37,18 @@ from .uvu_direct import UVUDirectGenerator
 class UVUDetGenerator(UVUDirectGenerator):
     _allow_det = True
     SPLIT_WORDS = 80
+    # int64 words of one on-the-fly grouping of the edges in the workspace: group pointers and fill cursors
+    # (node_count + 1 each), the position list (nnz), the counters (node_count + 1) and the ticket of the
+    # counting kernel
+    GROUP_WORDS = "(3 * (node_count + 1) + nnz + 1)"
+
+    @staticmethod
+    def group_bytes(nnz: int, nodes: int) -> int:
+        return (3 * (nodes + 1) + nnz + 1) * 8
 
     def __init__(self, problem: TPProblem, prefetch_backward=None, vector_stores: bool = True,
                  forward_perm: bool = False, backward_perm: bool = False, idx_ctype: str = "i64",
-                 allow_split: bool = True, lds=None):
+                 allow_split: bool = True, lds=None, long_node=None):
         super().__init__(problem, "conv_det", vector_stores=vector_stores)
         self.idx_ctype = idx_ctype
         # True: the forward walks the receiver-grouped edge order listed in the workspace (built on
@@ -56,12 +64,12 @@ class UVUDetGenerator(UVUDirectGenerator):
         self.ordered_backward = True
         extra = " + node_count"
         if backward_perm:
-            # behind the forward's grouping (pointers | cursors | position list), so that both stay valid
-            # side by side and a graph prepared once serves forward and backward calls alike
-            base = "(2 * (node_count + 1) + nnz)"
+            # behind the forward's grouping (pointers | cursors | position list | counters | ticket), so that
+            # both stay valid side by side and a graph prepared once serves forward and backward calls alike
+            base = self.GROUP_WORDS
             self.bwd_ptr_off = base
             self.bwd_list = f"((const i64*)ws + {base} + 2 * (node_count + 1))"
-            self.bwd_order = f"((const i64*)ws + {base} + 2 * (node_count + 1) + nnz)"
+            self.bwd_order = f"((const i64*)ws + 2 * {base})"
             self.dypart_off = f"(2 * {base}{extra}) * sizeof(i64)"
         else:
             self.bwd_ptr_off = "(node_count + 1)"
@@ -126,6 +134,17 @@ class UVUDetGenerator(UVUDirectGenerator):
                             and 16 * (fwd_words + self.lds_elems) * 4 <= 160 * 1024)
         self.uniform_rows = False          # validity is per lane (edge lists differ between sub-rows)
         self.chunk_in_grid = True
+        # A node whose edge list is longer than LONG times the mean (at least PIECE_MIN_EDGES) is not walked
+        # by its own wavefront: the edge list is cut at multiples of that length, and every piece of a long
+        # node is walked by one of the wavefronts launched behind the nodes (two per tile of the list: the
+        # piece of the long node that ends in the tile and of the one that begins in it).  A piece leaves its
+        # sums in a partial row of the workspace; the wavefront that finishes last (a counter per long node)
+        # adds the pieces in list order and writes the node's row, so the result does not depend on timing
+        # (reference: the edge list dealt to the warps in equal shares and a fix-up kernel for the seams,
+        # templates/loop_unroll_conv_det.cuh:33-133).  0: every node is walked by one wavefront.
+        self.LONG = max(0, int(tunables.current.long_node)) if long_node is None else int(long_node)
+        # byte offset (C expression) of the piece area in the workspace: counters, then partial rows
+        self.piece_base = f"((({self.flags_off} + 4ull * ((nnz + 255) / 256)) + 255ull) & ~255ull)"
 
     @contextlib.contextmanager
     def _group(self, h: int):
@@ -160,11 +179,50 @@ class UVUDetGenerator(UVUDirectGenerator):
         return "u"
 
     # ------------------------------------------------------------------ common
-    def _node_setup(self, E: Emitter, ptr_off: str, order: str = None) -> None:
-        """One node per wavefront.  With multiplicity <= 32 the wavefront's R = 64/P lane groups walk
-        interleaved sub-lists of the node's edges (edge beg + it*R + sub) and their partial sums are
-        combined in a fixed order at the end, which shortens the serial edge loop R-fold."""
+    PIECE_MIN_EDGES = 32          # OEQ_PIECE_MIN_EDGES of the C ABI
+    PIECE_GROUP = 32              # pieces added by one wavefront at the first level of a long node's sum
+
+    def piece_tiles(self, nnz: int, nodes: int) -> int:
+        """Tiles of the edge list (host mirror of oeq_piece_tiles in the kernels and of the launch grid)."""
+        if not self.LONG or nnz == 0 or nodes == 0:
+            return 0
+        t = max(self.PIECE_MIN_EDGES, self.LONG * (-(-nnz // nodes)))
+        return -(-nnz // t)
+
+    @property
+    def piece_row_words(self) -> int:
+        return max(self.D1, self.D3)
+
+    def piece_bytes(self, nnz: int, nodes: int) -> int:
+        """Counters (four ints per tile and chunk: group and node level of both slots) and partial rows (two
+        per tile) of the piece area."""
+        tiles = self.piece_tiles(nnz, nodes)
+        if tiles == 0:
+            return 0
+        return 256 + ((16 * self.NCH * tiles + 255) & ~255) + 2 * tiles * self.piece_row_words * self.itemsize
+
+    def emit_piece_helpers(self) -> str:
+        """Device functions shared by the kernels of one code object (rendered once by the templates)."""
+        return "\n".join([
+            "// edges per piece of a long node's list, and tiles of that length in the whole list",
+            "static __device__ __forceinline__ u64 oeq_piece_edges(u64 nnz, u64 node_count) {",
+            f"    const u64 t_ = {self.LONG}ull * (node_count ? (nnz + node_count - 1) / node_count : 0);",
+            f"    return t_ < {self.PIECE_MIN_EDGES}ull ? {self.PIECE_MIN_EDGES}ull : t_;",
+            "}",
+            "static __device__ __forceinline__ u64 oeq_piece_tiles(u64 nnz, u64 node_count) {",
+            "    const u64 t_ = oeq_piece_edges(nnz, node_count);",
+            f"    return {'(nnz + t_ - 1) / t_' if self.LONG else '0'};",
+            "}"])
+
+    def _node_setup(self, E: Emitter, ptr_off: str, order: str = None, key=None) -> None:
+        """One node per wavefront, or - for the wavefronts launched behind the nodes - one piece of a long
+        node's edge list.  With multiplicity <= 32 the wavefront's R = 64/P lane groups walk interleaved
+        sub-lists of the edges (edge beg + it*R + sub) and their partial sums are combined in a fixed order
+        at the end, which shortens the serial edge loop R-fold.  ``key(E, pos)`` emits statements that
+        set ``kv_`` (i64) to the node owning list position ``pos`` (anything out of range: not a node);
+        without it every node is walked whole."""
         R = self.R
+        self.pieces = bool(self.LONG and key)
         # The launch is ordered chunk by chunk (blockIdx.y): the wavefronts in flight then gather from one
         # chunk's share of X / dZ, a fraction of the tensor that the 256 MB Infinity Cache can hold.  Giving
         # the chunks of a node consecutive workgroup ids instead measured slower (256 channels: forward
@@ -172,21 +230,151 @@ class UVUDetGenerator(UVUDirectGenerator):
         E("const int c = blockIdx.y; (void)c;")
         E("const u64 bx_ = blockIdx.x;")
         E(f"const int u = c * {self.P} + ul;")
+        E(f"const i64* __restrict__ ptr = (const i64*)ws + {ptr_off};")
+        E("u64 node = node_count; i64 beg = 0, end = 0;")
+        if self.pieces:
+            E("// pieces are in use when the launch has wavefronts behind the nodes (the entry point that must not")
+            E("// allocate launches none: every node is then walked whole)")
+            E("const bool pieces_on = gridDim.x > node_count, piece = bx_ >= node_count;")
+            E("const u64 TL = oeq_piece_edges(nnz, node_count), tiles_ = oeq_piece_tiles(nnz, node_count);")
+            E("u64 slot = 0, qh = 0; int npieces = 0;")
+            E("if (!piece) {")
+            E.level += 1
         if order:
             E(f"const i64 nd_ = bx_ < node_count ? {order}[bx_] : -1;")
-            E("const u64 node = nd_ >= 0 ? (u64)nd_ : node_count;")
+            E("if (nd_ >= 0 && (u64)nd_ < node_count) node = (u64)nd_;")
         else:
-            E("const u64 node = bx_;")
-        E("const bool nv = node < node_count;")
-        E(f"const i64* __restrict__ ptr = (const i64*)ws + {ptr_off};")
-        E("i64 beg = 0, end = 0;")
-        E("if (nv && nnz > 0) { beg = ptr[node]; end = ptr[node + 1]; }")
+            E("if (bx_ < node_count) node = bx_;")
+        E("if (node < node_count && nnz > 0) { beg = ptr[node]; end = ptr[node + 1]; }")
         E("if (beg < 0) beg = 0;")
         E("if (end > (i64)nnz) end = (i64)nnz;")
         E("if (end < beg) end = beg;")
+        if self.pieces:
+            E("if (pieces_on && (u64)(end - beg) > TL) { node = node_count; end = beg; }     // a long node: walked in pieces, see below")
+            E.level -= 1
+            E("} else {")
+            E.level += 1
+            E("const u64 w_ = bx_ - node_count, q_ = w_ >> 1; const bool head_ = (w_ & 1) != 0;")
+            E("const u64 a0_ = q_ * TL, a1_ = min(a0_ + TL, nnz);")
+            E("if (a0_ < nnz) {")
+            E.level += 1
+            E("i64 kv_ = -1;")
+            key(E, "(head_ ? a1_ - 1 : a0_)")
+            E("if (kv_ >= 0 && kv_ < (i64)node_count) {")
+            E.level += 1
+            E("i64 b_ = ptr[kv_], e_ = ptr[kv_ + 1];")
+            E("if (b_ < 0) b_ = 0;")
+            E("if (e_ > (i64)nnz) e_ = (i64)nnz;")
+            E("if (e_ < b_) e_ = b_;")
+            E("// the tile's head piece belongs to the long node that begins in it, the other to the one that began before it")
+            E("if ((u64)(e_ - b_) > TL && (head_ ? (u64)b_ >= a0_ : (u64)b_ < a0_)) {")
+            E("    node = (u64)kv_; beg = head_ ? b_ : (i64)a0_; end = min(e_, (i64)a1_); slot = w_;")
+            E("    qh = (u64)b_ / TL; npieces = (int)((u64)(e_ - 1) / TL - qh) + 1;")
+            E("}")
+            E.level -= 1
+            E("}")
+            E.level -= 1
+            E("}")
+            E.level -= 1
+            E("}")
+        E("const bool nv = node < node_count;")
         E("const int len = (int)(end - beg);")
         E(f"const int maxlen = (len + {R - 1}) / {R};")
         self.noderow_of = (lambda r: ("node", "nv"))
+
+    def emit_node_output(self, E: Emitter, blocks, used, regs_of, ptr: str, rowdim: int, via_lds: bool,
+                         zero_unused: bool, add_existing: bool) -> None:
+        """The sums a wavefront holds for its node (registers ``regs_of(block)`` of the blocks in ``used``) ->
+        row ``node`` of ``ptr``; blocks nothing contributes to are zero-filled (``zero_unused``); with
+        ``add_existing`` the row already holds the sums of an earlier launch and is added to.  A piece
+        stores its sums in its partial row instead; the piece of a node that finishes last adds all pieces
+        in list order and writes the node's row."""
+        for blk in blocks:
+            if blk.idx in used and blk.dim:
+                self.emit_sub_sum(E, regs_of(blk))
+
+        def store(E, base: str, row: str, existing: bool, zero: bool):
+            for blk in blocks:
+                if blk.dim == 0:
+                    continue
+                E("{")
+                E.level += 1
+                dst = f"{base} + {row} * {rowdim} + {blk.off} + u * {blk.D}"
+                if blk.idx in used and self.R == 1 and via_lds:
+                    self.emit_block_store(E, blk, regs_of(blk), base, rowdim, row, (lambda r: (row, "nv")), "store",
+                                          via_lds=True)
+                elif blk.idx in used:
+                    if existing:            # the launches of the earlier groups have written this row: add to it
+                        E(f"if ({self.store_act(blk)}) {{ const T* __restrict__ q_ = {dst}; "
+                          + " ".join(f"{n} += q_[{m}];" for m, n in enumerate(regs_of(blk))) + " }")
+                    self.emit_record_store(E, regs_of(blk), dst, self.store_act(blk))
+                elif zero:
+                    self.emit_record_store(E, ["(T)0"] * blk.D, dst, self.store_act(blk))
+                E.level -= 1
+                E("}")
+        if not self.pieces:
+            store(E, ptr, "node", add_existing, zero_unused)
+            return
+        G = self.PIECE_GROUP
+        E("if (!piece) {")
+        E.level += 1
+        store(E, ptr, "node", add_existing, zero_unused)
+        E.level -= 1
+        E("} else if (nv) {")
+        E.level += 1
+        E("// counters: one per slot for the groups of pieces, one per slot for the whole node")
+        E(f"int* __restrict__ tk_ = (int*)((char*)ws + {self.piece_base}) + (u64)c * 4 * tiles_;")
+        E(f"T* __restrict__ prow_ = (T*)((char*)ws + {self.piece_base} + ((16ull * {self.NCH} * tiles_ + 255ull) & ~255ull) + 256ull);")
+        store(E, "prow_", "slot", False, False)
+        E(f"// Piece k of the node sits in slot 2 qh + 1 (k = 0) or 2 (qh + k).  The pieces are added in two levels, each")
+        E(f"// by whoever finishes last: groups of {G} consecutive pieces in list order (the sum replaces the group's first")
+        E(f"// piece), then the groups in order.  Which wavefront adds does not change what is added in which order.")
+        E(f"const int k_own_ = slot == 2 * qh + 1 ? 0 : (int)(slot / 2 - qh);")
+        E(f"int first_ = (k_own_ / {G}) * {G}, cnt_ = min({G}, npieces - first_), stride_ = 1, level_ = 0;")
+        E("oeq_release_agent();")
+        E("int old_ = 0;")
+        E("if (lane == 0) old_ = oeq_ticket_add(tk_ + (first_ == 0 ? 2 * qh + 1 : 2 * (qh + (u64)first_)));")
+        E("old_ = __builtin_amdgcn_readfirstlane(old_);")
+        E("bool go_ = old_ == cnt_ - 1;")
+        E("while (go_) {")
+        E.level += 1
+        E("oeq_acquire_agent();")
+        for blk in blocks:
+            if blk.idx in used and blk.dim:
+                E(" ".join(f"{n} = (T)0;" for n in regs_of(blk)))
+        E("for (int i_ = 0; i_ < cnt_; ++i_) {")
+        E.level += 1
+        E("const int kk_ = first_ + i_ * stride_;")
+        E("const u64 srow_ = kk_ == 0 ? 2 * qh + 1 : 2 * (qh + (u64)kk_);")
+        for blk in blocks:
+            if blk.idx in used and blk.dim:
+                E(f"{{ const T* __restrict__ q_ = prow_ + srow_ * {rowdim} + {blk.off} + {self.uclamp(blk, 0)} * {blk.D}; "
+                  + " ".join(f"{n} += q_[{m}];" for m, n in enumerate(regs_of(blk))) + " }")
+        E.level -= 1
+        E("}")
+        E("const u64 grow_ = first_ == 0 ? 2 * qh + 1 : 2 * (qh + (u64)first_);       // slot of the group's first piece")
+        E(f"if (level_ == 1 || npieces <= {G}) {{")
+        E.level += 1
+        store(E, ptr, "node", add_existing, zero_unused)
+        E("if (lane == 0) tk_[level_ == 1 ? 2 * tiles_ + 2 * qh + 1 : grow_] = 0;")
+        E("go_ = false;")
+        E.level -= 1
+        E("} else {")
+        E.level += 1
+        store(E, "prow_", "grow_", False, False)
+        E("if (lane == 0) tk_[grow_] = 0;")
+        E("oeq_release_agent();")
+        E("old_ = 0;")
+        E("if (lane == 0) old_ = oeq_ticket_add(tk_ + 2 * tiles_ + 2 * qh + 1);")
+        E("old_ = __builtin_amdgcn_readfirstlane(old_);")
+        E(f"first_ = 0; cnt_ = (npieces + {G - 1}) / {G}; stride_ = {G}; level_ = 1;")
+        E("go_ = old_ == cnt_ - 1;")
+        E.level -= 1
+        E("}")
+        E.level -= 1
+        E("}")
+        E.level -= 1
+        E("}")
 
     def ld(self, ptr: str, idx) -> str:
         return f"oeq_ldnt({ptr} + {idx})" if self.nontemporal else f"{ptr}[{idx}]"
@@ -221,7 +409,7 @@ class UVUDetGenerator(UVUDirectGenerator):
     def backward_steps(self):
         """Launches of the segmented backward behind the pointer / position-list preparation."""
         steps = [self.order_step()] if self.ordered_backward else []
-        steps += [dict(kernel=name, num_threads=64, grid_kind=2, work_per_block=1, grid_y=self.NCH)
+        steps += [dict(kernel=name, num_threads=64, grid_kind=3, work_per_block=1, num_blocks=self.LONG, grid_y=self.NCH)
                   for name, _ in self.backward_kernels()]
         if self.dy_slots > 1:
             steps.append(dict(kernel="backward_dy_reduce", num_threads=256, grid_kind=1,
@@ -273,20 +461,36 @@ class UVUDetGenerator(UVUDirectGenerator):
         fwd, bwd, _ = super().plan()
         for s in fwd:
             if s["kernel"] == "forward":
-                s["work_per_block"] = 1
+                s.update(work_per_block=1, grid_kind=3, num_blocks=self.LONG)
         bwd = [s for s in bwd if s["kernel"] == "prep_backward"] + self.backward_steps()
 
         def ws(nnz=0, nodes=0):
-            return 2 * (nodes + 1) * 8 + self.order_bytes(nodes) + self.dy_partial_bytes(nnz) + self.flag_bytes(nnz)
+            return self.main_bytes(nnz, nodes) + self.piece_bytes(nnz, nodes)
         return fwd, bwd, ws
+
+    def main_bytes(self, nnz: int, nodes: int) -> int:
+        """Workspace in front of the piece area (``piece_base``): both pointer arrays, the node order, the dY
+        partial rows and the flags of edges naming no node, rounded up to 256 bytes."""
+        b = 2 * (nodes + 1) * 8 + self.order_bytes(nodes) + self.dy_partial_bytes(nnz) + self.flag_bytes(nnz)
+        return (b + 255) & ~255
+
+    def forward_workspace_model(self):
+        """(fixed, per node, per edge) bytes the forward steps use when no node is cut into pieces."""
+        return 8, 8, 0
 
     # ================================================================= forward
     def conv_det_forward_body(self) -> str:
         E = Emitter()
         self.emit_lane_direct(E, lds=True)
-        self._node_setup(E, "0")
         if self.forward_perm:
             E("const i64* __restrict__ eperm = (const i64*)ws + 2 * (node_count + 1);")
+
+        def key(E, pos):
+            if self.forward_perm:
+                E(f"{{ const i64 e0_ = eperm[{pos}]; if (e0_ >= 0 && e0_ < (i64)nnz) kv_ = (i64)rows[e0_]; }}")
+            else:
+                E(f"kv_ = (i64)rows[{pos}];")
+        self._node_setup(E, "0", key=key)
         self._cur_c = "e"
         for oi in self.used_out:
             E("T " + ", ".join(f"z{oi}_{k} = (T)0" for k in range(self.out[oi].D)) + ";")
@@ -347,23 +551,8 @@ class UVUDetGenerator(UVUDirectGenerator):
         else:
             self.emit_pingpong_loop(E, names, load_idx, load, compute)
         E("const bool rv = nv;")
-        for o in self.out:
-            if o.dim == 0:
-                continue
-            E("{")
-            E.level += 1
-            if o.idx in self.used_out and self.R == 1:
-                self.emit_block_store(E, o, [f"z{o.idx}_{k}" for k in range(o.D)], "Z", self.D3, "node",
-                                      self.noderow_of, "store", via_lds=True)
-            elif o.idx in self.used_out:
-                zs = [f"z{o.idx}_{k}" for k in range(o.D)]
-                self.emit_sub_sum(E, zs)
-                self.emit_record_store(E, zs, f"Z + node * {self.D3} + {o.off} + u * {o.D}", self.store_act(o))
-            else:
-                self.emit_record_store(E, ["(T)0"] * o.D, f"Z + node * {self.D3} + {o.off} + u * {o.D}",
-                                       self.store_act(o))
-            E.level -= 1
-            E("}")
+        self.emit_node_output(E, self.out, self.used_out, lambda o: [f"z{o.idx}_{k}" for k in range(o.D)], "Z", self.D3,
+                              via_lds=True, zero_unused=True, add_existing=False)
         return E.text()
 
     def uclamp(self, blk, c) -> str:
@@ -542,9 +731,12 @@ class UVUDetGenerator(UVUDirectGenerator):
     def _backward_body(self, grp: int) -> str:
         E = Emitter()
         self.emit_lane_direct(E, lds=False)
-        self._node_setup(E, self.bwd_ptr_off, self.bwd_order if self.ordered_backward else None)
         list_t = "IDX" if self.bwd_list == "tperm" else "i64"
         E(f"const {list_t}* __restrict__ elist = {self.bwd_list};     // edge ids in (sender, ...) order")
+
+        def key(E, pos):
+            E(f"{{ const i64 e0_ = (i64)elist[{pos}]; if (e0_ >= 0 && e0_ < (i64)nnz) kv_ = (i64)cols[e0_]; }}")
+        self._node_setup(E, self.bwd_ptr_off, self.bwd_order if self.ordered_backward else None, key=key)
         self.emit_invalid_edge_rows(E, grp)
         self._cur_c = "e"
         # this node's own X chunk (fixed over the edge loop)
@@ -632,19 +824,8 @@ class UVUDetGenerator(UVUDirectGenerator):
         else:
             self.emit_pingpong_loop(E, names, load_idx, load, compute, prefetch_first=self.prefetch_backward)
         E("rv = nv;")
-        for a in self.in1:
-            if a.dim == 0:
-                continue
-            dst = f"Xg + node * {self.D1} + {a.off} + u * {a.D}"
-            if a.idx in self.used_in1:
-                dxs = [f"dx{a.idx}_{m}" for m in range(a.D)]
-                self.emit_sub_sum(E, dxs)
-                if grp > 0:            # the launches of the earlier groups have written this row: add to it
-                    E(f"if ({self.store_act(a)}) {{ const T* __restrict__ q_ = {dst}; "
-                      + " ".join(f"dx{a.idx}_{m} += q_[{m}];" for m in range(a.D)) + " }")
-                self.emit_record_store(E, dxs, dst, self.store_act(a))
-            elif grp == 0:
-                self.emit_record_store(E, ["(T)0"] * a.D, dst, self.store_act(a))
+        self.emit_node_output(E, self.in1, self.used_in1, lambda a: [f"dx{a.idx}_{m}" for m in range(a.D)], "Xg", self.D1,
+                              via_lds=False, zero_unused=(grp == 0), add_existing=(grp > 0))
         return E.text()
 
     def _forward_slabs(self):

@@ -62,6 +62,7 @@ class UVURecvGenerator(UVUDetGenerator):
         # the preparation's per-256-edge flags are not used here (pass 1 visits every edge and writes the
         # rows of edges naming no node itself): they go behind the spill
         self.flags_off = f"({self.spill_off} + nnz * {self.spill_row}ull * sizeof(T))"
+        self.piece_base = f"((({self.flags_off} + 4ull * ((nnz + 255) / 256)) + 255ull) & ~255ull)"
 
     def describe(self) -> str:
         return super().describe() + f" receiver-order backward (spill {self.spill_row} words/edge)"
@@ -70,7 +71,7 @@ class UVURecvGenerator(UVUDetGenerator):
     def backward_steps(self):
         steps = [dict(kernel="backward", num_threads=64, grid_kind=1, work_per_block=self.MIN_TILE_ITERS * self.R,
                       num_blocks=self.MAX_TILES, grid_y=self.NCH),
-                 dict(kernel="backward_dx", num_threads=64, grid_kind=2, work_per_block=1, grid_y=self.NCH)]
+                 dict(kernel="backward_dx", num_threads=64, grid_kind=3, work_per_block=1, num_blocks=self.LONG, grid_y=self.NCH)]
         if self.dy_slots > 1:
             steps.append(dict(kernel="backward_dy_reduce", num_threads=256, grid_kind=1,
                               work_per_block=self.dy_rows_per_block))
@@ -83,9 +84,12 @@ class UVURecvGenerator(UVUDetGenerator):
         fwd, bwd, _ = super().plan()
 
         def ws(nnz=0, nodes=0):
-            head = (2 * (nodes + 1) + nodes) * 8 + self.dy_partial_bytes(nnz)
-            return ((head + 255) & ~255) + self.spill_bytes(nnz) + self.flag_bytes(nnz)
+            return self.main_bytes(nnz, nodes) + self.piece_bytes(nnz, nodes)
         return fwd, bwd, ws
+
+    def main_bytes(self, nnz: int, nodes: int) -> int:
+        head = (2 * (nodes + 1) + nodes) * 8 + self.dy_partial_bytes(nnz)
+        return ((((head + 255) & ~255) + self.spill_bytes(nnz) + self.flag_bytes(nnz)) + 255) & ~255
 
     def backward_kernel_sources(self):
         w = self.waves_hint
@@ -228,8 +232,11 @@ class UVURecvGenerator(UVUDetGenerator):
         E = Emitter()
         P, NCH, U = self.P, self.NCH, self.DX_UNROLL
         self.emit_lane_direct(E, lds=False)
-        self._node_setup(E, self.bwd_ptr_off)
         E("const IDX* __restrict__ elist = tperm;     // edge ids in (sender, receiver) order")
+
+        def key(E, pos):
+            E(f"{{ const i64 e0_ = (i64)elist[{pos}]; if (e0_ >= 0 && e0_ < (i64)nnz) kv_ = (i64)cols[e0_]; }}")
+        self._node_setup(E, self.bwd_ptr_off, key=key)
         E(f"const T* __restrict__ spill = (const T*)((const char*)ws + {self.spill_off});")
         E("T " + ", ".join(f"acc{w} = (T)0" for w in range(self.NW)) + ";")
         E(f"for (int it = 0; it < maxlen; it += {U}) {{")
@@ -250,13 +257,6 @@ class UVURecvGenerator(UVUDetGenerator):
         for i in self.used_in1:
             names[i] = [f"acc{w + m}" for m in range(self.in1[i].D)]
             w += self.in1[i].D
-        for a in self.in1:
-            if a.dim == 0:
-                continue
-            dst = f"Xg + node * {self.D1} + {a.off} + u * {a.D}"
-            if a.idx in self.used_in1:
-                self.emit_sub_sum(E, names[a.idx])
-                self.emit_record_store(E, names[a.idx], dst, self.store_act(a))
-            else:
-                self.emit_record_store(E, ["(T)0"] * a.D, dst, self.store_act(a))
+        self.emit_node_output(E, self.in1, self.used_in1, lambda a: names[a.idx], "Xg", self.D1, via_lds=False,
+                              zero_unused=True, add_existing=False)
         return E.text()

@@ -57,6 +57,11 @@ class UVUSortedGenerator:
         self.T = self.fwd.T
         self.D1, self.D2, self.D3, self.WN = self.fwd.D1, self.fwd.D2, self.fwd.D3, self.fwd.WN
         self.NCH = self.fwd.NCH
+        # one piece area (counters and partial rows of long nodes) behind everything else, shared by both directions
+        if grouped_backward:
+            self.fwd.piece_base = self.bwd.piece_base
+        else:
+            self.fwd.piece_base = f"((({self.fwd.GROUP_WORDS}) * sizeof(i64) + 255ull) & ~255ull)"
 
     def describe(self) -> str:
         return ("sorted forward: " + self.fwd.describe()
@@ -71,24 +76,30 @@ class UVUSortedGenerator:
     def plan(self):
         ROW, NODE, FIXED = 1, 2, 0
         f = self.fwd
-        fwd = [dict(kernel="group_clear", num_threads=256, grid_kind=NODE, work_per_block=256, prep=True),
-               dict(kernel="group_count", num_threads=256, grid_kind=ROW, work_per_block=256, prep=True),
-               dict(kernel="group_scan", num_threads=self.SCAN_THREADS, grid_kind=FIXED, num_blocks=1, prep=True),
-               dict(kernel="group_fill", num_threads=256, grid_kind=ROW, work_per_block=256, prep=True),
-               dict(kernel="forward", num_threads=64, grid_kind=NODE, work_per_block=1, grid_y=f.NCH)]
+        S = self.SCAN_THREADS
+
+        def grouping(sfx):
+            return [dict(kernel="group_clear" + sfx, num_threads=256, grid_kind=NODE, work_per_block=256,
+                         prep=True, counter_clear=True),
+                    dict(kernel="group_count" + sfx, num_threads=S, grid_kind=ROW, work_per_block=S, prep=True),
+                    dict(kernel="group_fill" + sfx, num_threads=256, grid_kind=ROW, work_per_block=256, prep=True)]
+        fwd = grouping("") + [dict(kernel="forward", num_threads=64, grid_kind=3, work_per_block=1, num_blocks=f.LONG,
+                                   grid_y=f.NCH)]
+        G = f.group_bytes
         if not self.grouped_backward:
             _, bwd, _ = self.bwd.plan()
 
             def ws(nnz=0, nodes=0):
-                return (2 * (nodes + 1) + nnz) * 8
+                return ((G(nnz, nodes) + 255) & ~255) + f.piece_bytes(nnz, nodes)
             return fwd, bwd, ws
         b = self.bwd
-        bwd = [dict(kernel="group_clear_backward", num_threads=256, grid_kind=NODE, work_per_block=256, prep=True),
-               dict(kernel="group_count_backward", num_threads=256, grid_kind=ROW, work_per_block=256, prep=True),
-               dict(kernel="group_scan_backward", num_threads=self.SCAN_THREADS, grid_kind=FIXED, num_blocks=1, prep=True),
-               dict(kernel="group_fill_backward", num_threads=256, grid_kind=ROW, work_per_block=256, prep=True)]
-        bwd += b.backward_steps()
+        bwd = grouping("_backward") + b.backward_steps()
 
         def ws(nnz=0, nodes=0):
-            return 2 * (2 * (nodes + 1) + nnz) * 8 + b.order_bytes(nodes) + b.dy_partial_bytes(nnz) + b.flag_bytes(nnz)
+            main = 2 * G(nnz, nodes) + b.order_bytes(nodes) + b.dy_partial_bytes(nnz) + b.flag_bytes(nnz)
+            return ((main + 255) & ~255) + b.piece_bytes(nnz, nodes)
         return fwd, bwd, ws
+
+    def forward_workspace_model(self):
+        """(fixed, per node, per edge) bytes the forward steps use when no node is cut into pieces."""
+        return 32, 24, 8

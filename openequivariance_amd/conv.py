@@ -129,6 +129,10 @@ class _StreamWorkspace:
         self.captured = False        # a HIP graph capture has used this workspace
         self.fwd_key = self.bwd_key = None
         self.refs = {}               # index tensors of the cached keys, kept alive so that their addresses stay theirs
+        # (nnz, node_count) of the last completed call of each direction, while nothing else has written the
+        # workspace since: the counters of the on-the-fly grouping are then known to be zero where a call
+        # with the same sizes keeps them, and the step that clears them is skipped
+        self.zero_fwd = self.zero_bwd = None
 
 
 class TensorProductConv:
@@ -202,7 +206,10 @@ class TensorProductConv:
         need_ws = rt.STEP_NEEDS_WORKSPACE if ws(1, 1) > 0 else 0
         need_tp = rt.STEP_NEEDS_TPERM if self.backward_needs_tperm else 0
         code = rt.compile_source(source if source is not None else generator.render())
-        return rt.ConvImpl(code, _make_steps(fwd, need_ws), _make_steps(bwd, need_ws | need_tp))
+        impl = rt.ConvImpl(code, _make_steps(fwd, need_ws), _make_steps(bwd, need_ws | need_tp))
+        model = getattr(generator, "forward_workspace_model", None)
+        impl.set_forward_workspace(*(model() if model else (0, 0, 0)))
+        return impl
 
     def _ws_bytes(self, nnz: int, node_count: int) -> int:
         return max(f(nnz, node_count) for f in self._ws_fns)
@@ -239,7 +246,7 @@ class TensorProductConv:
                 rec.retired.append(rec.buffer)
             rec.size = int(need * 1.25) + 256
             rec.buffer = torch.empty(rec.size, dtype=torch.uint8, device="cuda")
-            rec.fwd_key = rec.bwd_key = None
+            rec.fwd_key = rec.bwd_key = rec.zero_fwd = rec.zero_bwd = None
             rec.refs.clear()
         return rec
 
@@ -299,24 +306,28 @@ class TensorProductConv:
 
     # ---------------------------------------------------------- raw entry points
     def exec_conv_rawptrs(self, L1_in, L2_in, weights, L3_out, rows, cols, nnz, node_count, workspace=0,
-                          transpose_perm=0, stream=None, prepared=False):
+                          transpose_perm=0, stream=None, prepared=False, counters_zero=False):
         """reference: extension/convolution.hpp:121-147.  Without ``workspace`` the operator's own scratch
         for the stream is used.  ``prepared=True`` promises that the workspace still holds the forward
         preparation of exactly this graph (left by an earlier forward call): the preparation kernels are
-        then skipped."""
+        then skipped.  ``counters_zero=True`` promises that the counters the operator keeps in the workspace
+        are zero (a zero-filled workspace, or one last written by a completed call of this operator with the
+        same sizes): the step that clears them is skipped."""
         nnz, node_count = int(nnz), int(node_count)
         if nnz > 0 and not (rows and cols):
             raise ValueError("rows / cols must be device pointers")
         impl = self._pick(L1_in, L2_in, weights, L3_out)
         if not workspace:
             rec = self._workspace_record(nnz, node_count, stream)
-            rec.fwd_key = None                                  # the caller's graph is unknown to the cache
+            rec.fwd_key = rec.zero_fwd = rec.zero_bwd = None    # the caller's graph is unknown to the cache
             workspace = rec.buffer.data_ptr() if self._ws_bytes(nnz, node_count) else 0
         impl.exec_conv_rawptrs(L1_in, L2_in, weights, L3_out, rows, cols, nnz, node_count,
-                               workspace, transpose_perm, self._stream() if stream is None else stream, prepared)
+                               workspace, transpose_perm, self._stream() if stream is None else stream, prepared,
+                               counters_zero)
 
     def backward_rawptrs(self, L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_grad, rows, cols, nnz,
-                         node_count, workspace=0, transpose_perm=0, stream=None, prepared=False, impl=None):
+                         node_count, workspace=0, transpose_perm=0, stream=None, prepared=False, impl=None,
+                         counters_zero=False):
         """reference: extension/convolution.hpp:149-173; ``workspace`` and ``prepared`` as in
         exec_conv_rawptrs (the backward keeps its own preparation in the workspace).  ``impl`` selects
         another kernel set of this operator (see _backward_variant) instead of the default one."""
@@ -329,11 +340,11 @@ class TensorProductConv:
             impl = self._pick(L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_grad)
         if not workspace:
             rec = self._workspace_record(nnz, node_count, stream)
-            rec.bwd_key = None
+            rec.bwd_key = rec.zero_fwd = rec.zero_bwd = None
             workspace = rec.buffer.data_ptr() if self._ws_bytes(nnz, node_count) else 0
         impl.backward_rawptrs(L1_in, L1_grad, L2_in, L2_grad, weights, weights_grad, L3_grad, rows, cols,
                               nnz, node_count, workspace, transpose_perm,
-                              self._stream() if stream is None else stream, prepared)
+                              self._stream() if stream is None else stream, prepared, counters_zero)
 
     def _time_backward_variants(self, run, names=("atomic", "grouped"), repeats: int = 3) -> str:
         """Fastest of the backward variants on the caller's own tensors: one untimed call each (compilation,
@@ -354,14 +365,14 @@ class TensorProductConv:
         return min(best, key=best.get)
 
     def _cached_call(self, which: str, rows, cols, tperm, E: int, N: int, launch, tag: str = "") -> None:
-        """Run ``launch(workspace pointer, prepared)`` for the torch operators.  The graph preparation a
+        """Run ``launch(workspace pointer, prepared, counters_zero)`` for the torch operators.  The graph preparation a
         call leaves in the stream's workspace is reused by the next call of the same direction when it
         names the same graph: same index tensors (address and in-place version counter), same sizes.  The
         tensors are kept referenced while their key is cached, so the addresses cannot be handed to other
         tensors meanwhile.  Under HIP graph capture, and on a workspace that a capture has used, the
         preparation always runs: a replay may rewrite the workspace behind the cache's back."""
         if self._ws_bytes(E, N) == 0:
-            launch(0, False)
+            launch(0, False, False)
             return
         rec = self._workspace_record(E, N)
         if torch.cuda.is_current_stream_capturing():
@@ -369,11 +380,18 @@ class TensorProductConv:
         key = None
         if self.graph_cache and not rec.captured:
             key = (tag, E, N) + tuple((t.data_ptr(), t._version) for t in (rows, cols, tperm) if t is not None)
-        attr = which + "_key"
+        attr, zattr, other = which + "_key", "zero_" + which, "zero_" + ("bwd" if which == "fwd" else "fwd")
         prepared = key is not None and getattr(rec, attr) == key
+        # every call leaves the grouping counters it used zeroed; a call with other sizes keeps them elsewhere
+        # (the kernel sets of the backward variants differ in whether they group at all, hence the tag)
+        counters_zero = not rec.captured and getattr(rec, zattr) == (E, N, tag)
+        if (getattr(rec, other) or (None,))[:2] != (E, N):
+            setattr(rec, other, None)
         setattr(rec, attr, None)
-        launch(rec.buffer.data_ptr(), prepared)
+        setattr(rec, zattr, None)
+        launch(rec.buffer.data_ptr(), prepared, counters_zero)
         setattr(rec, attr, key)
+        setattr(rec, zattr, None if rec.captured else (E, N, tag))
         rec.refs[which] = (rows, cols, tperm) if key is not None else None
 
     # ------------------------------------------------------------------ torch ops
@@ -392,9 +410,9 @@ class TensorProductConv:
             # the atomic kernels accumulate into Z; the deterministic ones write every row
             out = (torch.empty if self.forward_overwrites else torch.zeros)((N, L3_dim), dtype=x.dtype, device=x.device)
             with torch.cuda.device(x.device):
-                self._cached_call("fwd", rows, cols, tperm, E, N, lambda ws, prepared: self.exec_conv_rawptrs(
+                self._cached_call("fwd", rows, cols, tperm, E, N, lambda ws, prepared, zero: self.exec_conv_rawptrs(
                     x.data_ptr(), y.data_ptr(), w.data_ptr(), out.data_ptr(), rows.data_ptr(), cols.data_ptr(), E, N,
-                    ws, tperm.data_ptr() if tperm is not None else 0, prepared=prepared))
+                    ws, tperm.data_ptr() if tperm is not None else 0, prepared=prepared, counters_zero=zero))
             return out
 
         def bwd_run(x, y, w, g, rows, cols, tperm, E, N, variant=None):
@@ -404,10 +422,10 @@ class TensorProductConv:
                 impl, overwrites, variant = None, self.backward_overwrites, None     # misaligned views: the default set only
             xg = (torch.empty_like if overwrites else torch.zeros_like)(x)
             yg, wg = torch.empty_like(y), torch.empty_like(w)
-            self._cached_call("bwd", rows, cols, tperm, E, N, lambda ws, prepared: self.backward_rawptrs(
+            self._cached_call("bwd", rows, cols, tperm, E, N, lambda ws, prepared, zero: self.backward_rawptrs(
                 x.data_ptr(), xg.data_ptr(), y.data_ptr(), yg.data_ptr(), w.data_ptr(), wg.data_ptr(), g.data_ptr(),
                 rows.data_ptr(), cols.data_ptr(), E, N, ws, tperm.data_ptr() if tperm is not None else 0,
-                prepared=prepared, impl=impl), tag=variant or "")
+                prepared=prepared, impl=impl, counters_zero=zero), tag=variant or "")
             return [xg, yg, wg]
 
         def bwd_impl(L1_in, L2_in, weights, L3_grad, rows, cols, tperm):

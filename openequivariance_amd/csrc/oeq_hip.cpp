@@ -84,16 +84,33 @@ int load_steps(Module& m, const void* code, size_t code_size, const oeq_step* st
     return 0;
 }
 
-uint64_t grid_of(const oeq_step& d, uint64_t rows, uint64_t nodes) {
+// Edges per piece of a long node's edge list: the kernels compute the same number from nnz and node_count.
+uint64_t piece_edges(uint64_t factor, uint64_t rows, uint64_t nodes) {
+    const uint64_t mean = nodes ? (rows + nodes - 1) / nodes : 0;
+    const uint64_t t = factor * mean;
+    return t < OEQ_PIECE_MIN_EDGES ? OEQ_PIECE_MIN_EDGES : t;
+}
+
+uint64_t grid_of(const oeq_step& d, uint64_t rows, uint64_t nodes, bool pieces) {
     if (d.grid_kind == OEQ_GRID_FIXED) return d.num_blocks;
+    if (d.grid_kind == OEQ_GRID_PER_NODE_AND_PIECE) {
+        // one workgroup per node, then two per tile of the edge list (the piece of a long node that ends
+        // in the tile and the piece of one that begins in it); num_blocks holds the long-node factor
+        uint64_t g = (nodes + d.work_per_block - 1) / d.work_per_block;
+        if (pieces && d.num_blocks != 0 && rows > 0 && nodes > 0) {
+            const uint64_t t = piece_edges(d.num_blocks, rows, nodes);
+            g += 2 * ((rows + t - 1) / t);
+        }
+        return g;
+    }
     uint64_t work = (d.grid_kind == OEQ_GRID_PER_ROW) ? rows : nodes;
     uint64_t g = (work + d.work_per_block - 1) / d.work_per_block;
     if (d.num_blocks != 0 && g > d.num_blocks) g = d.num_blocks;
     return g;
 }
 
-int launch(const Step& s, uint64_t rows, uint64_t nodes, void** args, void* stream) {
-    uint64_t g = grid_of(s.desc, rows, nodes);
+int launch(const Step& s, uint64_t rows, uint64_t nodes, void** args, void* stream, bool pieces = true) {
+    uint64_t g = grid_of(s.desc, rows, nodes, pieces);
     if (g == 0) return 0;
     if (g > 0x7fffffffull) return fail("grid of %llu workgroups is too large", (unsigned long long)g);
     const unsigned gy = s.desc.grid_y ? s.desc.grid_y : 1u;
@@ -123,6 +140,10 @@ struct oeq_tp {
 struct oeq_conv {
     Module mod;
     std::vector<Step> fwd, bwd;
+    // bytes of workspace the forward steps use when long nodes are not cut into pieces:
+    // fixed + per_node * node_count + per_edge * nnz (oeq_conv_set_forward_workspace)
+    uint64_t ws_fixed = 0, ws_per_node = 16, ws_per_edge = 8;
+    bool ws_model_set = false;
 };
 struct oeq_module {
     Module mod;
@@ -265,6 +286,8 @@ int oeq_tp_backward(oeq_tp* tp, uint64_t n, const void* L1, void* L1g, const voi
 }
 
 // ------------------------------------------------------------------- conv
+static int noalloc_scratch(void** out);
+
 int oeq_conv_create(const void* code, size_t code_size, const oeq_step* fs, int nf, const oeq_step* bs,
                     int nb, oeq_conv** out) {
     if (!code || !out || nf < 0 || nb < 0 || (nf && !fs) || (nb && !bs)) return fail("bad argument");
@@ -274,39 +297,53 @@ int oeq_conv_create(const void* code, size_t code_size, const oeq_step* fs, int 
         delete c;
         return 1;
     }
+    // Set-up is where the static scratch of oeq_conv_forward_noalloc is looked up on this device (the runtime
+    // materialises the array on first use): the entry point itself must not be the first to touch it, it may
+    // run under stream capture.  A failure here is reported by that entry point, not by this one.
+    void* scratch = nullptr;
+    if (noalloc_scratch(&scratch)) g_error.clear();
     *out = c;
     return 0;
 }
 
 void oeq_conv_destroy(oeq_conv* c) { delete c; }
 
+// A step is skipped when the call says that the state it would build is already in the workspace.
+static bool skipped(const oeq_step& d, uint32_t call_flags) {
+    if ((call_flags & OEQ_CALL_PREPARED) && (d.flags & OEQ_STEP_GRAPH_PREP)) return true;
+    if ((call_flags & OEQ_CALL_COUNTERS_ZERO) && (d.flags & OEQ_STEP_COUNTER_CLEAR)) return true;
+    return false;
+}
+
 static int conv_forward(oeq_conv* c, const void* L1, const void* L2, const void* W, void* L3,
                         const void* rows, const void* cols, uint64_t nnz, uint64_t node_count,
-                        void* workspace, const void* tperm, void* stream, bool prepared) {
+                        void* workspace, const void* tperm, void* stream, uint32_t call_flags, bool pieces = true) {
     if (!c) return fail("null handle");
     if (c->fwd.empty()) return fail("this operator was built without a forward plan");
     if (nnz > 0 && node_count == 0) return fail("convolution called with %llu edges but no nodes", (unsigned long long)nnz);
     if (nnz > 0 && (!rows || !cols)) return fail("forward: rows / cols are NULL");
     if ((nnz > 0 || node_count > 0) && check_pointers(c->fwd, workspace, tperm, "forward")) return 1;
+    if (call_flags & ~(uint32_t)(OEQ_CALL_PREPARED | OEQ_CALL_COUNTERS_ZERO)) return fail("forward: unknown call flags 0x%x", call_flags);
     void* args[] = {&L1, &L2, &W, &L3, &rows, &cols, &nnz, &node_count, &workspace, &tperm};
     for (auto& s : c->fwd) {
-        if (prepared && (s.desc.flags & OEQ_STEP_GRAPH_PREP)) continue;
-        if (launch(s, nnz, node_count, args, stream)) return 1;
+        if (skipped(s.desc, call_flags)) continue;
+        if (launch(s, nnz, node_count, args, stream, pieces)) return 1;
     }
     return 0;
 }
 
 static int conv_backward(oeq_conv* c, const void* L1, void* L1g, const void* L2, void* L2g, const void* W,
                          void* Wg, const void* L3g, const void* rows, const void* cols, uint64_t nnz,
-                         uint64_t node_count, void* workspace, const void* tperm, void* stream, bool prepared) {
+                         uint64_t node_count, void* workspace, const void* tperm, void* stream, uint32_t call_flags) {
     if (!c) return fail("null handle");
     if (c->bwd.empty()) return fail("this operator was built without a backward plan");
     if (nnz > 0 && node_count == 0) return fail("convolution called with %llu edges but no nodes", (unsigned long long)nnz);
     if (nnz > 0 && (!rows || !cols)) return fail("backward: rows / cols are NULL");
     if ((nnz > 0 || node_count > 0) && check_pointers(c->bwd, workspace, tperm, "backward")) return 1;
+    if (call_flags & ~(uint32_t)(OEQ_CALL_PREPARED | OEQ_CALL_COUNTERS_ZERO)) return fail("backward: unknown call flags 0x%x", call_flags);
     void* args[] = {&L1, &L1g, &L2, &L2g, &W, &Wg, &L3g, &rows, &cols, &nnz, &node_count, &workspace, &tperm};
     for (auto& s : c->bwd) {
-        if (prepared && (s.desc.flags & OEQ_STEP_GRAPH_PREP)) continue;
+        if (skipped(s.desc, call_flags)) continue;
         if (launch(s, nnz, node_count, args, stream)) return 1;
     }
     return 0;
@@ -315,25 +352,34 @@ static int conv_backward(oeq_conv* c, const void* L1, void* L1g, const void* L2,
 int oeq_conv_forward(oeq_conv* c, const void* L1, const void* L2, const void* W, void* L3,
                      const void* rows, const void* cols, uint64_t nnz, uint64_t node_count,
                      void* workspace, const void* tperm, void* stream) {
-    return conv_forward(c, L1, L2, W, L3, rows, cols, nnz, node_count, workspace, tperm, stream, false);
+    return conv_forward(c, L1, L2, W, L3, rows, cols, nnz, node_count, workspace, tperm, stream, 0);
 }
 
-int oeq_conv_forward_prepared(oeq_conv* c, const void* L1, const void* L2, const void* W, void* L3,
-                              const void* rows, const void* cols, uint64_t nnz, uint64_t node_count,
-                              void* workspace, const void* tperm, void* stream) {
-    return conv_forward(c, L1, L2, W, L3, rows, cols, nnz, node_count, workspace, tperm, stream, true);
+int oeq_conv_forward_ex(oeq_conv* c, const void* L1, const void* L2, const void* W, void* L3,
+                        const void* rows, const void* cols, uint64_t nnz, uint64_t node_count,
+                        void* workspace, const void* tperm, void* stream, uint32_t call_flags) {
+    return conv_forward(c, L1, L2, W, L3, rows, cols, nnz, node_count, workspace, tperm, stream, call_flags);
 }
 
 int oeq_conv_backward(oeq_conv* c, const void* L1, void* L1g, const void* L2, void* L2g, const void* W,
                       void* Wg, const void* L3g, const void* rows, const void* cols, uint64_t nnz,
                       uint64_t node_count, void* workspace, const void* tperm, void* stream) {
-    return conv_backward(c, L1, L1g, L2, L2g, W, Wg, L3g, rows, cols, nnz, node_count, workspace, tperm, stream, false);
+    return conv_backward(c, L1, L1g, L2, L2g, W, Wg, L3g, rows, cols, nnz, node_count, workspace, tperm, stream, 0);
 }
 
-int oeq_conv_backward_prepared(oeq_conv* c, const void* L1, void* L1g, const void* L2, void* L2g, const void* W,
-                               void* Wg, const void* L3g, const void* rows, const void* cols, uint64_t nnz,
-                               uint64_t node_count, void* workspace, const void* tperm, void* stream) {
-    return conv_backward(c, L1, L1g, L2, L2g, W, Wg, L3g, rows, cols, nnz, node_count, workspace, tperm, stream, true);
+int oeq_conv_backward_ex(oeq_conv* c, const void* L1, void* L1g, const void* L2, void* L2g, const void* W,
+                         void* Wg, const void* L3g, const void* rows, const void* cols, uint64_t nnz,
+                         uint64_t node_count, void* workspace, const void* tperm, void* stream, uint32_t call_flags) {
+    return conv_backward(c, L1, L1g, L2, L2g, W, Wg, L3g, rows, cols, nnz, node_count, workspace, tperm, stream, call_flags);
+}
+
+int oeq_conv_set_forward_workspace(oeq_conv* c, uint64_t fixed_bytes, uint64_t bytes_per_node, uint64_t bytes_per_edge) {
+    if (!c) return fail("null handle");
+    c->ws_fixed = fixed_bytes;
+    c->ws_per_node = bytes_per_node;
+    c->ws_per_edge = bytes_per_edge;
+    c->ws_model_set = true;
+    return 0;
 }
 
 // Device address of this GPU's copy of oeq_noalloc_scratch, looked up on first use per device.
@@ -359,9 +405,12 @@ int oeq_conv_forward_noalloc(oeq_conv* c, const void* L1, const void* L2, const 
                              const void* rows, const void* cols, uint64_t nnz, uint64_t node_count,
                              const void* tperm, void* stream) {
     if (!c) return fail("null handle");
-    // bytes the forward kernels of any plan use: two pointer arrays and one position list, int64
+    if (!c->ws_model_set)
+        return fail("oeq_conv_forward_noalloc: the operator's forward workspace size is unknown "
+                    "(call oeq_conv_set_forward_workspace after oeq_conv_create)");
     if (nnz > (1ull << 40) || node_count > (1ull << 40)) return fail("graph too large");
-    const uint64_t need = 8ull * (2ull * (node_count + 1ull) + nnz);
+    // what the forward steps of this operator's plan use with every node walked by one wavefront
+    const uint64_t need = c->ws_fixed + c->ws_per_node * node_count + c->ws_per_edge * nnz;
     if (need > (uint64_t)OEQ_NOALLOC_SCRATCH_BYTES)
         return fail("oeq_conv_forward_noalloc: %llu edges and %llu nodes need %llu bytes of scratch, the static "
                     "scratch holds %llu (use oeq_conv_forward with a caller-owned workspace)",
@@ -369,7 +418,7 @@ int oeq_conv_forward_noalloc(oeq_conv* c, const void* L1, const void* L2, const 
                     (unsigned long long)OEQ_NOALLOC_SCRATCH_BYTES);
     void* scratch = nullptr;
     if (noalloc_scratch(&scratch)) return 1;
-    return conv_forward(c, L1, L2, W, L3, rows, cols, nnz, node_count, scratch, tperm, stream, false);
+    return conv_forward(c, L1, L2, W, L3, rows, cols, nnz, node_count, scratch, tperm, stream, 0, /*pieces=*/false);
 }
 
 // ---------------------------------------------------------- generic module

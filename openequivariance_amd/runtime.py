@@ -21,8 +21,10 @@ LIB_PATH = PKG_DIR / "csrc" / "liboeq_hip.so"
 CACHE_DIR = tunables.current.cache_dir
 TARGET_ARCH = "gfx950"
 
-GRID_FIXED, GRID_PER_ROW, GRID_PER_NODE = 0, 1, 2
-STEP_NEEDS_WORKSPACE, STEP_NEEDS_TPERM, STEP_GRAPH_PREP = 1, 2, 4
+GRID_FIXED, GRID_PER_ROW, GRID_PER_NODE, GRID_PER_NODE_AND_PIECE = 0, 1, 2, 3
+STEP_NEEDS_WORKSPACE, STEP_NEEDS_TPERM, STEP_GRAPH_PREP, STEP_COUNTER_CLEAR = 1, 2, 4, 8
+CALL_PREPARED, CALL_COUNTERS_ZERO = 1, 2
+PIECE_MIN_EDGES = 32                     # OEQ_PIECE_MIN_EDGES
 NOALLOC_SCRATCH_BYTES = 16 << 20        # OEQ_NOALLOC_SCRATCH_BYTES
 
 
@@ -91,8 +93,9 @@ def lib() -> C.CDLL:
             "oeq_conv_destroy": (None, [vp]),
             "oeq_conv_forward": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, u64, u64, vp, vp, vp]),
             "oeq_conv_backward": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, u64, u64, vp, vp, vp]),
-            "oeq_conv_forward_prepared": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, u64, u64, vp, vp, vp]),
-            "oeq_conv_backward_prepared": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, u64, u64, vp, vp, vp]),
+            "oeq_conv_forward_ex": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, u64, u64, vp, vp, vp, C.c_uint32]),
+            "oeq_conv_backward_ex": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, u64, u64, vp, vp, vp, C.c_uint32]),
+            "oeq_conv_set_forward_workspace": (C.c_int, [vp, u64, u64, u64]),
             "oeq_conv_forward_noalloc": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, u64, u64, vp, vp]),
             "oeq_module_load": (C.c_int, [vp, sz, C.POINTER(vp)]),
             "oeq_module_unload": (None, [vp]),
@@ -120,7 +123,7 @@ EXPORTED_SYMBOLS = [
     "oeq_last_error", "oeq_device_props", "oeq_device_count", "oeq_compile", "oeq_free", "oeq_hiprtc_version",
     "oeq_tp_create", "oeq_tp_destroy", "oeq_tp_forward", "oeq_tp_backward",
     "oeq_conv_create", "oeq_conv_destroy", "oeq_conv_forward", "oeq_conv_backward",
-    "oeq_conv_forward_prepared", "oeq_conv_backward_prepared", "oeq_conv_forward_noalloc",
+    "oeq_conv_forward_ex", "oeq_conv_backward_ex", "oeq_conv_set_forward_workspace", "oeq_conv_forward_noalloc",
     "oeq_module_load", "oeq_module_unload", "oeq_module_launch",
     "oeq_timer_create", "oeq_timer_destroy", "oeq_timer_start", "oeq_timer_stop", "oeq_timer_clear_cache",
     "oeq_buffer_alloc", "oeq_buffer_free", "oeq_buffer_h2d", "oeq_buffer_d2h", "oeq_buffer_zero",
@@ -184,6 +187,38 @@ def compile_source(source: str, arch: str = TARGET_ARCH, options: Sequence[str] 
     return blob
 
 
+def kernel_metadata(code: bytes) -> dict:
+    """{kernel name: metadata} from the AMDGPU note of a code object: ``.vgpr_count``, ``.agpr_count``,
+    ``.sgpr_count``, ``.private_segment_fixed_size`` (scratch bytes per lane: register spills),
+    ``.group_segment_fixed_size`` (static LDS bytes)."""
+    import struct
+
+    import msgpack
+    if code[:4] != b"\x7fELF" or code[4] != 2:
+        raise ValueError("not a 64-bit ELF code object")
+    shoff, = struct.unpack_from("<Q", code, 0x28)
+    shentsize, shnum = struct.unpack_from("<HH", code, 0x3A)
+    out = {}
+    for i in range(shnum):
+        off = shoff + i * shentsize
+        sh_type, = struct.unpack_from("<I", code, off + 4)
+        sh_offset, sh_size = struct.unpack_from("<QQ", code, off + 0x18)
+        if sh_type != 7:                                  # SHT_NOTE
+            continue
+        pos, end = sh_offset, sh_offset + sh_size
+        while pos + 12 <= end:
+            namesz, descsz, ntype = struct.unpack_from("<III", code, pos)
+            pos += 12
+            name = code[pos:pos + namesz].rstrip(b"\0")
+            pos += (namesz + 3) & ~3
+            desc = code[pos:pos + descsz]
+            pos += (descsz + 3) & ~3
+            if name == b"AMDGPU" and ntype == 32:         # NT_AMDGPU_METADATA
+                for k in msgpack.unpackb(desc, raw=False, strict_map_key=False).get("amdhsa.kernels", []):
+                    out[k[".name"]] = k
+    return out
+
+
 # ------------------------------------------------------------------------ operators
 def _steps(steps: Sequence[Step]):
     arr = (Step * max(1, len(steps)))(*steps)
@@ -224,21 +259,28 @@ class ConvImpl:
         ba, nb = _steps(backward_steps)
         _check(lib().oeq_conv_create(code, len(code), fa, nf, ba, nb, C.byref(self._h)))
 
+    def set_forward_workspace(self, fixed_bytes: int, bytes_per_node: int, bytes_per_edge: int) -> None:
+        """Declares what the forward steps use of the workspace without piece workgroups (checked by
+        exec_conv_noalloc against the static scratch)."""
+        _check(lib().oeq_conv_set_forward_workspace(self._h, fixed_bytes, bytes_per_node, bytes_per_edge))
+
     def exec_conv_rawptrs(self, L1, L2, W, L3, rows, cols, nnz, node_count, workspace=0, tperm=0, stream=0,
-                          prepared=False):
-        """``prepared``: the workspace still holds this graph's forward preparation (see
-        oeq_conv_forward_prepared); the preparation kernels are then not launched."""
-        fn = lib().oeq_conv_forward_prepared if prepared else lib().oeq_conv_forward
-        _check(fn(self._h, L1, L2, W, L3, rows, cols, nnz, node_count, workspace, tperm, stream))
+                          prepared=False, counters_zero=False):
+        """``prepared``: the workspace still holds this graph's forward preparation (OEQ_CALL_PREPARED); the
+        preparation kernels are then not launched.  ``counters_zero``: the operator's counters in the
+        workspace are known to be zero (OEQ_CALL_COUNTERS_ZERO); the step that clears them is skipped."""
+        flags = (CALL_PREPARED if prepared else 0) | (CALL_COUNTERS_ZERO if counters_zero else 0)
+        _check(lib().oeq_conv_forward_ex(self._h, L1, L2, W, L3, rows, cols, nnz, node_count, workspace, tperm, stream, flags))
 
     def exec_conv_noalloc(self, L1, L2, W, L3, rows, cols, nnz, node_count, tperm=0, stream=0):
         """The forward with the library's static scratch as its workspace: allocates nothing."""
         _check(lib().oeq_conv_forward_noalloc(self._h, L1, L2, W, L3, rows, cols, nnz, node_count, tperm, stream))
 
     def backward_rawptrs(self, L1, L1g, L2, L2g, W, Wg, L3g, rows, cols, nnz, node_count,
-                         workspace=0, tperm=0, stream=0, prepared=False):
-        fn = lib().oeq_conv_backward_prepared if prepared else lib().oeq_conv_backward
-        _check(fn(self._h, L1, L1g, L2, L2g, W, Wg, L3g, rows, cols, nnz, node_count, workspace, tperm, stream))
+                         workspace=0, tperm=0, stream=0, prepared=False, counters_zero=False):
+        flags = (CALL_PREPARED if prepared else 0) | (CALL_COUNTERS_ZERO if counters_zero else 0)
+        _check(lib().oeq_conv_backward_ex(self._h, L1, L1g, L2, L2g, W, Wg, L3g, rows, cols, nnz, node_count, workspace,
+                                          tperm, stream, flags))
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None

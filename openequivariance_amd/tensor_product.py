@@ -20,16 +20,18 @@ from .autograd_glue import double_backward_terms
 from .codegen.uvu import UVUGenerator
 from .codegen.uvu_direct import UVUDirectGenerator
 from .problem import TPProblem
-from .weight_order import WeightReorder, is_identity
+from .weight_order import WeightReorder
 from .wigner import wigner_3j
 
 
 def _make_steps(descs, flags: int = 0):
     """Plan dictionaries of a generator -> ``runtime.Step`` records.  ``flags`` (STEP_NEEDS_*) apply to
-    every step of the plan; a step's own ``prep=True`` marks it as graph preparation."""
+    every step of the plan; a step's own ``prep=True`` marks it as graph preparation, ``counter_clear=True``
+    as one that only zeroes counters which the operator's other steps leave zeroed again."""
     return [rt.Step.make(d["kernel"], d["num_threads"], d.get("smem", 0), d.get("grid_kind", rt.GRID_PER_ROW),
                          d.get("work_per_block", 1), d.get("num_blocks", 0), d.get("grid_y", 1),
-                         flags | (rt.STEP_GRAPH_PREP if d.get("prep") else 0)) for d in descs]
+                         flags | (rt.STEP_GRAPH_PREP if d.get("prep") else 0)
+                         | (rt.STEP_COUNTER_CLEAR if d.get("counter_clear") else 0)) for d in descs]
 
 
 def select_generator(config: TPProblem):
@@ -99,9 +101,6 @@ class TensorProduct(TensorProductBase):
         self._internal_unaligned = None       # kernels without 16-byte vector stores, compiled on first need
 
         self._reorder = WeightReorder(config)
-        if is_identity(self._reorder.perm):
-            # same convention as the reference: the attribute is still callable
-            pass
         self.reorder_weights_e3nn_to_oeq = self._reorder.e3nn_to_oeq
         self.reorder_weights_oeq_to_e3nn = self._reorder.oeq_to_e3nn
 

@@ -79,6 +79,18 @@ def conv_inputs(prob, nodes, nnz, seed, dtype=np.float32, sh_lmax=None):
     return tuple(np.ascontiguousarray(a.astype(dtype)) for a in (X, Y, W, G))
 
 
+def hub_graph(nodes, nnz, seed, hub_in, hub_out, in_edges, out_edges):
+    """A random graph of ``nnz`` edges in which node ``hub_in`` receives ``in_edges`` of them and node
+    ``hub_out`` sends ``out_edges`` (the rest uniform): two long edge lists next to short ones."""
+    rng = np.random.default_rng(seed)
+    rows = rng.integers(0, nodes, nnz)
+    cols = rng.integers(0, nodes, nnz)
+    pick = rng.permutation(nnz)
+    rows[pick[:in_edges]] = hub_in
+    cols[pick[in_edges:in_edges + out_edges]] = hub_out
+    return rows.astype(np.int64), cols.astype(np.int64)
+
+
 def with_invalid_edges(rows, cols, nodes, seed, count=7):
     """A copy of the edge list in which ``count`` edges name a node that does not exist (sender or
     receiver negative or >= nodes), and the mask of the edges left valid."""

@@ -61,6 +61,11 @@ static inline int oeq_shfl_xor_i32(int v, int mask) { g_xi[threadIdx.x] = v; oeq
 #define __builtin_amdgcn_readfirstlane(x) oeq_shfl_i32((x), 0)
 struct VT { T v[16 / sizeof(T)]; T& operator[](int i) { return v[i]; } const T& operator[](int i) const { return v[i]; } };
 #define OEQ_DMA(BYTES, POLICY, g, lds_base) memcpy((char*)(lds_base) + ((BYTES) == 12 ? 16 : (BYTES)) * (threadIdx.x & 63), (g), (BYTES))
+static inline void oeq_release_agent() {}
+static inline void oeq_acquire_agent() {}
+static inline int oeq_ticket_add(int* p) { std::lock_guard<std::mutex> g(g_atomic_mutex); return (*p)++; }
+static inline i64 oeq_lds_claim(i64* slot, i64 key) { std::lock_guard<std::mutex> g(g_atomic_mutex); const i64 old = *slot; if (old == -1) *slot = key; return old; }
+static inline int oeq_lds_add(int* p, int v) { std::lock_guard<std::mutex> g(g_atomic_mutex); const int o = *p; *p += v; return o; }
 static inline void oeq_wait_vm() {}
 static inline void oeq_wait_lds() {}
 static inline T oeq_wave_sum63(T v) { g_xT[threadIdx.x] = v; oeq_sync(); T t = 0; for (int i = 0; i < 64; ++i) t += g_xT[(threadIdx.x & ~63) + i]; oeq_sync(); return t; }
@@ -205,13 +210,11 @@ CONV_EXTRA_ORDER = r"""
 CONV_EXTRA_SORTED = r"""
         else if (k == "group_clear") FWD_CALL(group_clear);
         else if (k == "group_count") FWD_CALL(group_count);
-        else if (k == "group_scan") FWD_CALL(group_scan);
         else if (k == "group_fill") FWD_CALL(group_fill);
 """
 CONV_EXTRA_GROUPED_BWD = r"""
         else if (k == "group_clear_backward") BWD_CALL(group_clear_backward);
         else if (k == "group_count_backward") BWD_CALL(group_count_backward);
-        else if (k == "group_scan_backward") BWD_CALL(group_scan_backward);
         else if (k == "group_fill_backward") BWD_CALL(group_fill_backward);
 """
 CONV_EXTRA_DYRED = r"""
@@ -247,6 +250,12 @@ def grid_of(step: Dict, rows: int, nodes: int) -> int:
     kind = step.get("grid_kind", 1)
     if kind == 0:
         return step["num_blocks"]
+    if kind == 3:                            # one workgroup per node, then two per tile of the edge list
+        g = (nodes + step["work_per_block"] - 1) // step["work_per_block"]
+        if step.get("num_blocks", 0) and rows > 0 and nodes > 0:
+            t = max(32, step["num_blocks"] * ((rows + nodes - 1) // nodes))
+            g += 2 * ((rows + t - 1) // t)
+        return g
     work = rows if kind == 1 else nodes
     wpb = step["work_per_block"]
     g = (work + wpb - 1) // wpb

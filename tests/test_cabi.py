@@ -57,9 +57,11 @@ def test_error_reporting_without_device():
     L = rt.lib()
     assert L.oeq_tp_forward(None, 1, None, None, None, None, None, None) != 0
     assert b"null handle" in L.oeq_last_error()
-    for fn in (L.oeq_conv_forward, L.oeq_conv_forward_prepared):
-        assert fn(None, None, None, None, None, None, None, 0, 0, None, None, None) != 0
-        assert b"null handle" in L.oeq_last_error()
+    assert L.oeq_conv_forward(None, None, None, None, None, None, None, 0, 0, None, None, None) != 0
+    assert b"null handle" in L.oeq_last_error()
+    assert L.oeq_conv_forward_ex(None, None, None, None, None, None, None, 0, 0, None, None, None, rt.CALL_PREPARED) != 0
+    assert b"null handle" in L.oeq_last_error()
+    assert L.oeq_conv_set_forward_workspace(None, 0, 0, 0) != 0
     assert L.oeq_conv_forward_noalloc(None, None, None, None, None, None, None, 0, 0, None, None) != 0
     assert b"null handle" in L.oeq_last_error()
     n = ctypes.c_int(-1)

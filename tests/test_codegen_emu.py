@@ -84,6 +84,62 @@ def test_conv(variant):
         assert rel_err(got, ref) < TOL
 
 
+HUB_CASES = {
+    # name: (irreps, generator factory, deterministic?)
+    "det_two_sublists_lds": (common.NEQUIP, lambda p: UVUDetGenerator(p, lds=True), True),
+    "det_two_sublists_registers": (common.NEQUIP, lambda p: UVUDetGenerator(p, lds=False), True),
+    "det_two_chunks_two_groups": (("70x0e+70x1o+70x2e", "1x0e+1x1o+1x2e+1x3o", "70x0e+70x1o+70x2e+70x3o"), UVUDetGenerator, True),
+    "det_receiver_order": (common.NEQUIP, None, True),
+    "unsorted_grouped": (common.NEQUIP, lambda p: UVUSortedGenerator(p, grouped_backward=True), False),
+    "unsorted_atomic_backward": (common.NEQUIP, lambda p: UVUSortedGenerator(p, grouped_backward=False), False),
+}
+
+
+@pytest.mark.parametrize("case", sorted(HUB_CASES))
+def test_conv_long_nodes_walked_in_pieces(case):
+    """A receiver with 150 incoming and a sender with 130 outgoing edges among 12 nodes and 400 edges (mean 34:
+    pieces of 68 edges): the hubs' lists are cut at multiples of 68 list positions, each piece is walked by a
+    wavefront of its own into a partial row, the piece finishing last adds them; short nodes, nodes spanning
+    a cut without being long, and the zero-filled rows of nodes without edges are as before."""
+    from openequivariance_amd.codegen.uvu_recv import UVURecvGenerator
+    irreps, make, det = HUB_CASES[case]
+    prob, oprob = common.channelwise(irreps)
+    g = (make or UVURecvGenerator)(prob)
+    nodes, nnz = 12, 400
+    rows, cols = common.hub_graph(nodes - 1, nnz, 21, hub_in=3, hub_out=5, in_edges=150, out_edges=130)   # node 11: no edges
+    tperm = None
+    if det:
+        rows, cols, tperm, _ = otp.coord_graph(rows, cols)
+    X, Y, W, G = common.conv_inputs(prob, nodes, nnz, 22)
+    fwd, bwd, ws = g.plan()
+    f = g.fwd if hasattr(g, "fwd") else g
+    assert f.LONG == 2 and f.piece_tiles(nnz, nodes) == 6
+    assert emu.grid_of([s for s in fwd if s["kernel"] == "forward"][0], nnz, nodes) == nodes + 12
+    junk = np.arange(nnz)
+    out = emu.run_conv(g, fwd, X, Y, W, rows, cols, tperm=tperm if det else junk, ws_bytes=ws(nnz, nodes))
+    assert rel_err(out["Z"], otp.conv_forward(oprob, X, Y, W, rows, cols)) < TOL
+    assert not out["Z"][11].any()
+    bt = tperm if det else (junk if g.grouped_backward else None)
+    out = emu.run_conv(g, bwd, X, Y, W, rows, cols, G=G, tperm=bt, ws_bytes=ws(nnz, nodes))
+    for got, ref in zip((out["Xg"], out["Yg"], out["Wg"]), otp.conv_backward(oprob, X, Y, W, G, rows, cols)):
+        assert rel_err(got, ref) < TOL
+
+
+def test_conv_long_node_of_more_pieces_than_one_group():
+    """A receiver with 1250 of 1600 edges among 100 nodes: 40 pieces of 32 edges, added in two levels (groups of
+    32 pieces, then the two groups)."""
+    prob, oprob = common.channelwise(common.NEQUIP)
+    g = UVUDetGenerator(prob)
+    nodes, nnz = 100, 1600
+    rows, cols = common.hub_graph(nodes, nnz, 23, hub_in=41, hub_out=17, in_edges=1250, out_edges=0)
+    rows, cols, tperm, _ = otp.coord_graph(rows, cols)
+    assert g.piece_tiles(nnz, nodes) == 50 and (rows == 41).sum() > 32 * g.PIECE_GROUP
+    X, Y, W, G = common.conv_inputs(prob, nodes, nnz, 24)
+    fwd, _, ws = g.plan()
+    out = emu.run_conv(g, fwd, X, Y, W, rows, cols, tperm=tperm, ws_bytes=ws(nnz, nodes))
+    assert rel_err(out["Z"], otp.conv_forward(oprob, X, Y, W, rows, cols)) < TOL
+
+
 @pytest.mark.parametrize("staged", [True, False])
 def test_conv_det_long_edge_lists(staged):
     """Edge lists of about 13 edges per node (6-7 iterations of two sub-lists) reach the steady state of

@@ -46,7 +46,12 @@ def test_launch_plans():
     assert [s["kernel"] for s in bwd] == ["prep_backward", "order_backward", "backward", "backward_dy_reduce"]
     assert bwd[1]["num_blocks"] == 1
     flags = 8 + 4 * 4                                                   # one int per 256 edges (+ alignment slack)
-    assert ws(1000, 10) == 2 * 11 * 8 + 10 * 8 + 4 * 1000 * 16 * 4 + flags       # pointers | node order | dY partials | flags
+    main = 2 * 11 * 8 + 10 * 8 + 4 * 1000 * 16 * 4 + flags               # pointers | node order | dY partials | flags
+    tiles = -(-1000 // 200)                                             # long nodes: pieces of twice the mean of 100 edges
+    pieces = 256 + ((16 * 4 * tiles + 255) & ~255) + 2 * tiles * g.D3 * 4   # four counters per tile and chunk | two partial rows per tile
+    assert fwd[1]["grid_kind"] == bwd[2]["grid_kind"] == 3 and fwd[1]["num_blocks"] == g.LONG == 2
+    assert ws(1000, 10) == ((main + 255) & ~255) + pieces
+    assert g.forward_workspace_model() == (8, 8, 0)                     # the forward alone, every node walked whole
     prob, _ = common.fully_connected(common.DENSE)
     fwd, bwd, ws = UVWGenerator(prob).plan()
     assert [s["kernel"] for s in bwd] == ["prep_backward", "backward", "backward_dw", "backward_reduce"]
@@ -123,8 +128,8 @@ def test_staged_conv_selection(monkeypatch):
 
 def test_unsorted_conv_backward_selection(monkeypatch):
     """Unsorted edge lists: the backward scatters dX with atomics while a row of X is very short, and groups
-    the edges by sender (four more grouping launches, the segmented backward, larger workspace) from
-    128 values per edge on."""
+    the edges by sender (three more grouping launches - the first of them only clears counters and may be
+    skipped -, the segmented backward, larger workspace) from 128 values per edge on."""
     from openequivariance_amd.codegen.uvu_sorted import UVUSortedGenerator
     from openequivariance_amd.problem import ChannelwiseTPP
     from openequivariance_amd import tunables
@@ -135,14 +140,20 @@ def test_unsorted_conv_backward_selection(monkeypatch):
     assert not small.grouped_backward and large.grouped_backward
     _, bwd, ws = small.plan()
     assert [s["kernel"] for s in bwd] == ["backward"]
-    assert ws(1000, 10) == (2 * 11 + 1000) * 8
-    _, bwd, ws = large.plan()
-    assert [s["kernel"] for s in bwd] == ["group_clear_backward", "group_count_backward", "group_scan_backward",
-                                          "group_fill_backward", "order_backward", "backward", "backward_dy_reduce"]
-    assert bwd[5]["grid_y"] == 4 and bwd[5]["work_per_block"] == 1
+    group = (3 * 11 + 1000 + 1) * 8           # pointers, cursors, counters (11 each), position list, ticket
+    tiles = -(-1000 // 200)                   # pieces of 2 x the mean of 100 edges per node
+    pieces = lambda g, chunks: 256 + ((16 * chunks * tiles + 255) & ~255) + 2 * tiles * max(g.D1, g.D3) * 4
+    assert ws(1000, 10) == ((group + 255) & ~255) + pieces(small, 1)
+    fwd, bwd, ws = large.plan()
+    assert [s["kernel"] for s in fwd] == ["group_clear", "group_count", "group_fill", "forward"]
+    assert [bool(s.get("counter_clear")) for s in fwd] == [True, False, False, False]
+    assert [s["kernel"] for s in bwd] == ["group_clear_backward", "group_count_backward", "group_fill_backward",
+                                          "order_backward", "backward", "backward_dy_reduce"]
+    assert bwd[4]["grid_y"] == 4 and bwd[4]["work_per_block"] == 1 and bwd[4]["grid_kind"] == 3
     # the forward's grouping and the backward's lie side by side (a prepared workspace serves both)
-    assert ws(1000, 10) == (2 * (2 * 11 + 1000) + 10) * 8 + 4 * 1000 * 16 * 4 + 8 + 4 * 4
-    assert all(s.get("prep") for s in bwd[:5]) and not any(s.get("prep") for s in bwd[5:])
+    main = 2 * group + 10 * 8 + 4 * 1000 * 16 * 4 + 8 + 4 * 4
+    assert ws(1000, 10) == ((main + 255) & ~255) + pieces(large, 4)
+    assert all(s.get("prep") for s in bwd[:4]) and not any(s.get("prep") for s in bwd[4:])
     src = large.render()
     for name in ("group_fill_backward", "backward_dy_reduce", "void backward("):
         assert name in src
@@ -160,7 +171,8 @@ def test_backward_split_over_output_block_groups():
     assert sorted(sum(mace.out_groups, [])) == mace.used_out and all(mace.out_groups)
     _, bwd, ws = mace.plan()
     assert [s["kernel"] for s in bwd] == ["prep_backward", "order_backward", "backward", "backward_g1", "backward_dy_reduce"]
-    assert ws(1000, 10) == (2 * 11 + 10) * 8 + 4 * 1000 * 16 * 4 + 8 + 4 * 4
+    assert mace.main_bytes(1000, 10) == (((2 * 11 + 10) * 8 + 4 * 1000 * 16 * 4 + 8 + 4 * 4) + 255) & ~255
+    assert ws(1000, 10) == mace.main_bytes(1000, 10) + mace.piece_bytes(1000, 10)
     src = mace.render()
     assert "void backward_g1(" in src and "c * 2 + 1" in src
     with mace._group(1):
