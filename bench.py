@@ -319,6 +319,235 @@ def stream_calibration():
     print(json.dumps(out))
 
 
+
+# ---------------------------------------------------------------------------------------------------
+# Probe: would a banded, channel-sliced sender-order backward of the large convolution move fewer bytes
+# across the fabric?  Stand-in kernels with the real access shapes of config 5 (13 paths, 256 channels,
+# dZ rows of 11 008 words, W rows of 3 328) and sum arithmetic.
+MUL = 256
+# (in1 block, out words D, Z column start, W column start)
+PATHS = [(0, 1, 0, 0), (1, 1, 256, 256), (2, 1, 512, 512),
+         (0, 3, 768, 768), (1, 3, 1536, 1024), (1, 3, 2304, 1280), (2, 3, 3072, 1536), (2, 3, 3840, 1792),
+         (0, 5, 4608, 2048), (1, 5, 5888, 2304), (1, 5, 7168, 2560), (2, 5, 8448, 2816), (2, 5, 9728, 3072)]
+IN1 = [(0, 1), (256, 3), (1024, 5)]      # offset, D
+D1, D3, WN, D2 = 2304, 11008, 3328, 16
+
+
+def band_probe_source(S, group, name, nt=1, dyw=1, noG=0, noW=0, noX=0):
+    """Wavefront = (band k of receivers -> XCD k mod 8, slice j of S channels, tile of senders); lane group
+    sub (64 / S groups) walks a contiguous run of senders of band k in (band, sender, receiver) order, keeps
+    the sender's dX partial in registers, gathers the dZ slice of each edge's receiver (from the band: a
+    working set of N / K receivers x S channels x 43 words per XCD), streams the W slice in and the dW slice
+    out.  noG = 1 gathers from 8 rows only (every gather hits cache), 2 drops the gathers; noW drops the W
+    loads (1), the dW stores (2) or both (3); noX the X loads; dyw = 0 the dY partial stores."""
+    paths = [p for p in PATHS if group is None or p[0] in group]
+    blocks = sorted({p[0] for p in paths})
+    R = 64 // S
+    L = []
+    A = L.append
+    A("typedef long long i64; typedef unsigned long long u64;")
+    A("static __device__ __forceinline__ float ldnt(const float* p) { return %s; }" % ("__builtin_nontemporal_load(p)" if nt else "*p"))
+    A("static __device__ __forceinline__ void stnt(float* p, float v) { %s; }" % ("__builtin_nontemporal_store(v, p)" if nt else "*p = v"))
+    A(f'extern "C" __global__ __launch_bounds__(64) void {name}(const float* __restrict__ X, float* __restrict__ Xp, const float* __restrict__ W, float* __restrict__ Wg,')
+    A("    const float* __restrict__ G, const float* __restrict__ Y, float* __restrict__ Yp, const i64* __restrict__ blist, const i64* __restrict__ bptr,")
+    A("    const i64* __restrict__ rows, const i64* __restrict__ cols, u64 nnz, u64 N, int K, int SPG, int NSL, int tiles)")
+    A("{")
+    A(f"  const int lane = threadIdx.x, sub = lane / {S}, ul = lane % {S};")
+    A("  const u64 bid = blockIdx.x; const int xcd = (int)(bid & 7); const u64 turn = bid >> 3;")
+    A("  const int phases = K / 8;")
+    A("  const u64 per_xcd = (u64)NSL * phases * tiles; if (turn >= per_xcd) return;")
+    A("  const int j = (int)(turn / ((u64)phases * tiles)); const u64 rem = turn % ((u64)phases * tiles);")
+    A("  const int phase = (int)(rem / tiles); const u64 tile = rem % tiles; const int k = phase * 8 + xcd;")
+    A(f"  u64 sa = (tile * {R} + sub) * (u64)SPG; if (sa > N) sa = N; u64 sb = sa + SPG; if (sb > N) sb = N;")
+    A("  const i64 pa = bptr[(u64)k * (N + 1) + sa], pb = bptr[(u64)k * (N + 1) + sb];")
+    A("  const int len = (int)(pb - pa); int maxlen = len;")
+    for m in (32, 16, 8, 4, 2, 1):
+        if m >= S:
+            A(f"  maxlen = max(maxlen, __shfl_xor(maxlen, {m}, 64));")
+    A(f"  const int u = j * {S} + ul;")
+    names = []
+    for t, (b, D, zo, wo) in enumerate(paths):
+        names += [f"g{t}_{d}" for d in range(D)] + [f"w{t}"]
+    for b in blocks:
+        names += [f"x{b}_{d}" for d in range(IN1[b][1])]
+    names += ["yv"]
+    A("  float " + ", ".join(f"N{n} = 0.f" for n in names) + ";")
+    for b in blocks:
+        A("  float " + ", ".join(f"dx{b}_{d} = 0.f" for d in range(IN1[b][1])) + ";")
+    A("  u64 Ie0 = 0, Ie1 = 0, Ir0 = 0, Ir1 = 0, Is0 = 0, Is1 = 0; bool Iv0 = false, Iv1 = false; i64 cur_s = -1;")
+
+    def idx(it, q):
+        A(f"  {{ const bool ev = ({it}) < len; const u64 pos = ev ? (u64)(pa + ({it})) : (u64)(nnz - 1); const u64 e = (u64)blist[pos];")
+        A(f"    Ie{q} = e; Iv{q} = ev; Ir{q} = " + ("(u64)(rows[e] & 7)" if noG == 1 else "(u64)rows[e]") + f";  Is{q} = (u64)cols[e]; }}")
+
+    def load(q):
+        A(f"  {{ const u64 e = Ie{q}, r = Ir{q}, s = Is{q};")
+        A(f"    const float* __restrict__ Wr = W + e * {WN}; const float* __restrict__ Gr = G + r * {D3}; const float* __restrict__ Xr = X + s * {D1};")
+        A(f"    Nyv = ldnt(Y + e * {D2} + (ul & 15));")
+        for t, (b, D, zo, wo) in enumerate(paths):
+            if noW & 1:
+                A(f"    Nw{t} = Nyv;")
+            else:
+                A(f"    Nw{t} = ldnt(Wr + {wo} + u);")
+        for t, (b, D, zo, wo) in enumerate(paths):
+            if noG == 2:
+                A("    " + " ".join(f"Ng{t}_{d} = Nyv;" for d in range(D)))
+            else:
+                A(f"    {{ const float* __restrict__ p_ = Gr + {zo} + u * {D}; " + " ".join(f"Ng{t}_{d} = p_[{d}];" for d in range(D)) + " }")
+        for b in blocks:
+            off, D = IN1[b]
+            if noX:
+                A("    " + " ".join(f"Nx{b}_{d} = Nyv;" for d in range(D)))
+            else:
+                A(f"    {{ const float* __restrict__ p_ = Xr + {off} + u * {D}; " + " ".join(f"Nx{b}_{d} = p_[{d}];" for d in range(D)) + " }")
+        A("  }")
+
+    def flush():
+        A("    if (cur_s >= 0) {")
+        A(f"      float* __restrict__ q_ = Xp + ((u64)k * N + (u64)cur_s) * {D1};")
+        for b in blocks:
+            off, D = IN1[b]
+            for d in range(D):
+                A(f"      q_[{off} + u * {D} + {d}] = dx{b}_{d}; dx{b}_{d} = 0.f;")
+        A("    }")
+    A("  if (maxlen > 0) {")
+    idx("0", 0)
+    load(0)
+    A("  }")
+    A("  if (maxlen > 1) {")
+    idx("1", 1)
+    A("  }")
+    A("  for (int it = 0; it < maxlen; it += 2) {")
+    for h in (0, 1):
+        if h == 1:
+            A("    if (it + 1 >= maxlen) break;")
+        A("    {")
+        A("    const float " + ", ".join(f"{n} = N{n}" for n in names) + ";")
+        A(f"    const u64 e = Ie{h}; const bool ev = Iv{h}; const i64 s = ev ? (i64)Is{h} : cur_s;")
+        A(f"    if (it + {h + 1} < maxlen) {{")
+        load(1 - h)
+        A("    }")
+        A(f"    if (it + {h + 2} < maxlen) {{")
+        idx(f"it + {h + 2}", h)
+        A("    }")
+        A("    if (s != cur_s) {")
+        flush()
+        A("      cur_s = s; }")
+        A("    float dy = 0.f;")
+        for t, (b, D, zo, wo) in enumerate(paths):
+            bd = IN1[b][1]
+            A(f"    {{ float sg = " + " + ".join(f"g{t}_{d}" for d in range(D)) + f"; float dw = sg * x{b}_0 * yv; ")
+            if noW & 2:
+                A(f"      if (ev && dw == 1.2345f) stnt(Wg + e * {WN} + {wo} + u, dw);")
+            else:
+                A(f"      if (ev) stnt(Wg + e * {WN} + {wo} + u, dw);")
+            A("      " + " ".join(f"dx{b}_{d} = __builtin_fmaf(sg * w{t}, yv, dx{b}_{d});" for d in range(bd)) + f" dy += sg * w{t}; }}")
+        if dyw:
+            for m in (8, 4, 2, 1):
+                A(f"    dy += __shfl_xor(dy, {m}, 64);")
+            A(f"    if (ev && ul < 16) Yp[((u64)(j * 3 + {0 if group is None else group[0]}) * nnz + e) * 16 + ul] = dy;")
+        A("    }")
+    A("  }")
+    A("  if (true) {")
+    flush()
+    A("  }")
+    A("}")
+    return "\n".join(L)
+
+
+
+
+def conv_band_probe():
+    """Times the stand-in for slices of 16 / 32 / 64 channels and 8 / 16 / 32 receiver bands, and - to see what
+    bounds the loop - with parts of the traffic switched off.  The sender-order backward it would replace
+    takes 7.5 ms on the same graph."""
+    import ctypes as C
+    import torch
+    from openequivariance_amd import runtime as rt
+    torch.manual_seed(0)
+    dev = torch.device("cuda:0")
+    N, deg = 20000, 40
+    rows = torch.repeat_interleave(torch.arange(N), torch.poisson(torch.full((N,), float(deg))).long())
+    E = rows.numel()
+    cols = torch.randint(0, N, (E,))
+    rows, cols = rows.to(dev), cols.to(dev)
+    W = torch.empty(E * WN, device=dev).normal_()
+    Wg = torch.empty(E * WN, device=dev)
+    G = torch.empty(N * D3, device=dev).normal_()
+    X = torch.empty(N * D1, device=dev).normal_()
+    Y = torch.empty(E * D2, device=dev).normal_()
+    stream = torch.cuda.current_stream().cuda_stream
+    modes = dict(full={}, gathers_always_hit=dict(noG=1), no_W_no_dW=dict(noW=3), no_gathers=dict(noG=2),
+                 only_W_loads=dict(noG=2, noX=1, dyw=0, noW=2), only_dW_stores=dict(noG=2, noX=1, dyw=0, noW=1),
+                 only_W_and_dW=dict(noG=2, noX=1, dyw=0))
+    variants = [(S, K, "full") for S in (16, 32, 64) for K in (8, 16, 32)] + [(64, 16, m) for m in modes if m != "full"] \
+        + [(16, 32, "no_W_no_dW")]
+    out = {"workload": "conv_band_probe", "edges": E, "nodes": N, "unit": "ms per backward-equivalent",
+           "sender_order_backward_ms": 7.5, "variants": []}
+    compiled = {}
+    for S, K, mode in variants:
+        R, NSL, SPG = 64 // S, MUL // S, 8
+        band = rows // ((N + K - 1) // K)
+        blist = torch.argsort((band * N + cols) * N + rows)
+        kk = (band * N + cols)[blist]
+        q = torch.arange(K, device=dev).repeat_interleave(N + 1) * N + torch.arange(N + 1, device=dev).repeat(K)
+        bptr = torch.searchsorted(kk, q).contiguous()
+        Xp = torch.empty(K * N * D1, device=dev)
+        Yp = torch.empty(NSL * 3 * E * 16, device=dev)
+        tiles = (N + R * SPG - 1) // (R * SPG)
+        if (S, mode) not in compiled:
+            compiled[(S, mode)] = rt.Module(rt.compile_source(band_probe_source(S, None, "probe", **modes[mode])))
+        grid = 8 * NSL * (K // 8) * tiles
+        args = [C.c_void_p(t.data_ptr()) for t in (X, Xp, W, Wg, G, Y, Yp, blist, bptr, rows, cols)] + \
+               [C.c_uint64(E), C.c_uint64(N), C.c_int(K), C.c_int(SPG), C.c_int(NSL), C.c_int(tiles)]
+        best = float("inf")
+        for rep in range(4):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            compiled[(S, mode)].launch("probe", grid, 64, args, stream=stream)
+            b.record()
+            b.synchronize()
+            if rep >= 1:
+                best = min(best, a.elapsed_time(b))
+        out["variants"].append({"channels_per_slice": S, "receiver_bands": K, "mode": mode, "ms": round(best, 3),
+                                "dZ_slice_per_XCD_MB": round(N / K * S * 43 * 4 / 1e6, 2)})
+        del Xp, Yp, blist, bptr, kk, q, band
+    print(json.dumps(out))
+
+
+def measure_torch_op(case, ev, steps, warmup, raw_ms):
+    """The operator a user calls (reference protocol: implementations/TensorProductBase.py:114-219 and
+    convolution/ConvolutionBase.py:251-411 time the torch op when torch_op=True): ``steps`` forward +
+    backward passes through the custom ops and autograd, output allocation and argument checks included.
+    Reports the wall clock per step, the HIP-event time of each direction, and what one call costs on the
+    host (time until the call returns, measured with the GPU idle before each call)."""
+    import torch
+    run_f, run_b = case.torch_step
+    for _ in range(max(warmup, 3)):           # (the unsorted operator times its backward variants on first use)
+        run_f()
+        run_b()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        ev.wrap("torch_forward", run_f)
+        ev.wrap("torch_backward", run_b)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    host = {"forward": [], "backward": []}
+    for _ in range(min(steps, 20)):
+        for name, fn in (("forward", run_f), ("backward", run_b)):
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            fn()
+            host[name].append((time.perf_counter() - t1) * 1e6)
+    torch.cuda.synchronize()
+    f_ms, b_ms = ev.mean_ms("torch_forward"), ev.mean_ms("torch_backward")
+    med = lambda v: sorted(v)[len(v) // 2]
+    return {"ms_per_step": round(wall_ms, 5), "forward_ms": round(f_ms, 5), "backward_ms": round(b_ms, 5),
+            "host_us_per_call": {"forward": round(med(host["forward"]), 1), "backward": round(med(host["backward"]), 1)},
+            "vs_raw_entry_points": round(wall_ms / raw_ms, 3) if raw_ms > 0 else None}
+
+
 def measure(name, steps, warmup, cold=True, cpu=True, cpu_sample=0, ceiling=True, cpu_seconds=10.0):
     """Build one workload, time ``steps`` forward+backward steps after ``warmup`` untimed ones and
     return (workload, record): whole-job throughput from the wall clock around the timed region, and
@@ -398,20 +627,34 @@ def measure(name, steps, warmup, cold=True, cpu=True, cpu_sample=0, ceiling=True
             "backward_ms_median": round(bm, 5), "backward_ms_min": round(bmin, 5),
             "fwd_bwd_frac": round((work["forward"] + work["backward"]) / ((fm + bm) * 1e-3) / scale / peak, 4)}
 
-    if case.forward_with_prep is not None:
-        # the timed launches reuse the graph preparation left in the workspace, as the layers of a model
-        # do; the same launches including the preparation, for callers that see every graph once
+    if wl.min_traffic:
+        # compulsory bytes + the per-edge rows any schedule must gather (or spill) when no cache holds them
+        mt = wl.min_traffic
+        roofline["min_traffic"] = dict(mt)
+        roofline["min_traffic_rate_GBs"] = {"forward": round(mt["forward"] / (fwd_ms * 1e-3) / 1e9, 1),
+                                            "backward": round(mt["backward"] / (bwd_ms * 1e-3) / 1e9, 1)}
+
+    if case.forward_prepared is not None:
+        # the timed launches prepare the graph on every call (the operators' default: a caller may hand over
+        # a new graph each time); the same launches with the preparation reused from the workspace, the
+        # regime of an operator built with graph_cache=True inside a model that calls one graph many times
         for _ in range(min(steps, 10)):
-            ev.wrap("forward_with_prep", case.forward_with_prep)
-            ev.wrap("backward_with_prep", case.backward_with_prep)
+            ev.wrap("forward_prepared", case.forward_prepared)
+            ev.wrap("backward_prepared", case.backward_prepared)
         torch.cuda.synchronize()
-        roofline["with_graph_preparation"] = {"forward_ms": round(ev.mean_ms("forward_with_prep"), 5),
-                                              "backward_ms": round(ev.mean_ms("backward_with_prep"), 5)}
+        fp, bp = ev.mean_ms("forward_prepared"), ev.mean_ms("backward_prepared")
+        roofline["prepared_graph"] = {"forward_ms": round(fp, 5), "backward_ms": round(bp, 5),
+                                      "fwd_bwd_frac": round((work["forward"] + work["backward"]) / ((fp + bp) * 1e-3) / scale / peak, 4)}
         case.forward()
         case.backward()
 
+    torch_op = None
+    if case.torch_step is not None:
+        torch_op = measure_torch_op(case, ev, steps, warmup, fwd_ms + bwd_ms)
+
     rec = {"value": round(value, 1), "unit": wl.unit, "ms_per_step": round(ms_per_step, 5), "dtype": wl.dtype,
            "data": wl.data_note, "config": {"workload": wl.description, **wl.config}, "roofline": roofline,
+           "torch_op": torch_op,
            "cpu_baseline": cpu_baseline(wl, case, cpu_sample, cpu_seconds) if cpu else None}
     del case
     torch.cuda.empty_cache()
@@ -431,6 +674,9 @@ def main():
     if args.workload == "stream_calibration":
         stream_calibration()
         return
+    if args.workload == "conv_band_probe":
+        conv_band_probe()
+        return
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (the path shards over rows/edges "
               "without communication and is measured on one)", file=sys.stderr)
@@ -447,7 +693,7 @@ def main():
            "value": rec["value"], "unit": rec["unit"], "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
            "ms_per_step": rec["ms_per_step"], "higher_is_better": True, "scaling": "weak",
            "vs_baseline": None, "dtype": rec["dtype"], "data": rec["data"], "config": rec["config"],
-           "roofline": rec["roofline"], "cpu_baseline": rec["cpu_baseline"],
+           "roofline": rec["roofline"], "torch_op": rec["torch_op"], "cpu_baseline": rec["cpu_baseline"],
            "device": torch.cuda.get_device_name(0)}
     if not args.workload and not args.headline_only:
         # the other BASELINE configurations, same protocol (same steps and warm-up, HIP events around every
@@ -467,7 +713,8 @@ def main():
                                 "algorithmic_per_launch": rf["algorithmic"],
                                 "traffic": {"forward": load_traffic(f"{name}:forward"), "backward": load_traffic(f"{name}:backward")},
                                 "flushed_caches": rf.get("flushed_caches"),
-                                "with_graph_preparation": rf.get("with_graph_preparation"), "cpu_baseline": r["cpu_baseline"],
+                                "prepared_graph": rf.get("prepared_graph"), "min_traffic": rf.get("min_traffic"),
+                                "torch_op": r.get("torch_op"), "cpu_baseline": r["cpu_baseline"],
                                 "bench_seconds": None}
             except Exception as exc:          # one workload failing must not hide the others
                 others[name] = {"error": f"{type(exc).__name__}: {exc}"}

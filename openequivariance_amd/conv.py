@@ -28,7 +28,7 @@ from .codegen.uvu_direct import UVUDirectGenerator
 from .codegen.uvu_recv import UVURecvGenerator
 from .codegen.uvu_sorted import UVUSortedGenerator
 from .problem import TPProblem
-from .tensor_product import _make_steps, validate_problem
+from .tensor_product import _contiguous, _make_steps, _on_device, validate_problem
 from .weight_order import WeightReorder
 from .wigner import wigner_3j
 
@@ -156,6 +156,8 @@ class TensorProductConv:
         # reference: LoopUnrollConv.py:53,78 (idx_type_map = {np.int32: "int", np.int64: "long"})
         self.idx_dtype = np.dtype(idx_dtype).type
         self._torch_idx = torch.int64 if self.idx_dtype == np.int64 else torch.int32
+        self._torch_dtype = {np.float32: torch.float32, np.float64: torch.float64}[config.irrep_dtype]
+        self._dims = (self.L1.dim, self.L2.dim, self.L3.dim, config.weight_numel)
         self.conv_id = TensorProductConv.next_conv_id
         TensorProductConv.next_conv_id += 1
 
@@ -174,8 +176,9 @@ class TensorProductConv:
         self.backward_needs_tperm = deterministic
         self.jit_kernel = self.generator.render()
         self._ws_fns = []
+        self._ws_last = (None, 0)          # (sizes, bytes) of the last workspace query
         self.internal = self._build(self.generator, self.jit_kernel)
-        self._workspaces: typing.Dict[int, _StreamWorkspace] = {}
+        self._workspaces: typing.Dict[tuple, _StreamWorkspace] = {}      # (device, stream) -> scratch
         # Unsorted edge lists: whether the backward scatters dX with float atomics or groups the edges by
         # sender first depends on the row length AND on the graph (atomics per edge against the gathers of
         # the segmented kernel); the generator's rule of thumb is only the starting point.  The torch
@@ -212,7 +215,10 @@ class TensorProductConv:
         return impl
 
     def _ws_bytes(self, nnz: int, node_count: int) -> int:
-        return max(f(nnz, node_count) for f in self._ws_fns)
+        key = (nnz, node_count, len(self._ws_fns))
+        if key != self._ws_last[0]:
+            self._ws_last = (key, max(f(nnz, node_count) for f in self._ws_fns))
+        return self._ws_last[1]
 
     def _backward_variant(self, name: str):
         """(kernel set, whether its backward overwrites dX) of a backward variant of the unsorted operator,
@@ -236,7 +242,8 @@ class TensorProductConv:
         lists.  A buffer that has been outgrown is freed unless a HIP graph capture has used it: a captured
         graph has the address baked in, so such buffers stay alive as long as the operator (the reference
         allocates its workspace once at a fixed size: ConvolutionBase.py:93-100)."""
-        sid = self._stream() if stream is None else int(stream)
+        dev = torch.cuda.current_device()
+        sid = (dev, self._stream(dev) if stream is None else int(stream))
         rec = self._workspaces.get(sid)
         if rec is None:
             rec = self._workspaces[sid] = _StreamWorkspace()
@@ -245,7 +252,7 @@ class TensorProductConv:
             if rec.captured and rec.buffer is not None:
                 rec.retired.append(rec.buffer)
             rec.size = int(need * 1.25) + 256
-            rec.buffer = torch.empty(rec.size, dtype=torch.uint8, device="cuda")
+            rec.buffer = torch.empty(rec.size, dtype=torch.uint8, device=f"cuda:{dev}")
             rec.fwd_key = rec.bwd_key = rec.zero_fwd = rec.zero_bwd = None
             rec.refs.clear()
         return rec
@@ -259,40 +266,50 @@ class TensorProductConv:
         return self._workspace_record(nnz, node_count, stream).buffer.data_ptr()
 
     @staticmethod
-    def _stream() -> int:
-        return torch.cuda.current_stream().cuda_stream
+    def _stream(device_index: typing.Optional[int] = None) -> int:
+        """torch's current stream on the device as a raw handle (the binding call is many times cheaper than
+        building a torch.cuda.Stream object per launch)."""
+        return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device() if device_index is None else device_index)
 
     def _check(self, x, y, w, rows, cols, tperm=None, g=None):
         """Shapes, dtypes and devices, before anything is launched: the kernels dereference every
         pointer they are handed, so a host tensor or a tensor of another GPU must never reach them."""
         E, N = rows.shape[0], x.shape[0]
+        d1, d2, d3, wn = self._dims
         if N >= 2 ** 31:
             raise ValueError("node count must be below 2^31")
-        if x.ndim != 2 or x.shape[1] != self.L1.dim:
-            raise ValueError(f"L1_in must have shape [nodes, {self.L1.dim}], got {tuple(x.shape)}")
-        if tuple(y.shape) != (E, self.L2.dim):
-            raise ValueError(f"L2_in must have shape [{E}, {self.L2.dim}], got {tuple(y.shape)}")
-        if tuple(w.shape) != (E, self.config.weight_numel):
-            raise ValueError(f"weights must have shape [{E}, {self.config.weight_numel}], got {tuple(w.shape)}")
-        if g is not None and tuple(g.shape) != (N, self.L3.dim):
-            raise ValueError(f"L3_grad must have shape [{N}, {self.L3.dim}], got {tuple(g.shape)}")
+        if x.ndim != 2 or x.shape[1] != d1:
+            raise ValueError(f"L1_in must have shape [nodes, {d1}], got {tuple(x.shape)}")
+        if y.shape != (E, d2):
+            raise ValueError(f"L2_in must have shape [{E}, {d2}], got {tuple(y.shape)}")
+        if w.shape != (E, wn):
+            raise ValueError(f"weights must have shape [{E}, {wn}], got {tuple(w.shape)}")
+        if g is not None and g.shape != (N, d3):
+            raise ValueError(f"L3_grad must have shape [{N}, {d3}], got {tuple(g.shape)}")
         if self.deterministic and tperm is None:
             raise ValueError("the deterministic convolution needs transpose_perm")
-        index = (("rows", rows), ("cols", cols)) + ((("transpose_perm", tperm),) if tperm is not None else ())
-        for name, t in index:
-            if t.dtype != self._torch_idx or tuple(t.shape) != (E,):
-                raise TypeError(f"{name} must be an {self._torch_idx} tensor of shape [{E}]")
-        tdt = {np.float32: torch.float32, np.float64: torch.float64}[self.config.irrep_dtype]
-        data = (("L1_in", x), ("L2_in", y), ("weights", w)) + ((("L3_grad", g),) if g is not None else ())
-        for name, t in data:
+        dev, tdt, idt = x.device, self._torch_dtype, self._torch_idx
+        for name, t in (("rows", rows), ("cols", cols), ("transpose_perm", tperm)):
+            if t is None:
+                continue
+            if t.dtype != idt or t.shape != (E,):
+                raise TypeError(f"{name} must be an {idt} tensor of shape [{E}]")
+            if t.device != dev or not t.is_cuda:
+                self._device_error(name, t, x)
+        for name, t in (("L1_in", x), ("L2_in", y), ("weights", w), ("L3_grad", g)):
+            if t is None:
+                continue
             if t.dtype != tdt:
                 raise TypeError(f"tensors must be {tdt}")
-        for name, t in data + index:
-            if not t.is_cuda:
-                raise ValueError(f"{name} is on {t.device}: every tensor, index tensors included, must be on the GPU "
-                                 "(there is no CPU implementation)")
-            if t.device != x.device:
-                raise ValueError(f"{name} is on {t.device}, L1_in on {x.device}: all tensors must share one device")
+            if t.device != dev or not t.is_cuda:
+                self._device_error(name, t, x)
+
+    @staticmethod
+    def _device_error(name, t, x):
+        if not t.is_cuda:
+            raise ValueError(f"{name} is on {t.device}: every tensor, index tensors included, must be on the GPU "
+                             "(there is no CPU implementation)")
+        raise ValueError(f"{name} is on {t.device}, L1_in on {x.device}: all tensors must share one device")
 
     def _pick(self, *ptrs):
         """The forward kernels write Z with 16-byte vector stores; a misaligned tensor (rare: a view
@@ -364,7 +381,8 @@ class TensorProductConv:
         self.last_tuning = best
         return min(best, key=best.get)
 
-    def _cached_call(self, which: str, rows, cols, tperm, E: int, N: int, launch, tag: str = "") -> None:
+    def _cached_call(self, which: str, rows, cols, tperm, E: int, N: int, launch, tag: str = "",
+                     stream: typing.Optional[int] = None) -> None:
         """Run ``launch(workspace pointer, prepared, counters_zero)`` for the torch operators.  The graph preparation a
         call leaves in the stream's workspace is reused by the next call of the same direction when it
         names the same graph: same index tensors (address and in-place version counter), same sizes.  The
@@ -374,7 +392,7 @@ class TensorProductConv:
         if self._ws_bytes(E, N) == 0:
             launch(0, False, False)
             return
-        rec = self._workspace_record(E, N)
+        rec = self._workspace_record(E, N, stream)
         if torch.cuda.is_current_stream_capturing():
             rec.captured = True
         key = None
@@ -402,17 +420,17 @@ class TensorProductConv:
         cid = self.conv_id
 
         def fwd_impl(L1_in, L2_in, weights, rows, cols, tperm):
-            x, y, w = L1_in.contiguous(), L2_in.contiguous(), weights.contiguous()
-            rows, cols = rows.contiguous(), cols.contiguous()
-            tperm = tperm.contiguous() if tperm is not None else None
+            x, y, w, rows, cols, tperm = _contiguous(L1_in, L2_in, weights, rows, cols, tperm)
             self._check(x, y, w, rows, cols, tperm)
             E, N = rows.shape[0], x.shape[0]
             # the atomic kernels accumulate into Z; the deterministic ones write every row
             out = (torch.empty if self.forward_overwrites else torch.zeros)((N, L3_dim), dtype=x.dtype, device=x.device)
-            with torch.cuda.device(x.device):
+            with _on_device(x.device):
+                stream = self._stream(x.device.index)
                 self._cached_call("fwd", rows, cols, tperm, E, N, lambda ws, prepared, zero: self.exec_conv_rawptrs(
                     x.data_ptr(), y.data_ptr(), w.data_ptr(), out.data_ptr(), rows.data_ptr(), cols.data_ptr(), E, N,
-                    ws, tperm.data_ptr() if tperm is not None else 0, prepared=prepared, counters_zero=zero))
+                    ws, tperm.data_ptr() if tperm is not None else 0, stream=stream, prepared=prepared,
+                    counters_zero=zero), stream=stream)
             return out
 
         def bwd_run(x, y, w, g, rows, cols, tperm, E, N, variant=None):
@@ -422,19 +440,18 @@ class TensorProductConv:
                 impl, overwrites, variant = None, self.backward_overwrites, None     # misaligned views: the default set only
             xg = (torch.empty_like if overwrites else torch.zeros_like)(x)
             yg, wg = torch.empty_like(y), torch.empty_like(w)
+            stream = self._stream(x.device.index)
             self._cached_call("bwd", rows, cols, tperm, E, N, lambda ws, prepared, zero: self.backward_rawptrs(
                 x.data_ptr(), xg.data_ptr(), y.data_ptr(), yg.data_ptr(), w.data_ptr(), wg.data_ptr(), g.data_ptr(),
                 rows.data_ptr(), cols.data_ptr(), E, N, ws, tperm.data_ptr() if tperm is not None else 0,
-                prepared=prepared, impl=impl, counters_zero=zero), tag=variant or "")
+                stream=stream, prepared=prepared, impl=impl, counters_zero=zero), tag=variant or "", stream=stream)
             return [xg, yg, wg]
 
         def bwd_impl(L1_in, L2_in, weights, L3_grad, rows, cols, tperm):
-            x, y, w, g = L1_in.contiguous(), L2_in.contiguous(), weights.contiguous(), L3_grad.contiguous()
-            rows, cols = rows.contiguous(), cols.contiguous()
-            tperm = tperm.contiguous() if tperm is not None else None
+            x, y, w, g, rows, cols, tperm = _contiguous(L1_in, L2_in, weights, L3_grad, rows, cols, tperm)
             self._check(x, y, w, rows, cols, tperm, g)
             E, N = rows.shape[0], x.shape[0]
-            with torch.cuda.device(x.device):
+            with _on_device(x.device):
                 if not self.autotune or E == 0:
                     return bwd_run(x, y, w, g, rows, cols, tperm, E, N)
                 size_class = (E.bit_length(), N.bit_length())

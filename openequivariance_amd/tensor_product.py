@@ -34,6 +34,27 @@ def _make_steps(descs, flags: int = 0):
                          | (rt.STEP_COUNTER_CLEAR if d.get("counter_clear") else 0)) for d in descs]
 
 
+class _NoSwitch:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def _contiguous(*tensors):
+    return tuple(t if t is None or t.is_contiguous() else t.contiguous() for t in tensors)
+
+
+def _on_device(device):
+    """Context that makes ``device`` current: nothing at all when it already is (the usual case; entering
+    torch.cuda.device costs several microseconds per call)."""
+    return _NO_SWITCH if device.index == torch.cuda.current_device() else torch.cuda.device(device)
+
+
 def select_generator(config: TPProblem):
     """The kernel generator of a batch tensor product: MFMA kernels for uvw with shared weights,
     streaming vector-ALU kernels for uvw with per-row weights, the persistent two-stage dW
@@ -97,7 +118,9 @@ class TensorProduct(TensorProductBase):
         self.workspace_bytes = ws()
         self._step_flags = rt.STEP_NEEDS_WORKSPACE if self.workspace_bytes else 0
         self.internal = rt.TPImpl(code, _make_steps(fwd, self._step_flags), _make_steps(bwd, self._step_flags))
-        self._workspaces = {}                 # stream -> scratch tensor (fixed size, never regrown)
+        self._torch_dtype = {np.float32: torch.float32, np.float64: torch.float64}[self.irrep_dtype]
+        self._dims = (self.L1.dim, self.L2.dim, self.L3.dim, config.weight_numel)
+        self._workspaces = {}                 # (device, stream) -> scratch tensor (fixed size, never regrown)
         self._internal_unaligned = None       # kernels without 16-byte vector stores, compiled on first need
 
         self._reorder = WeightReorder(config)
@@ -117,15 +140,17 @@ class TensorProduct(TensorProductBase):
         stream, so that two streams using one operator do not overwrite each other's partial sums."""
         if self.workspace_bytes == 0:
             return 0
-        sid = self._stream() if stream is None else int(stream)
-        buf = self._workspaces.get(sid)
+        dev = torch.cuda.current_device()
+        key = (dev, self._stream(dev) if stream is None else int(stream))
+        buf = self._workspaces.get(key)
         if buf is None:
-            buf = self._workspaces[sid] = torch.empty(self.workspace_bytes, dtype=torch.uint8, device="cuda")
+            buf = self._workspaces[key] = torch.empty(self.workspace_bytes, dtype=torch.uint8, device=f"cuda:{dev}")
         return buf.data_ptr()
 
     @staticmethod
-    def _stream() -> int:
-        return torch.cuda.current_stream().cuda_stream
+    def _stream(device_index: typing.Optional[int] = None) -> int:
+        """torch's current stream on the device as a raw handle."""
+        return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device() if device_index is None else device_index)
 
     def _pick(self, *ptrs):
         aligned = all(int(p) % 16 == 0 for p in ptrs)
@@ -189,11 +214,12 @@ class TensorProduct(TensorProductBase):
 
         @torch.library.custom_op(f"openequivariance_amd::tp_forward{self.tp_id}", mutates_args=(), device_types="cuda")
         def forward(L1_in: torch.Tensor, L2_in: torch.Tensor, weights: torch.Tensor) -> torch.Tensor:
-            x, y, w = L1_in.contiguous(), L2_in.contiguous(), weights.contiguous()
+            x, y, w = _contiguous(L1_in, L2_in, weights)
             self._check_inputs(x, y, w)
             out = torch.empty((x.shape[0], L3_dim), dtype=x.dtype, device=x.device)
-            with torch.cuda.device(x.device):
-                self.forward_raw(x.shape[0], x.data_ptr(), y.data_ptr(), out.data_ptr(), w.data_ptr())
+            with _on_device(x.device):
+                self.forward_raw(x.shape[0], x.data_ptr(), y.data_ptr(), out.data_ptr(), w.data_ptr(),
+                                 self._stream(x.device.index))
             return out
 
         @forward.register_fake
@@ -205,12 +231,12 @@ class TensorProduct(TensorProductBase):
         @torch.library.custom_op(f"openequivariance_amd::tp_grad_helper{self.tp_id}", mutates_args=(), device_types="cuda")
         def backward_helper(L1_in: torch.Tensor, L2_in: torch.Tensor, weights: torch.Tensor,
                             L3_grad: torch.Tensor) -> typing.List[torch.Tensor]:
-            x, y, w, g = L1_in.contiguous(), L2_in.contiguous(), weights.contiguous(), L3_grad.contiguous()
+            x, y, w, g = _contiguous(L1_in, L2_in, weights, L3_grad)
             self._check_inputs(x, y, w, g)
             xg, yg, wg = torch.empty_like(x), torch.empty_like(y), torch.empty_like(w)
-            with torch.cuda.device(x.device):
+            with _on_device(x.device):
                 self.backward_raw(x.shape[0], x.data_ptr(), xg.data_ptr(), y.data_ptr(), yg.data_ptr(),
-                                  w.data_ptr(), wg.data_ptr(), g.data_ptr())
+                                  w.data_ptr(), wg.data_ptr(), g.data_ptr(), self._stream(x.device.index))
             return [xg, yg, wg]
 
         @backward_helper.register_fake
@@ -241,23 +267,25 @@ class TensorProduct(TensorProductBase):
         """Shapes, dtypes and devices, before anything is launched (the kernels dereference every
         pointer they are handed)."""
         B = x.shape[0]
-        if x.ndim != 2 or x.shape[1] != self.L1.dim:
-            raise ValueError(f"L1_in must have shape [batch, {self.L1.dim}], got {tuple(x.shape)}")
-        if tuple(y.shape) != (B, self.L2.dim):
-            raise ValueError(f"L2_in must have shape [{B}, {self.L2.dim}], got {tuple(y.shape)}")
-        want = (self.config.weight_numel,) if self.config.shared_weights else (B, self.config.weight_numel)
-        if tuple(w.shape) != want:
+        d1, d2, d3, wn = self._dims
+        if x.ndim != 2 or x.shape[1] != d1:
+            raise ValueError(f"L1_in must have shape [batch, {d1}], got {tuple(x.shape)}")
+        if y.shape != (B, d2):
+            raise ValueError(f"L2_in must have shape [{B}, {d2}], got {tuple(y.shape)}")
+        want = (wn,) if self.config.shared_weights else (B, wn)
+        if w.shape != want:
             raise ValueError(f"weights must have shape {want}, got {tuple(w.shape)}")
-        if g is not None and tuple(g.shape) != (B, self.L3.dim):
-            raise ValueError(f"L3_grad must have shape [{B}, {self.L3.dim}], got {tuple(g.shape)}")
-        tdt = {np.float32: torch.float32, np.float64: torch.float64}[self.irrep_dtype]
-        data = (("L1_in", x), ("L2_in", y), ("weights", w)) + ((("L3_grad", g),) if g is not None else ())
-        for name, t in data:
+        if g is not None and g.shape != (B, d3):
+            raise ValueError(f"L3_grad must have shape [{B}, {d3}], got {tuple(g.shape)}")
+        dev, tdt = x.device, self._torch_dtype
+        for name, t in (("L1_in", x), ("L2_in", y), ("weights", w), ("L3_grad", g)):
+            if t is None:
+                continue
             if t.dtype != tdt:
                 raise TypeError(f"tensors must be {tdt}")
             if not t.is_cuda:
                 raise ValueError(f"{name} is on {t.device}: all tensors must be on the GPU (there is no CPU implementation)")
-            if t.device != x.device:
+            if t.device != dev:
                 raise ValueError(f"{name} is on {t.device}, L1_in on {x.device}: all tensors must share one device")
 
     # ------------------------------------------------------------------ timing

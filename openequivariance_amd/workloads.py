@@ -49,10 +49,13 @@ class Case:
     forward: Callable[[], None]
     backward: Callable[[], None]
     host: Dict[str, np.ndarray] = field(default_factory=dict)
-    # convolutions: the same launches including the graph preparation (CSR pointers, position lists,
-    # node order), which ``forward`` / ``backward`` reuse from the workspace
-    forward_with_prep: Optional[Callable[[], None]] = None
-    backward_with_prep: Optional[Callable[[], None]] = None
+    # convolutions: ``forward`` / ``backward`` prepare the graph (CSR pointers, position lists, node order) on
+    # every call, as the operators do by default; these reuse the preparation left in the workspace, the
+    # regime of an operator built with graph_cache=True whose layers call one graph many times
+    forward_prepared: Optional[Callable[[], None]] = None
+    backward_prepared: Optional[Callable[[], None]] = None
+    # the operator a user calls: forward through the torch custom op, backward through autograd
+    torch_step: Optional[Callable[[], None]] = None
 
 
 @dataclass
@@ -74,6 +77,7 @@ class Workload:
     w_scale: float = 1.0
     alg_bytes: Dict[str, int] = field(default_factory=dict)
     alg_flops: Dict[str, int] = field(default_factory=dict)
+    min_traffic: Dict[str, int] = field(default_factory=dict)
     # True: X, W and G are drawn on the GPU with torch's generator (the large workload's weights
     # are 10.6 GB; drawing them on the host takes minutes); the graph and Y still come from numpy
     device_inputs: bool = False
@@ -188,6 +192,8 @@ class Workload:
             def bwd():
                 op.backward_raw(n, p["X"], p["Xg"], p["Y"], p["Yg"], p["W"], p["Wg"], p["G"], stream)
             self.units = n
+            leaves = [t[k].detach().requires_grad_(True) for k in ("X", "Y", "W")]
+            torch_step = self._torch_step(op.forward, leaves, (), t["G"])
         else:
             op = TensorProductConv(prob, torch_op=True, deterministic=self.deterministic)
             E, N = h["rows"].size, self.nodes
@@ -201,29 +207,51 @@ class Workload:
             ws = op.workspace_ptr(E, N)
             det = self.deterministic
 
-            def fwd(prepared=True):
+            def fwd(prepared=False, zero=True):
                 if not op.forward_overwrites:
                     t["Z"].zero_()              # atomic kernels accumulate: part of the operator's work
                 op.exec_conv_rawptrs(p["X"], p["Y"], p["W"], p["Z"], p["rows"], p["cols"], E, N, ws, tp_ptr, stream,
-                                     prepared=prepared)
+                                     prepared=prepared, counters_zero=zero)
 
-            def bwd(prepared=True):
+            def bwd(prepared=False, zero=True):
                 if not op.backward_overwrites:
                     t["Xg"].zero_()             # likewise for the backward that scatters dX with atomics
                 op.backward_rawptrs(p["X"], p["Xg"], p["Y"], p["Yg"], p["W"], p["Wg"], p["G"], p["rows"], p["cols"],
-                                    E, N, ws, tp_ptr, stream, prepared=prepared)
-            # a model calls one graph many times (forward, backward and double backward of every layer):
-            # the graph is prepared once, here, and the timed launches reuse the workspace
-            fwd(False)
-            bwd(False)
-            return Case(op, t, fwd, bwd, h, lambda: fwd(False), lambda: bwd(False))
-        return Case(op, t, fwd, bwd, h)
+                                    E, N, ws, tp_ptr, stream, prepared=prepared, counters_zero=zero)
+            # the first calls clear the grouping counters of the (uninitialised) workspace; every call leaves
+            # them zeroed, so the timed ones skip that step, as the torch operator does on its own workspace
+            fwd(zero=False)
+            bwd(zero=False)
+            leaves = [t[k].detach().requires_grad_(True) for k in ("X", "Y", "W")]
+            index = tuple(t[k] for k in ("rows", "cols", "tperm") if k in t)
+            return Case(op, t, fwd, bwd, h, lambda: fwd(True), lambda: bwd(True),
+                        self._torch_step(op.forward, leaves, index, t["G"]))
+        return Case(op, t, fwd, bwd, h, torch_step=torch_step)
+
+    @staticmethod
+    def _torch_step(forward, leaves, index, G):
+        """One forward + backward through the torch operator: returns (run forward, run backward of its result)."""
+        state = {}
+
+        def run_forward():
+            for a in leaves:
+                a.grad = None
+            state["z"] = forward(*leaves, *index)
+
+        def run_backward():
+            state.pop("z").backward(G)
+        return run_forward, run_backward
 
     def _fill_conv_bytes(self, prob, E, N):
         s = 4 if self.dtype == "f32" else 8
         d1, d2, d3, wn = prob.irreps_in1.dim, prob.irreps_in2.dim, prob.irreps_out.dim, prob.weight_numel
         self.alg_bytes = {"forward": E * (d2 + wn) * s + N * (d1 + d3) * s + E * 16,
                           "backward": 2 * E * (d2 + wn) * s + N * (2 * d1 + d3) * s + E * 24}
+        # What a schedule must move when no gathered row is found in a cache: the forward reads X[sender] per
+        # edge; the backward either gathers dZ[receiver] per edge (sender order) or gathers X[sender] and
+        # writes and re-reads a dX row per edge (receiver order), whichever is less.
+        self.min_traffic = {"forward": self.alg_bytes["forward"] + E * d1 * s,
+                            "backward": self.alg_bytes["backward"] + E * min(d3, 3 * d1) * s}
         self.config["edges"] = int(E)
 
 

@@ -57,6 +57,8 @@ static inline T oeq_fma(T a, T b, T c) { return std::fma(a, b, c); }
 static inline void oeq_atomic_add(T* p, T v) { std::lock_guard<std::mutex> g(g_atomic_mutex); *p += v; }
 static inline T oeq_shfl_xor(T v, int mask) { g_xT[threadIdx.x] = v; oeq_sync(); T r = g_xT[threadIdx.x ^ mask]; oeq_sync(); return r; }
 static inline int oeq_shfl_i32(int v, int src) { g_xi[threadIdx.x] = v; oeq_sync(); int r = g_xi[src & 63]; oeq_sync(); return r; }
+static i64 g_xl[1024];
+static inline i64 oeq_shfl_up_i64(i64 v, int delta) { g_xl[threadIdx.x] = v; oeq_sync(); const int l = threadIdx.x & 63; i64 r = l >= delta ? g_xl[threadIdx.x - delta] : v; oeq_sync(); return r; }
 static inline int oeq_shfl_xor_i32(int v, int mask) { g_xi[threadIdx.x] = v; oeq_sync(); int r = g_xi[threadIdx.x ^ mask]; oeq_sync(); return r; }
 #define __builtin_amdgcn_readfirstlane(x) oeq_shfl_i32((x), 0)
 struct VT { T v[16 / sizeof(T)]; T& operator[](int i) { return v[i]; } const T& operator[](int i) const { return v[i]; } };
