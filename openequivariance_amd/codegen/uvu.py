@@ -101,6 +101,12 @@ class UVUGenerator:
     """Builds the source text and the launch plan for one uvu problem."""
 
     idx_ctype = "i64"        # element type of the convolution's index tensors ("int" for int32 callers)
+    # Backward arithmetic per path.  True: t_i = sum_j s_ij y_j with dw = sum_i x_i t_i and dx_i += w t_i, and the
+    # products c g_k that several pairs share computed once - two multiply-adds per pair beyond s_ij, a fifth fewer
+    # vector instructions than one pair at a time.  The kernels are bound by memory and no faster for it (128 / 256
+    # channels, batch and convolution: within 1 %); a kernel that holds a whole dZ row in registers spills more with
+    # it and keeps the pair-at-a-time form (False).
+    regroup_pairs = True
 
     def __init__(self, problem: TPProblem, kind: str = "tp", dw_partials: int = 1024):
         if kind not in ("tp", "conv_atomic", "conv_det"):
@@ -399,10 +405,7 @@ class UVUGenerator:
     def emit_backward_block(self, E: Emitter, o: Block, wptr: str, dw_sink) -> None:
         """Given g_k = dZ[o][u, k] (registers g0..), update dx{a}_{i}, dy{f} and hand every
         dW value to ``dw_sink(E, path, v, expr)``.  Formulas: loop_unroll_tp.cuh:167-174 of the
-        reference, regrouped so that every (i, j) pair costs two multiply-adds beyond its
-        s_ij = sum_k c_ijk g_k:  t_i = sum_j s_ij y_j,  dy_j += s_ij (w x_i),  and per path
-        dw = sum_i x_i t_i,  dx_i += w t_i.  A product c g_k that several pairs share (same k, same
-        |c|) is computed once; its sign rides on the multiply-add."""
+        reference; see ``regroup_pairs`` for the two ways the pairs of a path are evaluated."""
         for p in self.paths_into(o.idx):
             if p.looped:
                 self.emit_backward_looped(E, p, wptr, dw_sink)
@@ -424,6 +427,8 @@ class UVUGenerator:
     def _emit_cg_products(self, E: Emitter, p: Path) -> None:
         """c * g_k for the pairs of ``p`` with a single output component, once per distinct (k, |c|)."""
         self._cg_names = {}
+        if not self.regroup_pairs:
+            return
         for (i, j), ks in p.ordered_pairs():
             if len(ks) == 1:
                 key = self._cg_key(*ks[0])
@@ -433,33 +438,49 @@ class UVUGenerator:
 
     def _emit_backward_pairs(self, E: Emitter, p: Path, w: str, ya, dya) -> None:
         """The (i, j) pairs of one copy of the second operand: declares and fills ``dw``, updates dx and dy."""
-        is_ = sorted({i for (i, _) in p.pairs})
-        for i in is_:
-            E(f"  const T wx{i} = {w} * x{p.a.idx}_{i};")
-        started = set()
-        E("  T " + ", ".join(f"t{i}" for i in is_) + ";")
-        for (i, j), ks in p.ordered_pairs():
-            if len(ks) == 1:
-                neg = "-" if ks[0][1] < 0 else ""
-                s = f"{neg}{self._cg_names[self._cg_key(*ks[0])]}"
-            else:
+        if not self.regroup_pairs:
+            # every pair on its own: dw += s x_i y_j, dx_i += s (w y_j), dy_j += s (w x_i)
+            js = sorted({j for (_, j) in p.pairs})
+            is_ = sorted({i for (i, _) in p.pairs})
+            for j in js:
+                E(f"  const T wy{j} = {w} * {ya(j)};")
+            for i in is_:
+                E(f"  const T wx{i} = {w} * x{p.a.idx}_{i};")
+            E("  T dw = (T)0;")
+            for (i, j), ks in p.ordered_pairs():
                 E("  {")
                 for n_, (k, val) in enumerate(ks):
                     E(f"    T s = {self.lit(val)} * g{k};" if n_ == 0 else f"    s = oeq_fma({self.lit(val)}, g{k}, s);")
-                s = "s"
-            if i in started:
-                E(f"    t{i} = oeq_fma({s}, {ya(j)}, t{i});")
-            else:
-                E(f"    t{i} = {s} * {ya(j)};")
-                started.add(i)
-            E(f"    {dya(j)} = oeq_fma({s}, wx{i}, {dya(j)});")
-            if len(ks) > 1:
+                E(f"    dw = oeq_fma(s, x{p.a.idx}_{i} * {ya(j)}, dw);")
+                E(f"    dx{p.a.idx}_{i} = oeq_fma(s, wy{j}, dx{p.a.idx}_{i});")
+                E(f"    {dya(j)} = oeq_fma(s, wx{i}, {dya(j)});")
                 E("  }")
-        E(f"  T dw = x{p.a.idx}_{is_[0]} * t{is_[0]};")
-        for i in is_[1:]:
-            E(f"  dw = oeq_fma(x{p.a.idx}_{i}, t{i}, dw);")
-        for i in is_:
-            E(f"  dx{p.a.idx}_{i} = oeq_fma({w}, t{i}, dx{p.a.idx}_{i});")
+            return
+        # one component i of the first operand after the other, t_i = sum_j s_ij y_j
+        by_i = {}
+        for (i, j), ks in sorted(p.pairs.items()):
+            by_i.setdefault(i, []).append((j, ks))
+        E("  T dw = (T)0;")
+        for i, lst in sorted(by_i.items()):
+            E("  {")
+            E(f"    const T wx = {w} * x{p.a.idx}_{i};")
+            E("    T t;")
+            for n_, (j, ks) in enumerate(lst):
+                shared = len(ks) == 1
+                if shared:
+                    s = ("-" if ks[0][1] < 0 else "") + self._cg_names[self._cg_key(*ks[0])]
+                else:
+                    E("    {")
+                    for m_, (k, val) in enumerate(ks):
+                        E(f"      T s = {self.lit(val)} * g{k};" if m_ == 0 else f"      s = oeq_fma({self.lit(val)}, g{k}, s);")
+                    s = "s"
+                E(f"      t = {s} * {ya(j)};" if n_ == 0 else f"      t = oeq_fma({s}, {ya(j)}, t);")
+                E(f"      {dya(j)} = oeq_fma({s}, wx, {dya(j)});")
+                if not shared:
+                    E("    }")
+            E(f"    dw = oeq_fma(x{p.a.idx}_{i}, t, dw);")
+            E(f"    dx{p.a.idx}_{i} = oeq_fma({w}, t, dx{p.a.idx}_{i});")
+            E("  }")
 
     # --------------------------------------------------------------- LDS slots
     def emit_slot_write(self, E: Emitter, blk: Block, name: str, act: str) -> None:

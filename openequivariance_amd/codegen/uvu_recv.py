@@ -30,6 +30,9 @@ from .uvu_det import UVUDetGenerator
 
 
 class UVURecvGenerator(UVUDetGenerator):
+    # pass 1 holds a dZ row in registers: the regrouped backward arithmetic spills 27 instead of 13 words per lane on
+    # the 128-channel MACE problem and measured 2.37 instead of 1.83 ms
+    regroup_pairs = False
     # Tile counts from 4096 to one tile per 16 edges and 2 / 4 / 8 spill rows in flight in pass 2 moved pass 1 by
     # less than 4 % (256 channels: 6.39 - 6.71 ms)
     MIN_TILE_ITERS = 8       # edge-loop iterations of the smallest tile

@@ -61,6 +61,7 @@ static i64 g_xl[1024];
 static inline i64 oeq_shfl_up_i64(i64 v, int delta) { g_xl[threadIdx.x] = v; oeq_sync(); const int l = threadIdx.x & 63; i64 r = l >= delta ? g_xl[threadIdx.x - delta] : v; oeq_sync(); return r; }
 static inline int oeq_shfl_xor_i32(int v, int mask) { g_xi[threadIdx.x] = v; oeq_sync(); int r = g_xi[threadIdx.x ^ mask]; oeq_sync(); return r; }
 #define __builtin_amdgcn_readfirstlane(x) oeq_shfl_i32((x), 0)
+static inline u64 oeq_uniform_u64(u64 v) { return v; }
 struct VT { T v[16 / sizeof(T)]; T& operator[](int i) { return v[i]; } const T& operator[](int i) const { return v[i]; } };
 #define OEQ_DMA(BYTES, POLICY, g, lds_base) memcpy((char*)(lds_base) + ((BYTES) == 12 ? 16 : (BYTES)) * (threadIdx.x & 63), (g), (BYTES))
 static inline void oeq_release_agent() {}
