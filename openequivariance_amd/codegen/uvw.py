@@ -108,6 +108,14 @@ class UVWGenerator:
         # copied between sets, has 0.9 instead of 2.1 vector-ALU instructions per MFMA and measured 0.341
         # against 0.331 ms; larger groups for the cheap work items 0.361 - 0.422 against 0.359 ms)
         self.fwd_group, self.fwd_unroll = (4, 1) if self.T == "float" else (1, 3)
+        # Tile shape: 16 x 16 x 4 in both types.  The fp32 forward on v_mfma_f32_32x32x2_f32 (32 batch rows per
+        # tile, half the weight-operand loads per FLOP) passed the same parity tests and measured 0.371 ms (w
+        # ranges of at most 96 accumulator registers, two wavefronts per SIMD) and 0.374 ms (whole output
+        # blocks, 160 accumulators, one wavefront) against 0.318 ms: the CG vector-ALU work per FLOP is the
+        # same in both shapes (one product per row and channel, used for all 64 w), a lane's X loads cover 8
+        # instead of 16 channels of a row per group (twice the cache lines per load instruction: texture
+        # addresser busy 50 % instead of 47 %, matrix core busy 51 % instead of 60 % of the kernel's cycles),
+        # and the accumulators of a 32-row tile leave no room for the operands of the next group.
         # backward dW: fetch the operands of the next step while the current one runs (two register sets);
         # in fp64 the second set crosses the 512-register limit even per pass (1.31 against 1.22 ms)
         self.dw_prefetch = self.T == "float"
@@ -190,6 +198,11 @@ class UVWGenerator:
         self.ws_elems = self.PART_OFF + self.DW_WORKGROUPS * self.WN
 
     # ------------------------------------------------------------------ helpers
+    def forward_attr(self) -> str:
+        """fp32: two wavefronts per SIMD (256 registers each) - the operands of the next group, of this path or
+        the next, need the room; fp64 accumulators are twice as wide and take what a single wavefront gets."""
+        return " __attribute__((amdgpu_waves_per_eu(2, 2)))" if self.T == "float" else ""
+
     def backward_attr(self) -> str:
         """Occupancy target of the dX/dY kernel: as many workgroups per CU (one wavefront per SIMD
         each) as the LDS tile allows; the register allocator then stays within that budget."""
@@ -385,60 +398,74 @@ class UVWGenerator:
             for k in range(o.D):
                 for nt in NTS:
                     E(f"V4 acc{k}_{nt} = {{0, 0, 0, 0}};")
-            for p in self.paths_into(o.idx):
+            # The K loops of the segment's paths form ONE software pipeline of groups of GS steps: the X records
+            # and weight slices of the next group are in flight while this group runs on the VALU and the matrix
+            # core, and the last group of a path (peeled off its loop) has the first group of the NEXT path in
+            # flight, so that only the first path of a work item waits for its operands with nothing to do.
+            # What bounds this kernel is the L2 -> L1 stream of operands (every wavefront re-reads the packed
+            # weights), so the bytes in flight per wavefront matter more than anything else here.
+            GS = self.fwd_group
+            paths = self.paths_into(o.idx)
+            groups = {p.t: _ceil(p.SU, GS) for p in paths}
+
+            def regs(p):
+                return [f"n{p.t}x{j}_{i}" for j in range(GS) for i in range(p.a.D)] \
+                    + [f"n{p.t}b{j}_{nt}" for j in range(GS) for nt in NTS]
+
+            def load(E, p, gexp):
+                NG = groups[p.t]
+                for j in range(GS):
+                    sexp = f"({gexp}) * {GS} + {j}"
+                    need_clamp = (NG * GS != p.SU)
+                    scl = f"min({sexp}, {p.SU - 1})" if need_clamp else sexp
+                    # K index -> channel: step s of lane group g is u = 16 (s / 4) + 4 g + s % 4, so that the
+                    # four steps of a group read four adjacent records of a row (one wide load per lane)
+                    uexp = f"16 * (({sexp}) >> 2) + 4 * g + (({sexp}) & 3)"
+                    ucl = uexp if (p.mu % 16 == 0 and not need_clamp) else f"min({uexp}, {p.mu - 1})"
+                    E(f"{{ const T* __restrict__ xp = Xr + {p.a.off} + ({ucl}) * {p.a.D}; " + " ".join(f"n{p.t}x{j}_{i} = xp[{i}];" for i in range(p.a.D)))
+                    E(f"  const T* __restrict__ bp = wsT + {p.wb} + (({scl}) * 64 + lane) * {NT}; " + " ".join(f"n{p.t}b{j}_{nt} = bp[{nt}];" for nt in NTS) + " }")
+
+            def steps(E, p, sgexp):
+                """The GS K steps of group ``sgexp`` of path p on the copies (c...) of its operand registers."""
+                NG = groups[p.t]
+                for j in range(GS):
+                    E("{")
+                    E.level += 1
+                    E("const T " + ", ".join(f"x{i} = cn{p.t}x{j}_{i}" for i in range(p.a.D)) + ";")
+                    self.emit_cg_apply(E, p, "x", "m", "t")
+                    if p.mu % 16 != 0 or NG * GS != p.SU:
+                        E(f"if (16 * ((({sgexp}) * {GS} + {j}) >> 2) + 4 * g + ((({sgexp}) * {GS} + {j}) & 3) >= {p.mu}) {{ " + " ".join(f"t{k} = (T)0;" for k in range(o.D)) + " }")
+                    for k in range(o.D):
+                        for nt in NTS:
+                            E(f"acc{k}_{nt} = oeq_mfma(t{k}, cn{p.t}b{j}_{nt}, acc{k}_{nt});")
+                    E.level -= 1
+                    E("}")
+
+            for p in paths:
+                E("T " + ", ".join(regs(p)) + ";")
+            load(E, paths[0], "0")
+            for pi, p in enumerate(paths):
+                NG = groups[p.t]
+                nxt = paths[pi + 1] if pi + 1 < len(paths) else None
                 E(f"{{ // path {p.t}: l = {p.a.l} x {p.b.l} -> {p.o.l}, coefficient {p.coeff:.9g}")
                 E.level += 1
-                # The K loop runs in groups of GS steps, software pipelined: the X records and weight
-                # slices of the next group are in flight while this group runs on the VALU and the
-                # matrix core.  What bounds this kernel is the L2 -> L1 stream of operands (every
-                # wavefront re-reads the packed weights), so the bytes in flight per wavefront matter
-                # more than anything else here.
-                GS = self.fwd_group
-                NG = _ceil(p.SU, GS)
-                sets = ("n",)
-                regs = [f"{q}x{j}_{i}" for q in sets for j in range(GS) for i in range(p.a.D)] \
-                    + [f"{q}b{j}_{nt}" for q in sets for j in range(GS) for nt in NTS]
-                E("T " + ", ".join(regs) + ";")
                 # the CG tensor is contracted with the row's Y once per path; the small matrix is applied per channel
                 self.emit_cg_matrix(E, p, "y", "m")
-
-                def load(E, gexp, q="n"):
-                    for j in range(GS):
-                        sexp = f"({gexp}) * {GS} + {j}"
-                        need_clamp = (NG * GS != p.SU)
-                        scl = f"min({sexp}, {p.SU - 1})" if need_clamp else sexp
-                        # K index -> channel: step s of lane group g is u = 16 (s / 4) + 4 g + s % 4, so that the
-                        # four steps of a group read four adjacent records of a row (one wide load per lane)
-                        uexp = f"16 * (({sexp}) >> 2) + 4 * g + (({sexp}) & 3)"
-                        ucl = uexp if (p.mu % 16 == 0 and not need_clamp) else f"min({uexp}, {p.mu - 1})"
-                        E(f"{{ const T* __restrict__ xp = Xr + {p.a.off} + ({ucl}) * {p.a.D}; " + " ".join(f"{q}x{j}_{i} = xp[{i}];" for i in range(p.a.D)))
-                        E(f"  const T* __restrict__ bp = wsT + {p.wb} + (({scl}) * 64 + lane) * {NT}; " + " ".join(f"{q}b{j}_{nt} = bp[{nt}];" for nt in NTS) + " }")
-
-                def steps(E, sgexp, q):
-                    """The GS K steps of group ``sgexp`` on the operands of register set q."""
-                    for j in range(GS):
-                        E("{")
-                        E.level += 1
-                        E("const T " + ", ".join(f"x{i} = {q}x{j}_{i}" for i in range(p.a.D)) + ";")
-                        self.emit_cg_apply(E, p, "x", "m", "t")
-                        if p.mu % 16 != 0 or NG * GS != p.SU:
-                            E(f"if (16 * ((({sgexp}) * {GS} + {j}) >> 2) + 4 * g + ((({sgexp}) * {GS} + {j}) & 3) >= {p.mu}) {{ " + " ".join(f"t{k} = (T)0;" for k in range(o.D)) + " }")
-                        for k in range(o.D):
-                            for nt in NTS:
-                                E(f"acc{k}_{nt} = oeq_mfma(t{k}, {q}b{j}_{nt}, acc{k}_{nt});")
-                        E.level -= 1
-                        E("}")
-                load(E, "0")
                 E(f"#pragma unroll {self.fwd_unroll}")
                 E(f"for (int sg = 0; sg < {NG}; ++sg) {{")
                 E.level += 1
-                E("const T " + ", ".join(f"c{r} = {r}" for r in regs) + ";")
+                E("const T " + ", ".join(f"c{r} = {r}" for r in regs(p)) + ";")
                 E(f"if (sg + 1 < {NG}) {{")
                 E.level += 1
-                load(E, "sg + 1")
+                load(E, p, "sg + 1")
                 E.level -= 1
+                if nxt is not None:
+                    E("} else {")
+                    E.level += 1
+                    load(E, nxt, "0")
+                    E.level -= 1
                 E("}")
-                steps(E, "sg", "cn")
+                steps(E, p, "sg")
                 E.level -= 1
                 E("}")
                 E.level -= 1
