@@ -714,6 +714,7 @@ def main():
                                 "traffic": {"forward": load_traffic(f"{name}:forward"), "backward": load_traffic(f"{name}:backward")},
                                 "flushed_caches": rf.get("flushed_caches"),
                                 "prepared_graph": rf.get("prepared_graph"), "min_traffic": rf.get("min_traffic"),
+                                "min_traffic_rate_GBs": rf.get("min_traffic_rate_GBs"),
                                 "torch_op": r.get("torch_op"), "cpu_baseline": r["cpu_baseline"],
                                 "bench_seconds": None}
             except Exception as exc:          # one workload failing must not hide the others

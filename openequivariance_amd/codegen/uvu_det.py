@@ -653,7 +653,7 @@ class UVUDetGenerator(UVUDirectGenerator):
         lane stride (measured on gfx950), 1- and 4-word transfers are packed."""
         return 4 if words == 3 else words
 
-    def emit_staged_loop(self, E: Emitter, pos_of, pos_list, nbr_list: str, dma, readback, compute, flush=None) -> None:
+    def emit_staged_loop(self, E: Emitter, pos_of, pos_list, nbr_list: str, dma, readback, compute, flush=None, pre=None) -> None:
         """The edge loop with the operands of the next edge in flight to LDS while the current edge is
         computed.  An LDS-DMA load holds no registers while it is outstanding, so this pipeline needs one
         register set where emit_pingpong_loop needs two.  Four stages, none of which consumes a load
@@ -668,7 +668,9 @@ class UVUDetGenerator(UVUDirectGenerator):
         requests, compute.  The compiler does not order LDS reads after an outstanding LDS-DMA write by
         itself, hence the explicit wait at the top; it waits for every earlier vector-memory access, which
         is why the per-edge stores are issued in front of the requests and not from inside the
-        arithmetic, where they would be the youngest accesses at the next wait."""
+        arithmetic, where they would be the youngest accesses at the next wait.  ``pre``, when given, is emitted
+        between the stores and the requests: register loads it issues (consumed by the arithmetic of this
+        iteration) are older than the requests and can be waited for without draining them."""
         def pos(it):
             return f"(({pos_of(it)}) < len ? (u64)(beg + {pos_of(it)}) : (u64)(nnz - 1))"
 
@@ -710,6 +712,8 @@ class UVUDetGenerator(UVUDirectGenerator):
             flush(E)
             E.level -= 1
             E("}")
+        if pre:
+            pre(E)
         # indices requested during the previous iteration
         E(f"v1 = v1 && {nbr_ok('rawN')}; n1 = v1 ? (u64)rawN : 0;")
         E(f"v2 = {edge_ok('rawE', 'it + 2')}; e2 = v2 ? (u64)rawE : 0;")

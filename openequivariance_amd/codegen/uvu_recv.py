@@ -30,16 +30,20 @@ from .uvu_det import UVUDetGenerator
 
 
 class UVURecvGenerator(UVUDetGenerator):
-    # pass 1 holds a dZ row in registers: the regrouped backward arithmetic spills 27 instead of 13 words per lane on
-    # the 128-channel MACE problem and measured 2.37 instead of 1.83 ms
+    # Arithmetic form of pass 1 (see UVUGenerator.regroup_pairs).  With register loads, pass 1 holds a dZ row and an
+    # edge's operands in registers and the regrouped form spills 27 instead of 13 words per lane on the 128-channel
+    # MACE problem (2.63 against 2.08 ms); with the operands staged through LDS it needs fewer registers than the
+    # pair-at-a-time form (175 against 218 there) and is faster on every shape measured (MACE 1.73 against 1.81 ms,
+    # 256 channels 6.97 against 7.55 ms).
     regroup_pairs = False
+    REGROUP_STAGED = True
     # Tile counts from 4096 to one tile per 16 edges and 2 / 4 / 8 spill rows in flight in pass 2 moved pass 1 by
     # less than 4 % (256 channels: 6.39 - 6.71 ms)
     MIN_TILE_ITERS = 8       # edge-loop iterations of the smallest tile
     MAX_TILES = 16384        # tiles per chunk of the largest launches (the tile then grows with the edge count)
     DX_UNROLL = 4            # spill rows in flight per lane group in pass 2
 
-    def __init__(self, problem: TPProblem, vector_stores: bool = True, idx_ctype: str = "i64", prefetch=None):
+    def __init__(self, problem: TPProblem, vector_stores: bool = True, idx_ctype: str = "i64", prefetch=None, staged=None):
         # pass 1 is one launch: the per-edge dX rows cannot be split over launches of output-block groups
         super().__init__(problem, vector_stores=vector_stores, idx_ctype=idx_ctype, allow_split=False)
         assert self.H == 1
@@ -59,6 +63,18 @@ class UVURecvGenerator(UVUDetGenerator):
         # large per-edge footprints: hold the allocation to two wavefronts per SIMD (a handful of spilled
         # words) instead of one
         self.waves_hint = 2 if held + per_edge > 100 else 0
+        # Pass 1 with the next edge's operands (X of the sender, W, Y) in flight to LDS by LDS-DMA, which holds
+        # no registers: dZ of the receiver and one edge's operands together leave no room for a second register
+        # set, so with register loads the loop runs one edge at a time with its load latency exposed.  Measured
+        # backward, register loads against staged (both pair-at-a-time): MACE problem 2.07 -> 1.83 ms, 256 channels
+        # with outputs of either parity 16.3 -> 9.9 ms, 256 channels 7.84 -> 7.74 ms, 32 channels 0.201 -> 0.179 ms.
+        # The staged kernels are left to the occupancy their register count gives (138 - 175: two or three
+        # wavefronts per SIMD; held to exactly two: 256 channels 6.97 instead of 6.76 ms).
+        self.can_stage = self.T == "float" and self.P >= self.D2      # (the Y slab holds one word per lane of a row's group)
+        self.staged_edges = self.can_stage and (True if staged is None else bool(staged))
+        self.regroup_pairs = bool(self.REGROUP_STAGED and self.staged_edges)
+        if self.staged_edges:
+            self.waves_hint = 0
         self.dypart_off = "(2 * (node_count + 1) + node_count) * sizeof(i64)"
         self.spill_off = (f"((({self.dypart_off} + {self.dy_slots if self.dy_slots > 1 else 0}ull * nnz * {self.D2} * sizeof(T)) "
                           "+ 255ull) & ~255ull)")
@@ -105,6 +121,8 @@ class UVURecvGenerator(UVUDetGenerator):
         E = Emitter()
         R, P, NCH = self.R, self.P, self.NCH
         self.emit_lane_direct(E, lds=False)
+        if self.staged_edges:
+            return self._edges_body_staged(E)
         E("// (tile, chunk) of this workgroup: ids are dealt to the 8 XCDs round robin, each XCD gets a contiguous run of items")
         E(f"const u64 tiles = gridDim.x, items = tiles * {NCH};")
         E("const u64 bid = blockIdx.x + (u64)blockIdx.y * gridDim.x;")
@@ -228,6 +246,155 @@ class UVURecvGenerator(UVUDetGenerator):
         self.emit_pingpong_loop(E, names, load_idx, load, compute, prefetch_first=self.prefetch_edges, pre=pre,
                                 index_decl="u64 I0e = 0, I1e = 0, I0n = 0, I1n = 0; i64 I0r = -1, I1r = -1; "
                                            "bool I0rv = false, I1rv = false, I0ev = false, I1ev = false;")
+        return E.text()
+
+    def _edges_body_staged(self, E: Emitter) -> str:
+        """Pass 1 through the LDS stage of the forward (same operands: X records of the sender, path weights, Y):
+        the edge loop of emit_staged_loop over the tile's consecutive edges, dZ of the receiver held in registers
+        and reloaded when the receiver changes, the edge's dW / dY / dX rows kept in registers and stored at the top
+        of the next iteration."""
+        R, P, NCH = self.R, self.P, self.NCH
+        nt = 2 if self.nontemporal else 0
+        E("// (tile, chunk) of this workgroup: ids are dealt to the 8 XCDs round robin, each XCD gets a contiguous run of items")
+        E(f"const u64 tiles = gridDim.x, items = tiles * {NCH};")
+        E("const u64 bid = blockIdx.x + (u64)blockIdx.y * gridDim.x;")
+        E("const u64 xcd = bid & 7, turn = bid >> 3;")
+        E("const u64 item = xcd * (items >> 3) + min(xcd, items & 7) + turn;")
+        E(f"const int c = (int)(item % {NCH}); (void)c;")
+        E(f"const u64 tile = item / {NCH};")
+        E(f"const int u = c * {P} + ul;")
+        E(f"const u64 per = ((nnz + tiles - 1) / tiles + {R - 1}) / {R} * {R};       // edges per tile")
+        E("const u64 beg = min(tile * per, nnz);")
+        E("const int len = (int)(min(beg + per, nnz) - beg);")
+        E(f"const int maxlen = (len + {R - 1}) / {R};")
+        E(f"T* __restrict__ spill = (T*)((char*)ws + {self.spill_off});")
+        self._cur_c = "e"
+        E("bool rv = false;")
+        for oi in self.used_out:
+            E("T " + ", ".join(f"G{oi}_{k} = (T)0" for k in range(self.out[oi].D)) + ";")
+        E("i64 cur_rcv = -1, rawR = -1, rcv0 = -1;")
+        slabs, words = self._forward_slabs()
+        y_off = words - 64
+        E(f"__shared__ __attribute__((aligned(16))) T stage[{words}];")
+        res = [f"pw_{p.t}_{v}" for p in self.paths for v in range(p.mv)] + [f"pdy{f}" for f in self.used_y] \
+            + [f"pdx{i}_{m}" for i in self.used_in1 for m in range(self.in1[i].D)]
+        E("T " + ", ".join(f"{n} = (T)0" for n in res) + "; u64 pe = 0; bool pv = false, pev = false;")
+
+        def dma(E, e, n):
+            E("{")
+            E.level += 1
+            E(f"const u64 e = {e}, sndc = {n};")
+            E("rawR = rows[e];")
+            E(f"const T* __restrict__ Wr = W + e * {self.WN};")
+            E(f"OEQ_DMA(4, {nt}, Y + e * {self.D2} + min(ul, {self.D2 - 1}), stage + {y_off});")
+            for kind, key, k0, w, so in slabs:
+                if kind == "W":
+                    p, v = key
+                    E(f"OEQ_DMA(4, {nt}, Wr + {self.widx(p, self.uclamp(p.a, 0), v)}, stage + {so});")
+            for kind, key, k0, w, so in slabs:
+                if kind == "X":
+                    a = self.in1[key]
+                    E(f"OEQ_DMA({4 * w}, 0, X + sndc * {self.D1} + {a.off} + {self.uclamp(a, 0)} * {a.D} + {k0}, stage + {so});")
+            E.level -= 1
+            E("}")
+
+        def readback(E):
+            # the receiver of this iteration's edge was requested with its operands (rawR is overwritten by the
+            # requests of this iteration, below)
+            E("rcv0 = rawR;")
+            E(f"const bool cur_ev = {self.edge_pos('it')} < len;")
+            E("rv = cur_rv && rcv0 >= 0 && rcv0 < (i64)node_count;")
+            for f in self.used_y:
+                E(f"const T y{f} = stage[{y_off} + sub * {P} + {f}];")
+            for kind, key, k0, w, so in slabs:
+                if kind == "W":
+                    p, v = key
+                    E(f"const T We_{p.t}_{v} = stage[{so} + lane];")
+            for i in self.used_in1:
+                a = self.in1[i]
+                parts = []
+                for kind, key, k0, w, so in slabs:
+                    if kind == "X" and key == i:
+                        parts += [f"stage[{so} + lane * {self.dma_stride(w)} + {r}]" for r in range(w)]
+                # dW and dY of an edge are proportional to x: zero it for idle lanes and invalid edges
+                E(f"const bool a{i}_ = {self.act(a)};")
+                E("const T " + ", ".join(f"xr{i}_{m} = {parts[m]}" for m in range(a.D)) + ";")
+                E("const T " + ", ".join(f"x{i}_{m} = a{i}_ ? xr{i}_{m} : (T)0" for m in range(a.D)) + ";")
+
+        def flush(E):
+            """Per-edge results of the edge computed last: dW row, dY row (or partial), dX row."""
+            E("{")
+            E.level += 1
+            E("const u64 e = pe;")
+            E(f"T* __restrict__ Wgr = Wg + e * {self.WN};")
+            for p in self.paths:
+                ok = "pev" if self.full(p.a) else f"(pev && u < {p.a.mul})"
+                for v in range(p.mv):
+                    E(f"if ({ok}) {self.st('Wgr', self.widx(p, 'u', v), f'pw_{p.t}_{v}')}")
+            writer = "ul == 0" if P < 64 else "lane == 63"
+            E(f"if (pev && {writer}) {{")
+            if self.dy_slots > 1:
+                E(f"    T* __restrict__ Ygr = (T*)((char*)ws + DYPART_OFF) + ((u64)c * nnz + e) * {self.D2};")
+            else:
+                E(f"    T* __restrict__ Ygr = Yg + e * {self.D2};")
+            for f in range(self.D2):
+                E(f"    Ygr[{f}] = " + (f"pdy{f};" if f in self.used_y else "(T)0;"))
+            E("}")
+            E("if (pev) {")
+            E(f"    T* __restrict__ sp = spill + ((e * {NCH} + c) * {self.NW}) * {P} + ul;")
+            w = 0
+            for i in self.used_in1:
+                for m in range(self.in1[i].D):
+                    E(f"    oeq_stnt(sp + {w * P}, pv ? pdx{i}_{m} : (T)0);")
+                    w += 1
+            E("}")
+            E.level -= 1
+            E("}")
+
+        def pre(E):
+            """dZ of this edge's receiver, when it differs from the one held."""
+            if R == 1:
+                # the receiver is the same for all lanes: a scalar branch, loads not predicated
+                E("const int rcv_u = __builtin_amdgcn_readfirstlane(rv ? (int)rcv0 : -1);")
+                E("if (rcv_u >= 0 && (i64)rcv_u != cur_rcv) {")
+                E.level += 1
+                E("cur_rcv = (i64)rcv_u;")
+            else:
+                E("if (rv && rcv0 != cur_rcv) {")
+                E.level += 1
+                E("cur_rcv = rcv0;")
+            for oi in self.used_out:
+                o = self.out[oi]
+                E(f"{{ const T* __restrict__ p_ = G + (u64)cur_rcv * {self.D3} + {o.off} + {self.uclamp(o, 0)} * {o.D}; "
+                  + " ".join(f"G{oi}_{k} = p_[{k}];" for k in range(o.D)) + " }")
+                if not self.full(o):
+                    E(f"if (!(u < {o.mul})) {{ " + " ".join(f"G{oi}_{k} = (T)0;" for k in range(o.D)) + " }")
+            E.level -= 1
+            E("}")
+
+        def compute(E, h):
+            E("const u64 e = cur_e;")
+            for f in self.used_y:
+                E(f"T dy{f} = (T)0;")
+            for i in self.used_in1:
+                E("T " + ", ".join(f"dx{i}_{m} = (T)0" for m in range(self.in1[i].D)) + ";")
+            for oi in self.used_out:
+                o = self.out[oi]
+                E("{")
+                E.level += 1
+                for k in range(o.D):
+                    E(f"const T g{k} = G{oi}_{k};")
+
+                def sink(E, p, v, expr):
+                    E(f"  pw_{p.t}_{v} = {expr};")
+                self.emit_backward_block(E, o, "Wr", sink)
+                E.level -= 1
+                E("}")
+            self.emit_dy_sum(E)
+            E(" ".join(f"pdy{f} = dy{f};" for f in self.used_y))
+            E(" ".join(f"pdx{i}_{m} = dx{i}_{m};" for i in self.used_in1 for m in range(self.in1[i].D)))
+            E("pe = e; pv = rv; pev = cur_ev;")
+        self.emit_staged_loop(E, self.edge_pos, None, "cols", dma, readback, compute, flush, pre=pre)
         return E.text()
 
     # ---------------------------------------------------------------- pass 2

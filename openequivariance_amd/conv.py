@@ -92,7 +92,7 @@ def sort_by_receiver(rows: "torch.Tensor", cols: "torch.Tensor", node_count: typ
 
 
 # d3 / d1 from which the deterministic backward walks the edges in receiver order (see select_conv_generator)
-RECV_ORDER_MIN_RATIO = 7
+RECV_ORDER_MIN_RATIO = 4.5
 
 
 def select_conv_generator(config: TPProblem, deterministic: bool, vector_stores: bool = True, idx_dtype=np.int64):
@@ -103,12 +103,20 @@ def select_conv_generator(config: TPProblem, deterministic: bool, vector_stores:
     if deterministic:
         order = tunables.current.det_backward
         if order is None:
-            # Static rule (no clock: which kernel runs must not depend on timing if results are to repeat
-            # bit for bit).  The sender order gathers a dZ row (d3 words) per edge, the receiver order an X
-            # row and spills a dX row (3 d1 words, half of them writes).  Measured backward, sender against
-            # receiver order: d3 / d1 = 3.9 (32 channels) 0.155 / 0.187 ms, 4.8 (256 channels) 7.48 / 7.78 ms,
-            # 7.9 (the 128-channel MACE problem) 2.15 / 2.07 ms.
-            order = "recv" if config.irreps_out.dim >= RECV_ORDER_MIN_RATIO * config.irreps_in1.dim else "send"
+            # Static rule, by the shape of the problem only (a clock would make the choice - and with it every
+            # bit of the result - differ between processes).  The sender order gathers a dZ row per edge (d3
+            # words, reads); the receiver order gathers an X row and writes and re-reads a dX row (3 d1 words,
+            # half of them writes), and pays off when pass 1 can stage its operands through LDS.  Measured
+            # backward, sender against receiver order: d3 / d1 = 3.9 (32 channels) 0.164 / 0.176 ms, 4.8 (256
+            # channels) 7.55 / 6.76 ms, 5.7 (32 channels, outputs of either parity) 0.225 / 0.208 ms, 7.1 (256
+            # channels, either parity) 10.96 / 9.32 ms, 7.9 (the 128-channel MACE problem) 2.15 / 1.73 ms.
+            # Without the stage (fp64, or fewer channels than Y components) pass 1 runs one edge at a time:
+            # 16.3 against 10.96 ms at 7.1; those problems keep the sender order.
+            order = "send"
+            if config.irreps_out.dim >= RECV_ORDER_MIN_RATIO * config.irreps_in1.dim:
+                g = UVURecvGenerator(config, vector_stores=vector_stores, idx_ctype=idx_ctype)
+                if g.staged_edges:
+                    return g
         if order == "recv":
             return UVURecvGenerator(config, vector_stores=vector_stores, idx_ctype=idx_ctype)
         return UVUDetGenerator(config, vector_stores=vector_stores, idx_ctype=idx_ctype)

@@ -180,17 +180,20 @@ def test_conv_blocks_no_path_touches_are_zero_filled():
         assert rel_err(got, ref) < TOL
 
 
+@pytest.mark.parametrize("staged", [False, True])
 @pytest.mark.parametrize("irreps,nodes,nnz,prefetch", [
     (("5x0e+3x1o+70x2e", "1x0e+1x1o+1x2e", "5x0e+3x1o+70x2e+7x3o"), 5, 11, None),      # two chunks, ragged
     (("1x0e+1x1o+16x3o", "1x0e+1x1o", "16x0e+16x0o+16x1e+16x1o"), 21, 265, None),    # four lane groups, unused block
     (("8x0e+8x1o", "1x0e+1x1o", "8x0e+8x1o"), 9, 100, False)])                       # eight lane groups, one register set
-def test_conv_receiver_order_backward(irreps, nodes, nnz, prefetch):
+def test_conv_receiver_order_backward(irreps, nodes, nnz, prefetch, staged):
     """The two-pass backward (per-edge dX rows spilled in receiver order, summed per sender in the order
     of the transpose permutation): tiles that end inside a receiver's edges, idle lane groups in the last
-    iteration of a tile, self loops, nodes without edges."""
+    iteration of a tile, self loops, nodes without edges; pass 1 with register loads and with the next
+    edge's operands staged through LDS."""
     from openequivariance_amd.codegen.uvu_recv import UVURecvGenerator
     prob, oprob = common.channelwise(irreps)
-    g = UVURecvGenerator(prob, prefetch=prefetch)
+    g = UVURecvGenerator(prob, prefetch=prefetch, staged=staged)
+    assert g.staged_edges == (staged and g.P >= g.D2)
     rows, cols, tperm, _ = otp.coord_graph(*common.random_graph(nodes, nnz, 7, self_loops=True))
     X, Y, W, G = common.conv_inputs(prob, nodes, nnz, 8)
     _, bwd, ws = g.plan()
@@ -200,12 +203,13 @@ def test_conv_receiver_order_backward(irreps, nodes, nnz, prefetch):
         assert rel_err(got, ref) < TOL
 
 
-@pytest.mark.parametrize("variant", ["det", "det_two_chunks", "grouped", "recv"])
+@pytest.mark.parametrize("variant", ["det", "det_two_chunks", "grouped", "recv", "recv_staged"])
 def test_conv_edges_naming_no_node(variant):
     """Edges whose sender or receiver is out of range contribute nothing, and their dW / dY rows come
     out as zeros from every backward variant (the emulator starts all outputs from junk)."""
     from openequivariance_amd.codegen.uvu_recv import UVURecvGenerator
     irreps = ("70x0e+70x1o", "1x0e+1x1o", "70x0e+70x1o") if variant == "det_two_chunks" else \
+        ("16x0e+16x1o", "1x0e+1x1o+1x2e", "16x0e+16x1o+16x2e") if variant == "recv_staged" else \
         ("8x0e+8x1o", "1x0e+1x1o+1x2e", "8x0e+8x1o+8x2e")
     prob, oprob = common.channelwise(irreps)
     nodes, nnz = 9, 300 if variant != "det_two_chunks" else 40
@@ -217,6 +221,7 @@ def test_conv_edges_naming_no_node(variant):
         rows, cols, valid = rows[order], cols[order], valid[order]
         tperm = np.lexsort((np.arange(nnz), rows, cols)).astype(np.int64)
     g = {"det": UVUDetGenerator, "det_two_chunks": UVUDetGenerator, "recv": UVURecvGenerator,
+         "recv_staged": lambda p: UVURecvGenerator(p, staged=True),
          "grouped": lambda p: UVUSortedGenerator(p, grouped_backward=True)}[variant](prob)
     X, Y, W, G = common.conv_inputs(prob, nodes, nnz, 8)
     Zr, dXr, dYr, dWr = common.conv_reference_on_valid_edges(otp, oprob, X, Y, W, G, rows, cols, valid)

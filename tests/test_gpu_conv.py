@@ -83,14 +83,18 @@ def test_conv_outputs_of_either_parity(cuda, which, deterministic):
         _run(prob, oprob, 30, 400, 38, deterministic, sh_lmax=3)
 
 
-def test_mace_conv_deterministic_backward_defaults_to_receiver_order(cuda):
-    """A dZ row of the MACE problem is 7.9 times as long as an X row: the static rule picks the two-pass
-    receiver-order backward (config 3 and 5, ratios 3.9 and 4.8, keep the sender order)."""
+def test_deterministic_backward_order_is_chosen_by_shape(cuda):
+    """Static rule: the two-pass receiver-order backward when a dZ row is at least 4.5 times as long as an X row
+    and pass 1 can stage its operands through LDS (fp32, at least as many channels per row group as Y
+    components): the MACE problem (7.9) and config 5 (4.8) take it, config 3 (3.9) and fp64 problems keep the
+    sender order."""
     from openequivariance_amd.codegen.uvu_recv import UVURecvGenerator
     from openequivariance_amd.conv import select_conv_generator
-    assert isinstance(select_conv_generator(common.channelwise(common.MACE)[0], True), UVURecvGenerator)
-    for irreps in (common.NEQUIP, common.LARGE):
-        assert not isinstance(select_conv_generator(common.channelwise(irreps)[0], True), UVURecvGenerator)
+    for irreps in (common.MACE, common.LARGE):
+        g = select_conv_generator(common.channelwise(irreps)[0], True)
+        assert isinstance(g, UVURecvGenerator) and g.staged_edges and g.regroup_pairs
+    assert not isinstance(select_conv_generator(common.channelwise(common.NEQUIP)[0], True), UVURecvGenerator)
+    assert not isinstance(select_conv_generator(common.channelwise(common.MACE, dtype=np.float64)[0], True), UVURecvGenerator)
     prob, oprob = common.channelwise(common.MACE)
     _run(prob, oprob, 60, 900, 40, True, sh_lmax=3)
 
@@ -108,20 +112,27 @@ def test_mace_conv_backward_split_over_output_blocks(cuda, deterministic, monkey
     _run(prob, oprob, 60, 900, 39, deterministic, sh_lmax=3)
 
 
-@pytest.mark.parametrize("which", ["nequip", "large", "mace", "ragged"])
-def test_receiver_order_backward(cuda, which, monkeypatch):
-    """The two-pass backward of the deterministic variant (forced for every shape here; by itself it is
-    chosen for rows of dZ at least seven times as long as rows of X): parity, and bit-equal repeats."""
+@pytest.mark.parametrize("staged", [True, False])
+@pytest.mark.parametrize("which", ["nequip", "large", "mace", "ragged", "few_channels"])
+def test_receiver_order_backward(cuda, which, staged, monkeypatch):
+    """The two-pass backward of the deterministic variant, forced for every shape here, pass 1 with the next
+    edge's operands staged through LDS and with plain register loads (what fp64 problems and rows with fewer
+    channels than Y components get): parity, and bit-equal repeats."""
     import torch
     from openequivariance_amd import tunables
     from openequivariance_amd.codegen.uvu_recv import UVURecvGenerator
     monkeypatch.setattr(tunables.current, "det_backward", "recv")
+    if not staged:
+        init = UVURecvGenerator.__init__
+        monkeypatch.setattr(UVURecvGenerator, "__init__", lambda self, *a, **k: init(self, *a, **{**k, "staged": False}))
     irreps = {"nequip": common.NEQUIP, "large": common.LARGE, "mace": common.MACE,
-              "ragged": ("5x0e+3x1o+70x2e", "1x0e+1x1o+1x2e", "5x0e+3x1o+70x2e+7x3o")}[which]
+              "ragged": ("5x0e+3x1o+70x2e", "1x0e+1x1o+1x2e", "5x0e+3x1o+70x2e+7x3o"),
+              "few_channels": ("8x0e+8x1o", "1x0e+1x1o+1x2e", "8x0e+8x1o+8x2e")}[which]
     prob, oprob = common.channelwise(irreps)
     nodes, nnz = (300, 9001) if which == "nequip" else (50, 1500)
     conv, (x, y, w, idx, z, g) = _run(prob, oprob, nodes, nnz, 61, True)
     assert isinstance(conv.generator, UVURecvGenerator)
+    assert conv.generator.staged_edges == (staged and which != "few_channels")
     first = [t.grad.clone() for t in (x, y, w)]
     for t in (x, y, w):
         t.grad = None
@@ -145,16 +156,22 @@ STAGED_SHAPES = {
 
 
 @pytest.mark.parametrize("shape", sorted(STAGED_SHAPES))
-@pytest.mark.parametrize("deterministic", [False, True])
-def test_lds_staged_edge_loop_shapes(cuda, shape, deterministic):
+@pytest.mark.parametrize("variant", ["unsorted", "det_send", "det_recv"])
+def test_lds_staged_edge_loop_shapes(cuda, shape, variant, monkeypatch):
     """Single-chunk fp32 problems run the edge loop that stages operands through LDS (deterministic:
-    forward and backward; unsorted: forward): every sub-list count, ragged multiplicities, and records of
-    1, 3, 5 and 7 words (one, one, two and two LDS-DMA transfers), with long and empty edge lists."""
+    forward and backward, in sender order and in pass 1 of the receiver order; unsorted: forward): every
+    sub-list count, ragged multiplicities, and records of 1, 3, 5 and 7 words (one, one, two and two LDS-DMA
+    transfers), with long and empty edge lists."""
+    from openequivariance_amd import tunables
     from openequivariance_amd.conv import select_conv_generator
+    deterministic = variant != "unsorted"
+    if deterministic:
+        monkeypatch.setattr(tunables.current, "det_backward", variant[4:])
     prob, oprob = common.channelwise(STAGED_SHAPES[shape])
     gen = select_conv_generator(prob, deterministic)
     staged = gen if deterministic else gen.fwd
-    assert staged.lds_forward and (staged.lds_backward or not deterministic)
+    assert staged.lds_forward
+    assert {"unsorted": True, "det_send": staged.lds_backward, "det_recv": getattr(staged, "staged_edges", False)}[variant]
     _run(prob, oprob, 23, 700, 40, deterministic)        # about 30 edges per node
     _run(prob, oprob, 200, 150, 41, deterministic)       # most nodes have no edge or a single one
 
