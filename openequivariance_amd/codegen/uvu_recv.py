@@ -34,7 +34,7 @@ class UVURecvGenerator(UVUDetGenerator):
     # edge's operands in registers and the regrouped form spills 27 instead of 13 words per lane on the 128-channel
     # MACE problem (2.63 against 2.08 ms); with the operands staged through LDS it needs fewer registers than the
     # pair-at-a-time form (175 against 218 there) and is faster on every shape measured (MACE 1.73 against 1.81 ms,
-    # 256 channels 6.97 against 7.55 ms).
+    # 256 channels with outputs of either parity 9.5 against 9.8 ms).
     regroup_pairs = False
     REGROUP_STAGED = True
     # Tile counts from 4096 to one tile per 16 edges and 2 / 4 / 8 spill rows in flight in pass 2 moved pass 1 by
@@ -69,7 +69,7 @@ class UVURecvGenerator(UVUDetGenerator):
         # backward, register loads against staged (both pair-at-a-time): MACE problem 2.07 -> 1.83 ms, 256 channels
         # with outputs of either parity 16.3 -> 9.9 ms, 256 channels 7.84 -> 7.74 ms, 32 channels 0.201 -> 0.179 ms.
         # The staged kernels are left to the occupancy their register count gives (138 - 175: two or three
-        # wavefronts per SIMD; held to exactly two: 256 channels 6.97 instead of 6.76 ms).
+        # wavefronts per SIMD).
         self.can_stage = self.T == "float" and self.P >= self.D2      # (the Y slab holds one word per lane of a row's group)
         self.staged_edges = self.can_stage and (True if staged is None else bool(staged))
         self.regroup_pairs = bool(self.REGROUP_STAGED and self.staged_edges)

@@ -92,7 +92,7 @@ def sort_by_receiver(rows: "torch.Tensor", cols: "torch.Tensor", node_count: typ
 
 
 # d3 / d1 from which the deterministic backward walks the edges in receiver order (see select_conv_generator)
-RECV_ORDER_MIN_RATIO = 4.5
+RECV_ORDER_MIN_RATIO = 5.5
 
 
 def select_conv_generator(config: TPProblem, deterministic: bool, vector_stores: bool = True, idx_dtype=np.int64):
@@ -107,11 +107,12 @@ def select_conv_generator(config: TPProblem, deterministic: bool, vector_stores:
             # bit of the result - differ between processes).  The sender order gathers a dZ row per edge (d3
             # words, reads); the receiver order gathers an X row and writes and re-reads a dX row (3 d1 words,
             # half of them writes), and pays off when pass 1 can stage its operands through LDS.  Measured
-            # backward, sender against receiver order: d3 / d1 = 3.9 (32 channels) 0.164 / 0.176 ms, 4.8 (256
-            # channels) 7.55 / 6.76 ms, 5.7 (32 channels, outputs of either parity) 0.225 / 0.208 ms, 7.1 (256
-            # channels, either parity) 10.96 / 9.32 ms, 7.9 (the 128-channel MACE problem) 2.15 / 1.73 ms.
-            # Without the stage (fp64, or fewer channels than Y components) pass 1 runs one edge at a time:
-            # 16.3 against 10.96 ms at 7.1; those problems keep the sender order.
+            # backward, sender against receiver order, each as the first operator of a fresh process and in
+            # steady state: d3 / d1 = 3.9 (32 channels) 0.162 / 0.175 ms, 4.8 (256 channels) 7.53 / 7.68 ms, 5.7
+            # (32 channels, outputs of either parity) 0.223 / 0.208 ms, 7.1 (256 channels, either parity) 10.94 /
+            # 9.43 ms, 7.9 (the 128-channel MACE problem) 2.14 / 1.71 ms.  Without the stage (fp64, or fewer
+            # channels than Y components) pass 1 runs one edge at a time: 16.3 against 10.96 ms at 7.1; those
+            # problems keep the sender order.
             order = "send"
             if config.irreps_out.dim >= RECV_ORDER_MIN_RATIO * config.irreps_in1.dim:
                 g = UVURecvGenerator(config, vector_stores=vector_stores, idx_ctype=idx_ctype)

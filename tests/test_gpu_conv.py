@@ -84,16 +84,18 @@ def test_conv_outputs_of_either_parity(cuda, which, deterministic):
 
 
 def test_deterministic_backward_order_is_chosen_by_shape(cuda):
-    """Static rule: the two-pass receiver-order backward when a dZ row is at least 4.5 times as long as an X row
+    """Static rule: the two-pass receiver-order backward when a dZ row is at least 5.5 times as long as an X row
     and pass 1 can stage its operands through LDS (fp32, at least as many channels per row group as Y
-    components): the MACE problem (7.9) and config 5 (4.8) take it, config 3 (3.9) and fp64 problems keep the
-    sender order."""
+    components): the MACE problem (7.9) and configs 3 and 5 with outputs of either parity (5.7, 7.1) take it,
+    configs 3 and 5 themselves (3.9, 4.8) and fp64 problems keep the sender order."""
+    from openequivariance_amd import workloads
     from openequivariance_amd.codegen.uvu_recv import UVURecvGenerator
     from openequivariance_amd.conv import select_conv_generator
-    for irreps in (common.MACE, common.LARGE):
+    for irreps in (common.MACE, workloads.NEQUIP_ALL, workloads.LARGE_ALL):
         g = select_conv_generator(common.channelwise(irreps)[0], True)
         assert isinstance(g, UVURecvGenerator) and g.staged_edges and g.regroup_pairs
-    assert not isinstance(select_conv_generator(common.channelwise(common.NEQUIP)[0], True), UVURecvGenerator)
+    for irreps in (common.NEQUIP, common.LARGE):
+        assert not isinstance(select_conv_generator(common.channelwise(irreps)[0], True), UVURecvGenerator)
     assert not isinstance(select_conv_generator(common.channelwise(common.MACE, dtype=np.float64)[0], True), UVURecvGenerator)
     prob, oprob = common.channelwise(common.MACE)
     _run(prob, oprob, 60, 900, 40, True, sh_lmax=3)
