@@ -515,6 +515,75 @@ def conv_band_probe():
     print(json.dumps(out))
 
 
+MFMA_PROBE_SRC = r"""
+// Wavefronts that do nothing but matrix-core instructions on NACC independent accumulators, with VALU dependent
+// multiply-adds on the operand registers after each of them.  SHAPE 32: v_mfma_f32_32x32x2_f32, 16: v_mfma_f32_16x16x4_f32.
+typedef float V4 __attribute__((ext_vector_type(4)));
+typedef float V16 __attribute__((ext_vector_type(16)));
+extern "C" __global__ void __launch_bounds__(64) oeq_mfma_probe(float* out, int iters) {
+    const float a = (float)threadIdx.x * 1e-3f, b = (float)blockIdx.x * 1e-6f;
+#if SHAPE == 32
+    V16 acc[NACC];
+    for (int i = 0; i < NACC; ++i) for (int r = 0; r < 16; ++r) acc[i][r] = 0;
+#else
+    V4 acc[NACC];
+    for (int i = 0; i < NACC; ++i) for (int r = 0; r < 4; ++r) acc[i][r] = 0;
+#endif
+    float v[8] = {a, b, a + b, a - b, a * 2, b * 2, a + 1, b + 1};
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < NACC; ++i) {
+#if SHAPE == 32
+            acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(v[i & 7], v[(i + 1) & 7], acc[i], 0, 0, 0);
+#else
+            acc[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(v[i & 7], v[(i + 1) & 7], acc[i], 0, 0, 0);
+#endif
+#pragma unroll
+            for (int q = 0; q < VALU; ++q) v[(i + q) & 7] = v[(i + q) & 7] * 1.0001f + v[(i + q + 3) & 7];
+        }
+    }
+    float s = 0;
+    for (int i = 0; i < NACC; ++i) s += acc[i][0] + acc[i][3];
+    for (int q = 0; q < 8; ++q) s += v[q];
+    if (s == 12345.678f) out[0] = s;
+}
+"""
+
+
+def mfma_rate_probe():
+    """What the fp32 matrix cores sustain on this GPU, and what vector-ALU instructions between the matrix
+    instructions cost: the yardstick for the dense uvw kernels (157.3 TFLOP/s is the datasheet figure at the
+    peak clock).  Grid = wavefronts per SIMD x 4 SIMDs x compute units, one wavefront per workgroup."""
+    import ctypes as C
+    import torch
+    from openequivariance_amd import runtime as rt
+    out = torch.zeros(16, device="cuda")
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    stream = torch.cuda.current_stream().cuda_stream
+    iters, nacc = 2000, 4
+    rec = {"workload": "mfma_rate_probe", "unit": "TFLOP/s", "peak": MFMA_FP32_PEAK_TFLOPS, "compute_units": cus,
+           "accumulators": nacc, "variants": []}
+    for shape in (16, 32):
+        for valu in (0, 1, 2, 4, 8):
+            for wps in (1, 2, 3):
+                opts = tuple(rt.DEFAULT_OPTIONS) + (f"-DSHAPE={shape}", f"-DNACC={nacc}", f"-DVALU={valu}")
+                mod = rt.Module(rt.compile_source(MFMA_PROBE_SRC, options=opts))
+                grid = cus * 4 * wps
+                best = float("inf")
+                for r in range(5):
+                    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    a.record()
+                    mod.launch("oeq_mfma_probe", grid, 64, [C.c_void_p(out.data_ptr()), C.c_int(iters)], stream=stream)
+                    b.record()
+                    b.synchronize()
+                    if r >= 1:
+                        best = min(best, a.elapsed_time(b))
+                flops = (4096 if shape == 32 else 2048) * nacc * iters * grid
+                rec["variants"].append({"mfma": "32x32x2" if shape == 32 else "16x16x4", "valu_per_mfma": valu,
+                                        "wavefronts_per_simd": wps, "TFLOP/s": round(flops / best / 1e9, 1)})
+    print(json.dumps(rec))
+
+
 def measure_torch_op(case, ev, steps, warmup, raw_ms):
     """The operator a user calls (reference protocol: implementations/TensorProductBase.py:114-219 and
     convolution/ConvolutionBase.py:251-411 time the torch op when torch_op=True): ``steps`` forward +
@@ -676,6 +745,9 @@ def main():
         return
     if args.workload == "conv_band_probe":
         conv_band_probe()
+        return
+    if args.workload == "mfma_rate_probe":
+        mfma_rate_probe()
         return
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (the path shards over rows/edges "

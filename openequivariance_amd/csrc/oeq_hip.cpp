@@ -66,6 +66,8 @@ int load_steps(Module& m, const void* code, size_t code_size, const oeq_step* st
         s.desc.kernel[sizeof(s.desc.kernel) - 1] = 0;
         if (s.desc.num_threads == 0 || s.desc.num_threads > 1024)
             return fail("step %d (%s): bad workgroup size %u", i, s.desc.kernel, s.desc.num_threads);
+        if (s.desc.grid_kind > OEQ_GRID_PER_NODE_AND_PIECE)
+            return fail("step %d (%s): unknown grid rule %u", i, s.desc.kernel, s.desc.grid_kind);
         if (s.desc.grid_kind != OEQ_GRID_FIXED && s.desc.work_per_block == 0)
             return fail("step %d (%s): work_per_block must be > 0", i, s.desc.kernel);
         if (s.desc.grid_kind == OEQ_GRID_FIXED && s.desc.num_blocks == 0)
