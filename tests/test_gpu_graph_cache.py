@@ -101,9 +101,10 @@ def test_cache_is_off_by_default_and_sees_writes_behind_torchs_back(cuda, determ
 
 
 @pytest.mark.parametrize("deterministic", [True, False])
-@pytest.mark.parametrize("irreps", [common.NEQUIP, common.LARGE], ids=["nequip", "large"])
+@pytest.mark.parametrize("irreps", [common.NEQUIP, common.LARGE, common.MACE], ids=["nequip", "large", "mace"])
 def test_int32_indices(cuda, deterministic, irreps):
-    """reference: LoopUnrollConv.py:53,78 accepts int32 and int64 index tensors."""
+    """reference: LoopUnrollConv.py:53,78 accepts int32 and int64 index tensors.  (The MACE problem takes the
+    receiver-order backward when deterministic.)"""
     import torch
     import openequivariance_amd as oeq
     prob, oprob = common.channelwise(irreps)
