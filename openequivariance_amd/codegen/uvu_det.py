@@ -301,14 +301,18 @@ class UVUDetGenerator(UVUDirectGenerator):
             if blk.idx in used and blk.dim:
                 self.emit_sub_sum(E, regs_of(blk))
 
-        def store(E, base: str, row: str, existing: bool, zero: bool):
+        def store(E, base: str, row: str, existing: bool, zero: bool, agent: bool = False):
             for blk in blocks:
                 if blk.dim == 0:
                     continue
                 E("{")
                 E.level += 1
                 dst = f"{base} + {row} * {rowdim} + {blk.off} + u * {blk.D}"
-                if blk.idx in used and self.R == 1 and via_lds:
+                if agent:                   # a partial row, read by a wavefront that may sit on another XCD
+                    if blk.idx in used:
+                        E(f"if ({self.store_act(blk)}) {{ T* __restrict__ p_ = {dst}; "
+                          + " ".join(f"oeq_st_agent(p_ + {m}, {n});" for m, n in enumerate(regs_of(blk))) + " }")
+                elif blk.idx in used and self.R == 1 and via_lds:
                     self.emit_block_store(E, blk, regs_of(blk), base, rowdim, row, (lambda r: (row, "nv")), "store",
                                           via_lds=True)
                 elif blk.idx in used:
@@ -333,20 +337,22 @@ class UVUDetGenerator(UVUDirectGenerator):
         E("// counters: one per slot for the groups of pieces, one per slot for the whole node")
         E(f"int* __restrict__ tk_ = (int*)((char*)ws + {self.piece_base}) + (u64)c * 4 * tiles_;")
         E(f"T* __restrict__ prow_ = (T*)((char*)ws + {self.piece_base} + ((16ull * {self.NCH} * tiles_ + 255ull) & ~255ull) + 256ull);")
-        store(E, "prow_", "slot", False, False)
+        store(E, "prow_", "slot", False, False, agent=True)
         E(f"// Piece k of the node sits in slot 2 qh + 1 (k = 0) or 2 (qh + k).  The pieces are added in two levels, each")
         E(f"// by whoever finishes last: groups of {G} consecutive pieces in list order (the sum replaces the group's first")
         E(f"// piece), then the groups in order.  Which wavefront adds does not change what is added in which order.")
+        E("// The partial rows are written and read at agent scope; a ticket is drawn when the row's stores have completed")
+        E("// (release / acquire fences here would write back and invalidate this XCD's whole L2 once per piece: with 256")
+        E("// nodes of 586 edges among 150 000 the forward took 0.32 ms with them and 0.22 ms without any pieces).")
         E(f"const int k_own_ = slot == 2 * qh + 1 ? 0 : (int)(slot / 2 - qh);")
         E(f"int first_ = (k_own_ / {G}) * {G}, cnt_ = min({G}, npieces - first_), stride_ = 1, level_ = 0;")
-        E("oeq_release_agent();")
+        E("oeq_wait_vm();")
         E("int old_ = 0;")
         E("if (lane == 0) old_ = oeq_ticket_add(tk_ + (first_ == 0 ? 2 * qh + 1 : 2 * (qh + (u64)first_)));")
         E("old_ = __builtin_amdgcn_readfirstlane(old_);")
         E("bool go_ = old_ == cnt_ - 1;")
         E("while (go_) {")
         E.level += 1
-        E("oeq_acquire_agent();")
         for blk in blocks:
             if blk.idx in used and blk.dim:
                 E(" ".join(f"{n} = (T)0;" for n in regs_of(blk)))
@@ -357,7 +363,7 @@ class UVUDetGenerator(UVUDirectGenerator):
         for blk in blocks:
             if blk.idx in used and blk.dim:
                 E(f"{{ const T* __restrict__ q_ = prow_ + srow_ * {rowdim} + {blk.off} + {self.uclamp(blk, 0)} * {blk.D}; "
-                  + " ".join(f"{n} += q_[{m}];" for m, n in enumerate(regs_of(blk))) + " }")
+                  + " ".join(f"{n} += oeq_ld_agent(q_ + {m});" for m, n in enumerate(regs_of(blk))) + " }")
         E.level -= 1
         E("}")
         E("const u64 grow_ = first_ == 0 ? 2 * qh + 1 : 2 * (qh + (u64)first_);       // slot of the group's first piece")
@@ -369,9 +375,9 @@ class UVUDetGenerator(UVUDirectGenerator):
         E.level -= 1
         E("} else {")
         E.level += 1
-        store(E, "prow_", "grow_", False, False)
+        store(E, "prow_", "grow_", False, False, agent=True)
         E("if (lane == 0) tk_[grow_] = 0;")
-        E("oeq_release_agent();")
+        E("oeq_wait_vm();")
         E("old_ = 0;")
         E("if (lane == 0) old_ = oeq_ticket_add(tk_ + 2 * tiles_ + 2 * qh + 1);")
         E("old_ = __builtin_amdgcn_readfirstlane(old_);")

@@ -81,6 +81,9 @@ class Workload:
     # True: X, W and G are drawn on the GPU with torch's generator (the large workload's weights
     # are 10.6 GB; drawing them on the host takes minutes); the graph and Y still come from numpy
     device_inputs: bool = False
+    # probe graphs: receivers drawn from the first ``receiver_pool`` nodes only (0: from all), so that the dZ
+    # rows the backward gathers fit a cache of a known size
+    receiver_pool: int = 0
 
     @property
     def data_note(self) -> str:
@@ -120,7 +123,7 @@ class Workload:
             rows = np.repeat(np.arange(N, dtype=np.int64), deg)
             cols = rng.integers(0, N, rows.size).astype(np.int64)
         else:
-            rows = rng.integers(0, N, E).astype(np.int64)
+            rows = rng.integers(0, self.receiver_pool or N, E).astype(np.int64)
             cols = rng.integers(0, N, E).astype(np.int64)
             clash = rows == cols
             cols[clash] = (cols[clash] + 1 + rng.integers(0, N - 1, int(clash.sum()))) % N
@@ -278,6 +281,14 @@ def get(name: str) -> Workload:
         w = Workload(name, "single-path uvu TP 1x2e (x) 1x3e -> 1x2e, batch 1000, fp32", "tp",
                      ("1x2e", "1x3e", "1x2e"), 1000, "rows/s", "hbm", "f32", 12345, {"batch": 1000, "paths": 1})
         w.alg_bytes = _tp_bytes(w.problem(), w.units, 4)
+        return w
+    if name.startswith("nequip_conv_det_receivers"):
+        # the deterministic NequIP convolution on a graph whose receivers are all among the first k nodes: a dZ
+        # working set of k x 4480 bytes for the backward's gathers (probe of what cache-resident dZ would buy)
+        k = int(name[len("nequip_conv_det_receivers"):])
+        w = get("nequip_conv_det")
+        w.name, w.receiver_pool = name, k
+        w.description += f", receivers among the first {k} nodes only"
         return w
     if name in ("nequip_conv_atomic", "nequip_conv_det"):
         det = name.endswith("det")

@@ -68,6 +68,8 @@ static inline void oeq_release_agent() {}
 static inline void oeq_acquire_agent() {}
 static inline int oeq_ticket_add(int* p) { std::lock_guard<std::mutex> g(g_atomic_mutex); return (*p)++; }
 static inline i64 oeq_lds_claim(i64* slot, i64 key) { std::lock_guard<std::mutex> g(g_atomic_mutex); const i64 old = *slot; if (old == -1) *slot = key; return old; }
+static inline void oeq_st_agent(T* p, T v) { *p = v; }
+static inline T oeq_ld_agent(const T* p) { return *p; }
 static inline int oeq_lds_add(int* p, int v) { std::lock_guard<std::mutex> g(g_atomic_mutex); const int o = *p; *p += v; return o; }
 static inline void oeq_wait_vm() {}
 static inline void oeq_wait_lds() {}

@@ -161,6 +161,26 @@ def test_conv_det_long_edge_lists(staged):
         assert rel_err(got, ref) < TOL
 
 
+def test_conv_long_runs_of_nodes_without_edges():
+    """Receivers only among the first three nodes and senders only among the last ten of 700: the CSR pointers of
+    the 690 nodes in between are written by the whole workgroup of the preparation kernels, not by one thread."""
+    prob, oprob = common.channelwise(("8x0e+8x1o", "1x0e+1x1o", "8x0e+8x1o"))
+    g = UVUDetGenerator(prob)
+    nodes, nnz = 700, 90
+    rng = np.random.default_rng(5)
+    rows, cols = rng.integers(0, 3, nnz), rng.integers(690, 700, nnz)
+    rows, cols, tperm, _ = otp.coord_graph(rows, cols)
+    X, Y, W, G = common.conv_inputs(prob, nodes, nnz, 6)
+    fwd, bwd, ws = g.plan()
+    out = emu.run_conv(g, fwd, X, Y, W, rows, cols, tperm=tperm, ws_bytes=ws(nnz, nodes))
+    assert rel_err(out["Z"], otp.conv_forward(oprob, X, Y, W, rows, cols)) < TOL
+    assert not out["Z"][3:].any()
+    out = emu.run_conv(g, bwd, X, Y, W, rows, cols, G=G, tperm=tperm, ws_bytes=ws(nnz, nodes))
+    for got, ref in zip((out["Xg"], out["Yg"], out["Wg"]), otp.conv_backward(oprob, X, Y, W, G, rows, cols)):
+        assert rel_err(got, ref) < TOL
+    assert not out["Xg"][:690].any()
+
+
 def test_conv_blocks_no_path_touches_are_zero_filled():
     """in1 holds a 16-channel l = 3 block that no path reads while the blocks in use have one channel: its
     dX columns must come out as zeros (the emulator starts the deterministic outputs from junk)."""
