@@ -43,9 +43,13 @@ class UVURecvGenerator(UVUDetGenerator):
     MAX_TILES = 16384        # tiles per chunk of the largest launches (the tile then grows with the edge count)
     DX_UNROLL = 4            # spill rows in flight per lane group in pass 2
 
-    def __init__(self, problem: TPProblem, vector_stores: bool = True, idx_ctype: str = "i64", prefetch=None, staged=None):
-        # pass 1 is one launch: the per-edge dX rows cannot be split over launches of output-block groups
-        super().__init__(problem, vector_stores=vector_stores, idx_ctype=idx_ctype, allow_split=False)
+    def __init__(self, problem: TPProblem, vector_stores: bool = True, idx_ctype: str = "i64", prefetch=None, staged=None,
+                 backward_perm: bool = False):
+        # pass 1 is one launch: the per-edge dX rows cannot be split over launches of output-block groups.
+        # ``backward_perm``: the edge list is in no order; pass 1 walks the receiver-grouped position list and pass
+        # 2 the sender-grouped one, both built in the workspace by the grouping kernels (pass 1 staged only).
+        super().__init__(problem, vector_stores=vector_stores, idx_ctype=idx_ctype, allow_split=False,
+                         backward_perm=backward_perm)
         assert self.H == 1
         self.lds_backward = False
         self.waves_per_eu = 0
@@ -75,7 +79,8 @@ class UVURecvGenerator(UVUDetGenerator):
         self.regroup_pairs = bool(self.REGROUP_STAGED and self.staged_edges)
         if self.staged_edges:
             self.waves_hint = 0
-        self.dypart_off = "(2 * (node_count + 1) + node_count) * sizeof(i64)"
+        if not backward_perm:
+            self.dypart_off = "(2 * (node_count + 1) + node_count) * sizeof(i64)"
         self.spill_off = (f"((({self.dypart_off} + {self.dy_slots if self.dy_slots > 1 else 0}ull * nnz * {self.D2} * sizeof(T)) "
                           "+ 255ull) & ~255ull)")
         # the preparation's per-256-edge flags are not used here (pass 1 visits every edge and writes the
@@ -107,7 +112,8 @@ class UVURecvGenerator(UVUDetGenerator):
         return fwd, bwd, ws
 
     def main_bytes(self, nnz: int, nodes: int) -> int:
-        head = (2 * (nodes + 1) + nodes) * 8 + self.dy_partial_bytes(nnz)
+        head = (2 * self.group_bytes(nnz, nodes) if self.backward_perm else 2 * (nodes + 1) * 8) + nodes * 8 \
+            + self.dy_partial_bytes(nnz)
         return ((((head + 255) & ~255) + self.spill_bytes(nnz) + self.flag_bytes(nnz)) + 255) & ~255
 
     def backward_kernel_sources(self):
@@ -264,11 +270,47 @@ class UVURecvGenerator(UVUDetGenerator):
         E(f"const u64 tile = item / {NCH};")
         E(f"const int u = c * {P} + ul;")
         E(f"const u64 per = ((nnz + tiles - 1) / tiles + {R - 1}) / {R} * {R};       // edges per tile")
-        E("const u64 beg = min(tile * per, nnz);")
-        E("const int len = (int)(min(beg + per, nnz) - beg);")
+        if self.backward_perm:
+            # positions of the receiver-grouped list: it holds the edges with a valid receiver, nothing behind them
+            E("i64 listed_ = ((const i64*)ws)[node_count]; if (listed_ < 0) listed_ = 0; if (listed_ > (i64)nnz) listed_ = (i64)nnz;")
+            E("const u64 last = (u64)listed_;")
+        else:
+            E("const u64 last = nnz;")
+        E("const u64 beg = min(tile * per, last);")
+        E("const int len = (int)(min(beg + per, last) - beg);")
         E(f"const int maxlen = (len + {R - 1}) / {R};")
         E(f"T* __restrict__ spill = (T*)((char*)ws + {self.spill_off});")
         self._cur_c = "e"
+        if self.backward_perm:
+            # Edges naming no receiver are in no group: nobody visits them.  The grouping kernels leave one flag per
+            # 256 edges; the first workgroup of every chunk ORs them and, only if one is set, walks the edge list
+            # and zeroes the rows of such edges: dW, dY (or this chunk's dY partial) and the dX row pass 2 will read.
+            E("if (tile == 0) {")
+            E.level += 1
+            E("const int* __restrict__ bad_ = (const int*)((const char*)ws + FLAGS_OFF);")
+            E("int any_ = 0;")
+            E("for (u64 q = lane; q < (nnz + 255) / 256; q += 64) any_ |= bad_[q];")
+            for m in (32, 16, 8, 4, 2, 1):
+                E(f"any_ |= oeq_shfl_xor_i32(any_, {m});")
+            E("if (any_) {")
+            E.level += 1
+            E("for (u64 e = lane; e < nnz; e += 64) {")
+            E.level += 1
+            E("const i64 r_ = rows[e];")
+            E("if (r_ >= 0 && r_ < (i64)node_count) continue;")
+            E(f"if (c == 0) for (int q = 0; q < {self.WN}; ++q) Wg[e * {self.WN} + q] = (T)0;")
+            if self.dy_slots > 1:
+                E(f"{{ T* __restrict__ p_ = (T*)((char*)ws + DYPART_OFF) + ((u64)c * nnz + e) * {self.D2}; "
+                  f"for (int q = 0; q < {self.D2}; ++q) p_[q] = (T)0; }}")
+            else:
+                E(f"if (c == 0) for (int q = 0; q < {self.D2}; ++q) Yg[e * {self.D2} + q] = (T)0;")
+            E(f"{{ T* __restrict__ p_ = spill + ((e * {NCH} + c) * {self.NW}) * {P}; for (int q = 0; q < {self.NW * P}; ++q) p_[q] = (T)0; }}")
+            E.level -= 1
+            E("}")
+            E.level -= 1
+            E("}")
+            E.level -= 1
+            E("}")
         E("bool rv = false;")
         for oi in self.used_out:
             E("T " + ", ".join(f"G{oi}_{k} = (T)0" for k in range(self.out[oi].D)) + ";")
@@ -394,7 +436,11 @@ class UVURecvGenerator(UVUDetGenerator):
             E(" ".join(f"pdy{f} = dy{f};" for f in self.used_y))
             E(" ".join(f"pdx{i}_{m} = dx{i}_{m};" for i in self.used_in1 for m in range(self.in1[i].D)))
             E("pe = e; pv = rv; pev = cur_ev;")
-        self.emit_staged_loop(E, self.edge_pos, None, "cols", dma, readback, compute, flush, pre=pre)
+        plist = None
+        if self.backward_perm:
+            E("const i64* __restrict__ rlist = (const i64*)ws + 2 * (node_count + 1);     // edge ids grouped by receiver")
+            plist = "rlist"
+        self.emit_staged_loop(E, self.edge_pos, plist, "cols", dma, readback, compute, flush, pre=pre)
         return E.text()
 
     # ---------------------------------------------------------------- pass 2
@@ -402,7 +448,10 @@ class UVURecvGenerator(UVUDetGenerator):
         E = Emitter()
         P, NCH, U = self.P, self.NCH, self.DX_UNROLL
         self.emit_lane_direct(E, lds=False)
-        E("const IDX* __restrict__ elist = tperm;     // edge ids in (sender, receiver) order")
+        if self.backward_perm:
+            E(f"const i64* __restrict__ elist = {self.bwd_list};     // edge ids grouped by sender")
+        else:
+            E("const IDX* __restrict__ elist = tperm;     // edge ids in (sender, receiver) order")
 
         def key(E, pos):
             E(f"{{ const i64 e0_ = (i64)elist[{pos}]; if (e0_ >= 0 && e0_ < (i64)nnz) kv_ = (i64)cols[e0_]; }}")

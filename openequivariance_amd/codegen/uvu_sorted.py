@@ -28,6 +28,7 @@ from ..problem import TPProblem
 from .common import jinja_env
 from .uvu_det import UVUDetGenerator
 from .uvu_direct import UVUDirectGenerator
+from .uvu_recv import UVURecvGenerator
 
 
 class UVUSortedGenerator:
@@ -42,15 +43,27 @@ class UVUSortedGenerator:
     # torch operator measures both on first use either way.
     ATOMIC_BACKWARD_MAX_D1 = 128
 
-    def __init__(self, problem: TPProblem, vector_stores: bool = True, grouped_backward=None, idx_ctype: str = "i64"):
+    # dZ row / X row from which the grouped backward runs in receiver order (same measurements as the rule of the
+    # deterministic operator, conv.RECV_ORDER_MIN_RATIO; here the receiver grouping costs a second counting sort)
+    RECV_ORDER_MIN_RATIO = 5.5
+
+    def __init__(self, problem: TPProblem, vector_stores: bool = True, grouped_backward=None, idx_ctype: str = "i64",
+                 recv_backward=None):
         self.problem = problem
         self.fwd = UVUDetGenerator(problem, forward_perm=True, vector_stores=vector_stores, idx_ctype=idx_ctype)
         if grouped_backward is None:
             forced = tunables.current.conv_backward               # "grouped" / "atomic": A/B runs
             grouped_backward = (forced == "grouped") if forced else self.fwd.D1 >= self.ATOMIC_BACKWARD_MAX_D1
         self.grouped_backward = grouped_backward
+        self.recv_backward = False
         if grouped_backward:
             self.bwd = UVUDetGenerator(problem, backward_perm=True, vector_stores=vector_stores, idx_ctype=idx_ctype)
+            if recv_backward is not False and (recv_backward or self.fwd.D3 >= self.RECV_ORDER_MIN_RATIO * self.fwd.D1):
+                # long dZ rows: the two-pass backward in receiver order (pass 1 over the receiver grouping, which the
+                # backward then builds as well; pass 2 over the sender grouping), where pass 1 can stage its operands
+                recv = UVURecvGenerator(problem, vector_stores=vector_stores, idx_ctype=idx_ctype, backward_perm=True)
+                if recv.staged_edges:
+                    self.bwd, self.recv_backward = recv, True
         else:
             self.bwd = UVUDirectGenerator(problem, "conv_atomic", vector_stores=vector_stores)
             self.bwd.idx_ctype = idx_ctype
@@ -93,9 +106,11 @@ class UVUSortedGenerator:
                 return ((G(nnz, nodes) + 255) & ~255) + f.piece_bytes(nnz, nodes)
             return fwd, bwd, ws
         b = self.bwd
-        bwd = grouping("_backward") + b.backward_steps()
+        bwd = (grouping("_recv") if self.recv_backward else []) + grouping("_backward") + b.backward_steps()
 
         def ws(nnz=0, nodes=0):
+            if self.recv_backward:
+                return b.main_bytes(nnz, nodes) + b.piece_bytes(nnz, nodes)
             main = 2 * G(nnz, nodes) + b.order_bytes(nodes) + b.dy_partial_bytes(nnz) + b.flag_bytes(nnz)
             return ((main + 255) & ~255) + b.piece_bytes(nnz, nodes)
         return fwd, bwd, ws

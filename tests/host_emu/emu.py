@@ -310,6 +310,8 @@ def run_conv(gen, steps: Sequence[Dict], X, Y, W, rows, cols, G=None, tperm=None
         extra += CONV_EXTRA_SORTED
         if gen.grouped_backward:
             extra += CONV_EXTRA_GROUPED_BWD
+            if gen.recv_backward:
+                extra += CONV_EXTRA_GROUPED_BWD.replace("_backward", "_recv")
             det = gen.bwd
     if det is not None:
         if det.ordered_backward:

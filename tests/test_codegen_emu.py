@@ -58,12 +58,13 @@ def test_generic_tp_shared_weights():
         assert rel_err(got, ref) < TOL
 
 
-@pytest.mark.parametrize("variant", ["atomic", "det", "sorted", "sorted_grouped_backward"])
+@pytest.mark.parametrize("variant", ["atomic", "det", "sorted", "sorted_grouped_backward", "sorted_recv_backward"])
 def test_conv(variant):
     prob, oprob = common.channelwise(common.NEQUIP)
     det = variant == "det"
     g = {"det": UVUDetGenerator, "sorted": lambda p: UVUSortedGenerator(p, grouped_backward=False),
-         "sorted_grouped_backward": lambda p: UVUSortedGenerator(p, grouped_backward=True),
+         "sorted_grouped_backward": lambda p: UVUSortedGenerator(p, grouped_backward=True, recv_backward=False),
+         "sorted_recv_backward": lambda p: UVUSortedGenerator(p, grouped_backward=True, recv_backward=True),
          "atomic": lambda p: UVUDirectGenerator(p, "conv_atomic")}[variant](prob)
     nodes, nnz = 7, 19
     rows, cols = common.random_graph(nodes, nnz, 5)
@@ -78,10 +79,11 @@ def test_conv(variant):
     out = emu.run_conv(g, fwd, X, Y, W, rows, cols, tperm=junk if variant.startswith("sorted") else tperm,
                        ws_bytes=ws(nnz, nodes))
     assert rel_err(out["Z"], otp.conv_forward(oprob, X, Y, W, rows, cols)) < TOL
-    out = emu.run_conv(g, bwd, X, Y, W, rows, cols, G=G, tperm=junk if variant == "sorted_grouped_backward" else tperm,
+    out = emu.run_conv(g, bwd, X, Y, W, rows, cols, G=G, tperm=junk if variant.endswith("_backward") else tperm,
                        ws_bytes=ws(nnz, nodes))
     for got, ref in zip((out["Xg"], out["Yg"], out["Wg"]), otp.conv_backward(oprob, X, Y, W, G, rows, cols)):
         assert rel_err(got, ref) < TOL
+    assert getattr(g, "recv_backward", False) == (variant == "sorted_recv_backward")
 
 
 HUB_CASES = {
@@ -90,7 +92,8 @@ HUB_CASES = {
     "det_two_sublists_registers": (common.NEQUIP, lambda p: UVUDetGenerator(p, lds=False), True),
     "det_two_chunks_two_groups": (("70x0e+70x1o+70x2e", "1x0e+1x1o+1x2e+1x3o", "70x0e+70x1o+70x2e+70x3o"), UVUDetGenerator, True),
     "det_receiver_order": (common.NEQUIP, None, True),
-    "unsorted_grouped": (common.NEQUIP, lambda p: UVUSortedGenerator(p, grouped_backward=True), False),
+    "unsorted_grouped": (common.NEQUIP, lambda p: UVUSortedGenerator(p, grouped_backward=True, recv_backward=False), False),
+    "unsorted_receiver_order": (common.NEQUIP, lambda p: UVUSortedGenerator(p, grouped_backward=True, recv_backward=True), False),
     "unsorted_atomic_backward": (common.NEQUIP, lambda p: UVUSortedGenerator(p, grouped_backward=False), False),
 }
 
@@ -223,31 +226,32 @@ def test_conv_receiver_order_backward(irreps, nodes, nnz, prefetch, staged):
         assert rel_err(got, ref) < TOL
 
 
-@pytest.mark.parametrize("variant", ["det", "det_two_chunks", "grouped", "recv", "recv_staged"])
+@pytest.mark.parametrize("variant", ["det", "det_two_chunks", "grouped", "grouped_recv", "recv", "recv_staged"])
 def test_conv_edges_naming_no_node(variant):
     """Edges whose sender or receiver is out of range contribute nothing, and their dW / dY rows come
     out as zeros from every backward variant (the emulator starts all outputs from junk)."""
     from openequivariance_amd.codegen.uvu_recv import UVURecvGenerator
     irreps = ("70x0e+70x1o", "1x0e+1x1o", "70x0e+70x1o") if variant == "det_two_chunks" else \
-        ("16x0e+16x1o", "1x0e+1x1o+1x2e", "16x0e+16x1o+16x2e") if variant == "recv_staged" else \
+        ("16x0e+16x1o", "1x0e+1x1o+1x2e", "16x0e+16x1o+16x2e") if variant in ("recv_staged", "grouped_recv") else \
         ("8x0e+8x1o", "1x0e+1x1o+1x2e", "8x0e+8x1o+8x2e")
     prob, oprob = common.channelwise(irreps)
     nodes, nnz = 9, 300 if variant != "det_two_chunks" else 40
     rows, cols = common.random_graph(nodes, nnz, 5, self_loops=True)
     rows, cols, valid = common.with_invalid_edges(rows, cols, nodes, 6)
     tperm = None
-    if variant != "grouped":
+    if not variant.startswith("grouped"):
         order = np.lexsort((cols, rows))
         rows, cols, valid = rows[order], cols[order], valid[order]
         tperm = np.lexsort((np.arange(nnz), rows, cols)).astype(np.int64)
     g = {"det": UVUDetGenerator, "det_two_chunks": UVUDetGenerator, "recv": UVURecvGenerator,
          "recv_staged": lambda p: UVURecvGenerator(p, staged=True),
-         "grouped": lambda p: UVUSortedGenerator(p, grouped_backward=True)}[variant](prob)
+         "grouped": lambda p: UVUSortedGenerator(p, grouped_backward=True, recv_backward=False),
+         "grouped_recv": lambda p: UVUSortedGenerator(p, grouped_backward=True, recv_backward=True)}[variant](prob)
     X, Y, W, G = common.conv_inputs(prob, nodes, nnz, 8)
     Zr, dXr, dYr, dWr = common.conv_reference_on_valid_edges(otp, oprob, X, Y, W, G, rows, cols, valid)
     fwd, bwd, ws = g.plan()
     junk = np.full(nnz, 12345, dtype=np.int64)
-    tp = junk if variant == "grouped" else tperm
+    tp = junk if variant.startswith("grouped") else tperm
     out = emu.run_conv(g, fwd, X, Y, W, rows, cols, tperm=tp, ws_bytes=ws(nnz, nodes))
     assert rel_err(out["Z"], Zr) < TOL
     out = emu.run_conv(g, bwd, X, Y, W, rows, cols, G=G, tperm=tp, ws_bytes=ws(nnz, nodes))

@@ -101,13 +101,28 @@ def test_deterministic_backward_order_is_chosen_by_shape(cuda):
     _run(prob, oprob, 60, 900, 40, True, sh_lmax=3)
 
 
+def test_unsorted_mace_conv_backward_in_receiver_order(cuda, monkeypatch):
+    """The unsorted operator's grouped backward takes the receiver order for long dZ rows: it then builds both
+    groupings (by receiver for pass 1, by sender for pass 2) in the backward call."""
+    from openequivariance_amd import tunables
+    monkeypatch.setattr(tunables.current, "autotune", False)
+    prob, oprob = common.channelwise(common.MACE)
+    conv, _ = _run(prob, oprob, 60, 900, 42, False, sh_lmax=3)
+    assert conv.generator.grouped_backward and conv.generator.recv_backward
+    prob, oprob = common.channelwise(common.NEQUIP)
+    conv, _ = _run(prob, oprob, 60, 900, 43, False, sh_lmax=2)
+    assert not conv.generator.recv_backward
+
+
 @pytest.mark.parametrize("deterministic", [False, True])
 def test_mace_conv_backward_split_over_output_blocks(cuda, deterministic, monkeypatch):
     """The MACE problem as a convolution in sender order: 104 registers of operands per edge, so the backward
     runs as two launches over two groups of output blocks (the second adds to dX; dY through per-group partials)."""
     from openequivariance_amd import tunables
     from openequivariance_amd.conv import select_conv_generator
+    from openequivariance_amd.codegen.uvu_sorted import UVUSortedGenerator
     monkeypatch.setattr(tunables.current, "det_backward", "send")
+    monkeypatch.setattr(UVUSortedGenerator, "RECV_ORDER_MIN_RATIO", 1e9)
     prob, oprob = common.channelwise(common.MACE)
     gen = select_conv_generator(prob, True)
     assert gen.H == 2 and sorted(sum(gen.out_groups, [])) == gen.used_out

@@ -110,7 +110,7 @@ def test_tensor_product_rejects_host_tensors_among_gpu_tensors(cuda):
     torch.cuda.synchronize()
 
 
-@pytest.mark.parametrize("variant", ["det", "det_recv", "unsorted_atomic", "unsorted_grouped"])
+@pytest.mark.parametrize("variant", ["det", "det_recv", "unsorted_atomic", "unsorted_grouped", "unsorted_grouped_recv"])
 @pytest.mark.parametrize("irreps", [common.NEQUIP, common.LARGE], ids=["nequip", "large"])
 def test_edges_naming_no_node_contribute_nothing(cuda, variant, irreps, monkeypatch):
     """Out-of-range senders / receivers: no fault, Z and dX as if those edges were absent, and their dW /
@@ -122,7 +122,10 @@ def test_edges_naming_no_node_contribute_nothing(cuda, variant, irreps, monkeypa
     monkeypatch.setattr(tunables.current, "autotune", False)
     monkeypatch.setattr(tunables.current, "det_backward", "recv" if variant == "det_recv" else "send")
     if variant.startswith("unsorted"):
+        from openequivariance_amd.codegen.uvu_sorted import UVUSortedGenerator
         monkeypatch.setattr(tunables.current, "conv_backward", variant.split("_")[1])
+        # (the grouped backward in receiver order is chosen for long dZ rows; here for every shape, or for none)
+        monkeypatch.setattr(UVUSortedGenerator, "RECV_ORDER_MIN_RATIO", 0 if variant.endswith("_recv") else 1e9)
     deterministic = variant.startswith("det")
     prob, oprob = common.channelwise(irreps)
     nodes, nnz = 40, 900
@@ -136,6 +139,7 @@ def test_edges_naming_no_node_contribute_nothing(cuda, variant, irreps, monkeypa
     X, Y, W, G = common.conv_inputs(prob, nodes, nnz, 73)
     Zr, dXr, dYr, dWr = common.conv_reference_on_valid_edges(otp, oprob, X, Y, W, G, rows, cols, valid)
     conv = oeq.TensorProductConv(prob, torch_op=True, deterministic=deterministic)
+    assert getattr(conv.generator, "recv_backward", False) == variant.endswith("grouped_recv")
     x, y, w = (torch.tensor(a, device=cuda, requires_grad=True) for a in (X, Y, W))
     idx = [torch.tensor(a, device=cuda) for a in index]
     for _ in range(2):                               # second pass: graph preparation reused
