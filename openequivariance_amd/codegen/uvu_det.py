@@ -130,7 +130,13 @@ class UVUDetGenerator(UVUDirectGenerator):
         # the forward likewise when the multiplicity fits one chunk: few wavefronts per node, so the
         # registers saved buy a fifth wavefront per SIMD (with several chunks per node it measured 1 % slower)
         fwd_words = self._forward_slabs()[1]
-        self.lds_forward = (self.T == "float" and self.P >= self.D2 and self.NCH == 1 and lds is not False
+        # (with several chunks it pays where an edge brings many operands: 26 - 27 words per lane, forward 0.650 ->
+        # 0.640 ms on the 128-channel MACE problem and 3.65 -> 3.49 ms on 256 channels with outputs of either
+        # parity; with 22 words, 256 channels and 13 paths, 2.583 -> 2.596 ms; not over a position list built on the
+        # fly - the unsorted MACE forward went 0.741 -> 0.775 ms)
+        fwd_operands = sum(self.in1[i].D for i in self.used_in1) + sum(p.mv for p in self.paths)
+        self.lds_forward = (self.T == "float" and self.P >= self.D2 and lds is not False
+                            and (self.NCH == 1 or (fwd_operands >= 26 and not forward_perm) or lds is True)
                             and 16 * (fwd_words + self.lds_elems) * 4 <= 160 * 1024)
         self.uniform_rows = False          # validity is per lane (edge lists differ between sub-rows)
         self.chunk_in_grid = True
