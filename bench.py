@@ -87,7 +87,7 @@ def load_traffic(key):
 
 
 def cpu_baseline(wl, case, sample, seconds=10.0):
-    """e3nn-equivalent torch implementation on the host cores, forward+backward, fp32, on a
+    """e3nn-equivalent torch implementation on the host cores, forward+backward, in the precision of the workload, on a
     bounded sample of the same seeded inputs (the op is independent per row/edge, so the rate of
     the sample is the rate of the workload).  This is the only place where the oracle package is
     used by the benchmark: as the thing timed beside the GPU, never as the product."""
@@ -95,7 +95,7 @@ def cpu_baseline(wl, case, sample, seconds=10.0):
     cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
     h = case.host
     if wl.mode == "uvw":
-        oprob = spec.fully_connected(*wl.irreps, shared_weights=True)
+        oprob = spec.fully_connected(*wl.irreps, shared_weights=wl.shared)
     elif wl.name == "readme_uvu":
         oprob = spec.Problem(*wl.irreps, [(0, 0, 0, "uvu", True)], shared_weights=False)
     else:
@@ -117,7 +117,8 @@ def cpu_baseline(wl, case, sample, seconds=10.0):
         sec = torch_cpu.time_forward_backward(oprob, *args_, threads=cores, repeats=reps, rows=rows, cols=cols)
         what = f"first {n} edges of the same seeded graph (all nodes), {reps} repeats"
     return {"value": round(n / sec, 1), "unit": wl.unit, "cores": cores, "kind": "port",
-            "sample": what + "; torch CPU einsum + autograd, fp32 (e3nn itself is not installable offline)"}
+            "sample": what + f"; torch CPU einsum + autograd, {'fp32' if wl.dtype == 'f32' else 'fp64'} "
+                      "(e3nn itself is not installable offline)"}
 
 
 COPY_SRC = r"""
@@ -732,7 +733,7 @@ def measure(name, steps, warmup, cold=True, cpu=True, cpu_sample=0, ceiling=True
 
 # every BASELINE configuration besides the headline one (config 2 = mace_uvu), and the MACE problem as a convolution
 OTHER_WORKLOADS = ("readme_uvu", "nequip_conv_det", "nequip_conv_atomic", "dense_uvw_f32", "dense_uvw_f64",
-                   "large_conv_det", "large_conv_atomic", "mace_conv_det")
+                   "large_conv_det", "large_conv_atomic", "mace_conv_det", "diffdock_uvw_f32")
 
 
 def main():

@@ -19,6 +19,7 @@ from . import runtime as rt
 from .autograd_glue import double_backward_terms
 from .codegen.uvu import UVUGenerator
 from .codegen.uvu_direct import UVUDirectGenerator
+from .codegen.uvw_batched import UVWBatchedGenerator
 from .problem import TPProblem
 from .weight_order import WeightReorder
 from .wigner import wigner_3j
@@ -158,6 +159,14 @@ class TensorProduct(TensorProductBase):
             # rare: a caller-supplied tensor that is not 16-byte aligned -> kernels without vector stores
             if self._internal_unaligned is None:
                 g = UVUDirectGenerator(self.config, "tp", vector_stores=False)
+                fwd, bwd, _ = g.plan()
+                self._internal_unaligned = rt.TPImpl(rt.compile_source(g.render()), _make_steps(fwd, self._step_flags),
+                                                     _make_steps(bwd, self._step_flags))
+            return self._internal_unaligned
+        if isinstance(self.generator, UVWBatchedGenerator) and self.generator.pairs and any(int(p) % 8 for p in ptrs):
+            # the same for the per-row-weights uvw kernels, which move fp32 weights two words at a time
+            if self._internal_unaligned is None:
+                g = UVWBatchedGenerator(self.config, pairs=False)
                 fwd, bwd, _ = g.plan()
                 self._internal_unaligned = rt.TPImpl(rt.compile_source(g.render()), _make_steps(fwd, self._step_flags),
                                                      _make_steps(bwd, self._step_flags))

@@ -28,6 +28,8 @@ NEQUIP_ALL = ("32x0e+32x1o+32x2e", "1x0e+1x1o+1x2e", "32x0e+32x1o+32x1e+32x2e+32
 LARGE_ALL = ("256x0e+256x1o+256x2e", "1x0e+1x1o+1x2e+1x3o", "256x0e+256x1o+256x1e+256x2e+256x2o")
 LARGE = ("256x0e+256x1o+256x2e", "1x0e+1x1o+1x2e+1x3o", "256x0e+256x1o+256x2e")
 DENSE = ("64x0e+64x1o+64x2e", "1x0e+1x1o+1x2e", "64x0e+64x1o+64x2e")
+# reference: benchmark/benchmark_configs.py:45-48 (the larger of its two per-row-weights problems)
+DIFFDOCK_L2 = ("10x1o+10x1e+48x0e+48x0o", "1x0e+1x1o+1x2e", "10x1o+10x1e+48x0e+48x0o")
 
 
 def _normal(rng, shape, dtype, scale=1.0, chunk=1 << 24):
@@ -84,9 +86,13 @@ class Workload:
     # probe graphs: receivers drawn from the first ``receiver_pool`` nodes only (0: from all), so that the dZ
     # rows the backward gathers fit a cache of a known size
     receiver_pool: int = 0
+    # uvw problems: one weight vector for the batch (True) or one per row (False)
+    shared: bool = True
 
     @property
     def data_note(self) -> str:
+        if self.device_inputs and self.kind == "tp":
+            return "synthetic (X, Y and dZ seeded on the host, the per-row weights drawn on the GPU)"
         return ("synthetic (graph and Y seeded on the host, X / W / dZ drawn on the GPU)" if self.device_inputs
                 else "synthetic")
 
@@ -108,7 +114,7 @@ class Workload:
     def problem(self) -> TPProblem:
         dt = np.float32 if self.dtype == "f32" else np.float64
         if self.mode == "uvw":
-            return FullyConnectedTPProblem(*self.irreps, shared_weights=True, internal_weights=False,
+            return FullyConnectedTPProblem(*self.irreps, shared_weights=self.shared, internal_weights=False,
                                            irrep_dtype=dt, weight_dtype=dt)
         if self.irreps == ("1x2e", "1x3e", "1x2e"):
             return TPProblem(*self.irreps, [(0, 0, 0, "uvu", True)], shared_weights=False, internal_weights=False)
@@ -149,7 +155,8 @@ class Workload:
             else:
                 h["Y"] = rng.uniform(size=(n, d2)).astype(dt)
             wshape = (wn,) if prob.shared_weights else (n, wn)
-            h["W"] = _normal(rng, wshape, dt, self.w_scale)
+            if not self.device_inputs:
+                h["W"] = _normal(rng, wshape, dt, self.w_scale)
             h["G"] = _normal(rng, (n, d3), dt)
         else:
             rows, cols, tperm = self.graph(rng)
@@ -170,7 +177,14 @@ class Workload:
         import torch
         prob, h = self.host_inputs()
         t = {k: torch.from_numpy(v).to(device) for k, v in h.items()}
-        if self.device_inputs:
+        if self.device_inputs and self.kind == "tp":
+            # per-row weights: the one large tensor is drawn on the GPU, the CPU baseline gets its first rows
+            gen = torch.Generator(device=device)
+            gen.manual_seed(self.seed)
+            t["W"] = torch.randn(h["X"].shape[0], prob.weight_numel, device=device, generator=gen,
+                                 dtype=torch.float32 if self.dtype == "f32" else torch.float64) * self.w_scale
+            h["W"] = t["W"][:8192].cpu().numpy()
+        elif self.device_inputs:
             gen = torch.Generator(device=device)
             gen.manual_seed(self.seed)
             tdt = torch.float32 if self.dtype == "f32" else torch.float64
@@ -333,9 +347,18 @@ def get(name: str) -> Workload:
         w.alg_flops = {"forward": dense * w.units, "backward": 2 * dense * w.units}
         w.alg_bytes = _tp_bytes(prob, w.units, 4 if dt == "f32" else 8)
         return w
+    if name in ("diffdock_uvw_f32", "diffdock_uvw_f64"):
+        dt = "f32" if name.endswith("f32") else "f64"
+        w = Workload(name, "uvw TP with a weight vector per row (DiffDock-L=2 of the reference's uvw benchmark), "
+                     "10x1o+10x1e+48x0e+48x0o (x) SH(lmax 2) -> 10x1o+10x1e+48x0e+48x0o, 12 instructions, 7128 weights "
+                     f"per row, batch 50000, {dt}, forward+backward", "tp", DIFFDOCK_L2, 50000, "rows/s", "hbm", dt,
+                     12351, {"batch": 50000, "paths": 12}, sh_lmax=2, mode="uvw", w_scale=0.2, shared=False,
+                     device_inputs=True)
+        w.alg_bytes = _tp_bytes(w.problem(), w.units, 4 if dt == "f32" else 8)
+        return w
     raise KeyError(f"unknown workload {name!r}")
 
 
 ALL = ("readme_uvu", "mace_uvu", "mace_uvu_all_parities", "nequip_conv_atomic", "nequip_conv_det", "nequip_conv_det_all_parities",
        "large_conv_det", "large_conv_atomic", "large_conv_det_all_parities", "mace_conv_det", "mace_conv_atomic",
-       "dense_uvw_f32", "dense_uvw_f64")
+       "dense_uvw_f32", "dense_uvw_f64", "diffdock_uvw_f32", "diffdock_uvw_f64")

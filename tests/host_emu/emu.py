@@ -24,6 +24,7 @@ CACHE = pathlib.Path(tempfile.gettempdir()) / "oeq_host_emu"
 
 EMU_PRELUDE = r"""
 #include <algorithm>
+#include <cassert>
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
@@ -77,6 +78,9 @@ static inline T oeq_wave_sum63(T v) { g_xT[threadIdx.x] = v; oeq_sync(); T t = 0
 template <int P> static inline T oeq_group_sum(T v) { g_xT[threadIdx.x] = v; oeq_sync(); T t = 0; for (int i = 0; i < P; ++i) t += g_xT[(threadIdx.x & ~(P - 1)) + i]; oeq_sync(); return t; }
 static inline T oeq_ldnt(const T* p) { return *p; }
 static inline void oeq_stnt(T* p, T v) { *p = v; }
+struct V2 { T v[2]; T& operator[](int i) { return v[i]; } const T& operator[](int i) const { return v[i]; } };
+static inline V2 oeq_ldnt2(const T* p) { assert((uintptr_t)p % (2 * sizeof(T)) == 0); V2 r; r[0] = p[0]; r[1] = p[1]; return r; }
+static inline void oeq_stnt2(T* p, V2 v) { assert((uintptr_t)p % (2 * sizeof(T)) == 0); p[0] = v[0]; p[1] = v[1]; }
 static inline void oeq_block_sync() { pthread_barrier_wait(&g_bar); }
 static inline void oeq_sched_fence() {}
 static inline void __syncthreads() { pthread_barrier_wait(&g_bar); }

@@ -372,9 +372,15 @@ def test_uvw_several_copies_of_the_second_operand(shared, monkeypatch):
     assert rel_err(ow.oeq_to_e3nn(oprob, out["Wg"]), dW) < TOL
 
 
-def test_uvw_per_row_weights():
+@pytest.mark.parametrize("a", [("5x0e+21x1o", "1x0e+1x1o+1x2e", "18x0e+7x1o+3x2e"),
+                               ("70x0e+35x1o", "1x0e+1x1o", "48x0e+33x1o"),
+                               ("10x0e+40x1o", "3x0e+2x1o", "36x0e+10x1o"),
+                               ("6x0e+20x1o", "1x0e+1x1o+1x2e", "18x0e+7x1o+4x2e")],
+                         ids=["narrow", "ragged_32_blocks", "several_copies", "even_and_odd_chunks"])
+@pytest.mark.parametrize("t_words", [4096, 150], ids=["one_phase", "several_phases"])
+def test_uvw_per_row_weights(a, t_words, monkeypatch):
     from openequivariance_amd.codegen.uvw_batched import UVWBatchedGenerator
-    a = ("5x0e+21x1o", "1x0e+1x1o+1x2e", "18x0e+7x1o+3x2e")
+    monkeypatch.setattr(UVWBatchedGenerator, "T_LDS_WORDS", t_words)
     prob, oprob = common.fully_connected(a, shared=False)
     g = UVWBatchedGenerator(prob)
     X, Y, We, G = common.tp_inputs(prob, 5, 10, w_scale=0.3)

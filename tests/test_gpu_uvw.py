@@ -230,3 +230,33 @@ def test_uvw_per_row_weights_wide(cuda):
     assert rel_err(x.grad.cpu().numpy(), dXr) <= FP32_TOL
     assert rel_err(y.grad.cpu().numpy(), dYr) <= FP32_TOL
     assert rel_err(ow.oeq_to_e3nn(oprob, w.grad.cpu().numpy()), dWr) <= FP32_TOL
+
+
+def test_uvw_per_row_weights_misaligned(cuda):
+    """fp32 per-row weights move two words per lane; tensors that start 4 bytes past an 8-byte boundary take the
+    kernels with one-word accesses (raw entry points, every tensor shifted)."""
+    import torch
+    import openequivariance_amd as oeq
+    prob, oprob = common.fully_connected(DIFFDOCK["DiffDock-L=1"], shared=False)
+    n = 41
+    X, Y, We, G = common.tp_inputs(prob, n, 47, w_scale=0.2)
+    W = ow.e3nn_to_oeq(oprob, We)
+    tp = oeq.TensorProduct(prob, torch_op=False)
+    assert tp.generator.pairs
+
+    def shifted(a):
+        flat = torch.empty(a.size + 1, dtype=torch.float32, device=cuda)
+        view = flat[1:].view(a.shape)
+        view.copy_(torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)))
+        assert view.data_ptr() % 8 == 4
+        return view
+    x, y, w, g = (shifted(a) for a in (X, Y, W, G))
+    z, xg, yg, wg = (shifted(np.zeros_like(a)) for a in (G, X, Y, W))
+    tp.forward_raw(n, x.data_ptr(), y.data_ptr(), z.data_ptr(), w.data_ptr())
+    tp.backward_raw(n, x.data_ptr(), xg.data_ptr(), y.data_ptr(), yg.data_ptr(), w.data_ptr(), wg.data_ptr(), g.data_ptr())
+    torch.cuda.synchronize()
+    dXr, dYr, dWr = otp.backward(oprob, X, Y, We, G)
+    assert rel_err(z.cpu().numpy(), otp.forward(oprob, X, Y, We)) <= FP32_TOL
+    assert rel_err(xg.cpu().numpy(), dXr) <= FP32_TOL
+    assert rel_err(yg.cpu().numpy(), dYr) <= FP32_TOL
+    assert rel_err(ow.oeq_to_e3nn(oprob, wg.cpu().numpy()), dWr) <= FP32_TOL
