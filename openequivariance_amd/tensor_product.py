@@ -57,13 +57,16 @@ def _on_device(device):
 
 
 def select_generator(config: TPProblem):
-    """The kernel generator of a batch tensor product: MFMA kernels for uvw with shared weights,
+    """The kernel generator of a batch tensor product: MFMA kernels for uvw with shared weights (vector-ALU
+    kernels with a row per lane when the weights are few and the multiplicities small),
     streaming vector-ALU kernels for uvw with per-row weights, the persistent two-stage dW
     reduction for uvu with shared weights, register-direct streaming kernels otherwise."""
     mode = validate_problem(config)
     if mode == "uvw" and config.shared_weights:
         from .codegen.uvw import UVWGenerator
-        return UVWGenerator(config)
+        from .codegen.uvw_rows import UVWRowsGenerator
+        # a few hundred weights on multiplicities far below a 16 x 16 tile: one row per lane on the vector ALU
+        return UVWRowsGenerator(config) if UVWRowsGenerator.suits(config) else UVWGenerator(config)
     if mode == "uvw":
         from .codegen.uvw_batched import UVWBatchedGenerator
         return UVWBatchedGenerator(config)

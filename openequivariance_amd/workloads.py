@@ -29,6 +29,9 @@ LARGE_ALL = ("256x0e+256x1o+256x2e", "1x0e+1x1o+1x2e+1x3o", "256x0e+256x1o+256x1
 LARGE = ("256x0e+256x1o+256x2e", "1x0e+1x1o+1x2e+1x3o", "256x0e+256x1o+256x2e")
 DENSE = ("64x0e+64x1o+64x2e", "1x0e+1x1o+1x2e", "64x0e+64x1o+64x2e")
 # reference: benchmark/benchmark_configs.py:45-48 (the larger of its two per-row-weights problems)
+# reference: benchmark/benchmark_configs.py:38-41 (the other two problems of its uvw benchmark; shared weights)
+TETRIS_POLY = {"1": ("1x0e+1x1o+1x2e+1x3o", "1x0e+1x1o+1x2e+1x3o", "64x0e+24x1e+24x1o+16x2e+16x2o"),
+               "2": ("64x0e+24x1e+24x1o+16x2e+16x2o", "1x0e+1x1o+1x2e+1x3o", "1x0o+6x0e")}
 DIFFDOCK_L2 = ("10x1o+10x1e+48x0e+48x0o", "1x0e+1x1o+1x2e", "10x1o+10x1e+48x0e+48x0o")
 
 
@@ -356,9 +359,19 @@ def get(name: str) -> Workload:
                      device_inputs=True)
         w.alg_bytes = _tp_bytes(w.problem(), w.units, 4 if dt == "f32" else 8)
         return w
+    if name.startswith("tetris_poly") and name[11:] in ("1_uvw_f32", "1_uvw_f64", "2_uvw_f32", "2_uvw_f64"):
+        which, dt = name[11], name[-3:]
+        irreps = TETRIS_POLY[which]
+        w = Workload(name, f"uvw TP with shared weights, tetris-poly-{which} of the reference's uvw benchmark, "
+                     f"{irreps[0]} (x) SH(lmax 3) -> {irreps[2]}, batch 50000, {dt}, forward+backward", "tp", irreps,
+                     50000, "rows/s", "hbm", dt, 12352, {"batch": 50000}, sh_lmax=3, mode="uvw", w_scale=0.2)
+        w.config["paths"] = len(w.problem().instructions)
+        w.alg_bytes = _tp_bytes(w.problem(), w.units, 4 if dt == "f32" else 8)
+        return w
     raise KeyError(f"unknown workload {name!r}")
 
 
 ALL = ("readme_uvu", "mace_uvu", "mace_uvu_all_parities", "nequip_conv_atomic", "nequip_conv_det", "nequip_conv_det_all_parities",
        "large_conv_det", "large_conv_atomic", "large_conv_det_all_parities", "mace_conv_det", "mace_conv_atomic",
-       "dense_uvw_f32", "dense_uvw_f64", "diffdock_uvw_f32", "diffdock_uvw_f64")
+       "dense_uvw_f32", "dense_uvw_f64", "diffdock_uvw_f32", "diffdock_uvw_f64",
+       "tetris_poly1_uvw_f32", "tetris_poly1_uvw_f64", "tetris_poly2_uvw_f32", "tetris_poly2_uvw_f64")

@@ -64,6 +64,7 @@ static inline int oeq_shfl_xor_i32(int v, int mask) { g_xi[threadIdx.x] = v; oeq
 #define __builtin_amdgcn_readfirstlane(x) oeq_shfl_i32((x), 0)
 static inline u64 oeq_uniform_u64(u64 v) { return v; }
 struct VT { T v[16 / sizeof(T)]; T& operator[](int i) { return v[i]; } const T& operator[](int i) const { return v[i]; } };
+typedef VT VTU;
 #define OEQ_DMA(BYTES, POLICY, g, lds_base) memcpy((char*)(lds_base) + ((BYTES) == 12 ? 16 : (BYTES)) * (threadIdx.x & 63), (g), (BYTES))
 static inline void oeq_release_agent() {}
 static inline void oeq_acquire_agent() {}
@@ -75,6 +76,7 @@ static inline int oeq_lds_add(int* p, int v) { std::lock_guard<std::mutex> g(g_a
 static inline void oeq_wait_vm() {}
 static inline void oeq_wait_lds() {}
 static inline T oeq_wave_sum63(T v) { g_xT[threadIdx.x] = v; oeq_sync(); T t = 0; for (int i = 0; i < 64; ++i) t += g_xT[(threadIdx.x & ~63) + i]; oeq_sync(); return t; }
+static inline T oeq_lane_value(T v, int l) { g_xT[threadIdx.x] = v; oeq_sync(); const T r = g_xT[(threadIdx.x & ~63) + l]; oeq_sync(); return r; }
 template <int P> static inline T oeq_group_sum(T v) { g_xT[threadIdx.x] = v; oeq_sync(); T t = 0; for (int i = 0; i < P; ++i) t += g_xT[(threadIdx.x & ~(P - 1)) + i]; oeq_sync(); return t; }
 static inline T oeq_ldnt(const T* p) { return *p; }
 static inline void oeq_stnt(T* p, T v) { *p = v; }
@@ -166,6 +168,12 @@ TP_EXTRA_UVW = r"""
         else if (k == "prep_forward") emu_run(gx, gy, threads, [&] { prep_forward(n, (const T*)X.data(), (const T*)Y.data(), (T*)Z.data(), (const T*)W.data(), ws.data()); });
 #define UVW_BWD(fn) emu_run(gx, gy, threads, [&] { fn(n, (const T*)X.data(), (T*)Xg.data(), (const T*)Y.data(), (T*)Yg.data(), (const T*)W.data(), (T*)Wg.data(), (const T*)G.data(), ws.data()); })
         else if (k == "prep_backward") UVW_BWD(prep_backward);
+        else if (k == "backward_dw") UVW_BWD(backward_dw);
+        else if (k == "backward_reduce") UVW_BWD(backward_reduce);
+"""
+
+TP_EXTRA_UVW_ROWS = r"""
+#define UVW_BWD(fn) emu_run(gx, gy, threads, [&] { fn(n, (const T*)X.data(), (T*)Xg.data(), (const T*)Y.data(), (T*)Yg.data(), (const T*)W.data(), (T*)Wg.data(), (const T*)G.data(), ws.data()); })
         else if (k == "backward_dw") UVW_BWD(backward_dw);
         else if (k == "backward_reduce") UVW_BWD(backward_reduce);
 """
@@ -283,7 +291,7 @@ def _run(exe: pathlib.Path, workdir: str) -> None:
 def run_tp(gen, steps: Sequence[Dict], X, Y, W, G=None, ws_bytes: int = 0):
     """Run TP steps; returns dict of outputs (Z or dX, dY, dW)."""
     dt = np.float32 if gen.T == "float" else np.float64
-    extra = TP_EXTRA_UVW if gen.kind == "uvw" else (TP_EXTRA_SHARED if gen.shared else "")
+    extra = TP_EXTRA_UVW if gen.kind == "uvw" else TP_EXTRA_UVW_ROWS if gen.kind == "uvw_rows" else (TP_EXTRA_SHARED if gen.shared else "")
     main = TP_MAIN.replace("@EXTRA@", extra)
     exe = build(gen.render(prelude=emu_prelude(gen.T)), main)
     n = X.shape[0]

@@ -392,3 +392,27 @@ def test_uvw_per_row_weights(a, t_words, monkeypatch):
     dX, dY, dW = otp.backward(oprob, X, Y, We, G)
     assert rel_err(out["Xg"], dX) < TOL and rel_err(out["Yg"], dY) < TOL
     assert rel_err(ow.oeq_to_e3nn(oprob, out["Wg"]), dW) < TOL
+
+
+@pytest.mark.parametrize("a,n", [(("1x0e+1x1o+1x2e+1x3o", "1x0e+1x1o+1x2e+1x3o", "64x0e+24x1e+24x1o+16x2e+16x2o"), 70),
+                                 (("64x0e+24x1e+24x1o+16x2e+16x2o", "1x0e+1x1o+1x2e+1x3o", "1x0o+6x0e"), 130),
+                                 (("3x0e+2x1o", "2x0e+1x1o", "5x0e+4x1o+1x2e"), 64),
+                                 (("8x0e+10x1o", "1x0e+1x1o", "9x0e+11x1o"), 97)],
+                         ids=["tetris_poly_1", "tetris_poly_2", "several_copies", "several_groups_on_both_sides"])
+def test_uvw_shared_weights_one_row_per_lane(a, n, monkeypatch):
+    """The vector-ALU kernels for uvw problems with few weights: ragged last tile, several tiles per wavefront
+    (the grid bound is lowered to 2 so that a wavefront accumulates dW over more than one tile)."""
+    from openequivariance_amd.codegen.uvw_rows import UVWRowsGenerator
+    monkeypatch.setattr(UVWRowsGenerator, "WAVES", 2)
+    prob, oprob = common.fully_connected(a, shared=True)
+    assert UVWRowsGenerator.suits(prob)
+    g = UVWRowsGenerator(prob)
+    X, Y, We, G = common.tp_inputs(prob, n, 11, w_scale=0.3)
+    W = ow.e3nn_to_oeq(oprob, We)
+    fwd, bwd, ws = g.plan()
+    out = emu.run_tp(g, fwd, X, Y, W, ws_bytes=ws())
+    assert rel_err(out["Z"], otp.forward(oprob, X, Y, We)) < TOL
+    out = emu.run_tp(g, bwd, X, Y, W, G, ws_bytes=ws())
+    dX, dY, dW = otp.backward(oprob, X, Y, We, G)
+    assert rel_err(out["Xg"], dX) < TOL and rel_err(out["Yg"], dY) < TOL
+    assert rel_err(ow.oeq_to_e3nn(oprob, out["Wg"]), dW) < TOL

@@ -260,3 +260,41 @@ def test_uvw_per_row_weights_misaligned(cuda):
     assert rel_err(xg.cpu().numpy(), dXr) <= FP32_TOL
     assert rel_err(yg.cpu().numpy(), dYr) <= FP32_TOL
     assert rel_err(ow.oeq_to_e3nn(oprob, wg.cpu().numpy()), dWr) <= FP32_TOL
+
+
+TETRIS_POLY = {"tetris-poly-1": ("1x0e+1x1o+1x2e+1x3o", "1x0e+1x1o+1x2e+1x3o", "64x0e+24x1e+24x1o+16x2e+16x2o"),
+               "tetris-poly-2": ("64x0e+24x1e+24x1o+16x2e+16x2o", "1x0e+1x1o+1x2e+1x3o", "1x0o+6x0e"),
+               # rows longer than a register group on both sides, a last group that is no whole number of vectors,
+               # two copies of the second operand
+               "several-groups": ("8x0e+10x1o", "2x0e+1x1o", "9x0e+11x1o")}
+
+
+@pytest.mark.parametrize("name", list(TETRIS_POLY))
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("waves", [1024, 3], ids=["one_tile_per_wavefront", "several_tiles_per_wavefront"])
+def test_uvw_few_weights_one_row_per_lane(cuda, name, dtype, waves, monkeypatch):
+    """The two shared-weight problems of the reference's uvw benchmark (benchmark/benchmark_configs.py:38-41): few
+    weights on multiplicities of 1 or 6, served by the vector-ALU kernels with a row per lane.  517 rows = 8 full
+    tiles and a ragged one; with 3 wavefronts each accumulates dW over three tiles."""
+    import torch
+    import openequivariance_amd as oeq
+    from openequivariance_amd.codegen.uvw_rows import UVWRowsGenerator
+    monkeypatch.setattr(UVWRowsGenerator, "WAVES", waves)
+    tol = FP32_TOL if dtype == np.float32 else FP64_TOL
+    prob, oprob = common.fully_connected(TETRIS_POLY[name], shared=True, dtype=dtype)
+    X, Y, We, G = common.tp_inputs(prob, 517, 48, dtype, w_scale=0.2)
+    tp = oeq.TensorProduct(prob, torch_op=True)
+    assert isinstance(tp.generator, UVWRowsGenerator)
+    W = ow.e3nn_to_oeq(oprob, We)
+    x, y, w = (torch.tensor(a, device=cuda, requires_grad=True) for a in (X, Y, W))
+    z = tp(x, y, w)
+    z.backward(torch.tensor(G, device=cuda))
+    dXr, dYr, dWr = otp.backward(oprob, X, Y, We, G)
+    assert rel_err(z.detach().cpu().numpy(), otp.forward(oprob, X, Y, We)) <= tol
+    assert rel_err(x.grad.cpu().numpy(), dXr) <= tol
+    assert rel_err(y.grad.cpu().numpy(), dYr) <= tol
+    assert rel_err(ow.oeq_to_e3nn(oprob, w.grad.cpu().numpy()), dWr) <= tol
+    # the sums over the batch run in a fixed order: a second backward repeats bit for bit
+    x2, y2, w2 = (t.detach().clone().requires_grad_(True) for t in (x, y, w))
+    tp(x2, y2, w2).backward(torch.tensor(G, device=cuda))
+    assert torch.equal(w2.grad, w.grad)
