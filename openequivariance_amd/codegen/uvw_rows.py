@@ -33,6 +33,8 @@ writing Z as records or as whole-row runs through the LDS slot is a tie in fp32 
 """
 from __future__ import annotations
 
+import numpy as np
+
 from ..problem import TPProblem
 from .common import Emitter, jinja_env
 from .uvw import UVWGenerator, _ceil
@@ -41,7 +43,8 @@ from .uvw import UVWGenerator, _ceil
 class UVWRowsGenerator(UVWGenerator):
     CHUNK_WORDS = 32      # words of a row's record held in registers at a time (per operand)
     WAVES = 2048          # upper bound of the dW kernel's persistent wavefronts = partial dW rows
-    MAX_WEIGHTS = 2048    # the contraction is unrolled: weights x (2 l3 + 1) vector FMAs
+    MAX_WEIGHTS = 2048    # the contraction is unrolled: weights x (2 l3 + 1) vector FMAs ...
+    MAX_FMAS = 6000       # ... which have to stay well within the 64 KB instruction cache
 
     @classmethod
     def suits(cls, problem: TPProblem) -> bool:
@@ -49,12 +52,19 @@ class UVWRowsGenerator(UVWGenerator):
         weight matrices fill less than half of the 16 x 16 tiles that cover them."""
         if not problem.shared_weights or problem.weight_numel > cls.MAX_WEIGHTS:
             return False
-        real = padded = 0
+        real = padded = nt = fmas = 0
         for ins in problem.instructions:
             mu, mw = problem.irreps_in1[ins.i_in1].mul, problem.irreps_out[ins.i_out].mul
+            mv, d3 = problem.irreps_in2[ins.i_in2].mul, problem.irreps_out[ins.i_out].ir.dim
             real += mu * mw
             padded += 16 * _ceil(mu, 16) * 16 * _ceil(mw, 16)
-        return 2 * real < padded
+            nt += mu * mv * d3
+            fmas += mu * mv * mw * d3
+        if fmas > cls.MAX_FMAS:
+            return False
+        # the dW kernel keeps T of a tile's rows in LDS: at least 8 rows of it must fit its share
+        itemsize = 4 if problem.irrep_dtype == np.float32 else 8
+        return 2 * real < padded and 8 * (nt | 1) * itemsize <= cls.DW_T_BYTES
 
     def __init__(self, problem: TPProblem):
         super().__init__(problem)
@@ -64,6 +74,13 @@ class UVWRowsGenerator(UVWGenerator):
             raise ValueError(f"UVWRowsGenerator unrolls the contraction: at most {self.MAX_WEIGHTS} weights")
         self.kind = "uvw_rows"
         self.WNP = 64 * _ceil(self.WN, 64)
+        # rows of a dW tile: as many (up to DW_ROWS) as keep T of the tile within its share of the LDS
+        _, nt = self.t_offsets()
+        self.dw_rows = self.DW_ROWS
+        while self.dw_rows > 8 and self.dw_rows * (nt | 1) * self.itemsize > self.DW_T_BYTES:
+            self.dw_rows //= 2
+        if self.dw_rows * (nt | 1) * self.itemsize > self.DW_T_BYTES:
+            raise ValueError("UVWRowsGenerator: T of 8 rows does not fit the LDS share of the dW kernel")
         self.ws_elems = self.WAVES * self.npos
 
     def describe(self) -> str:
@@ -354,21 +371,22 @@ class UVWRowsGenerator(UVWGenerator):
         that keeps the workgroup within DW_LDS_BYTES so that four fit a compute unit."""
         _, nt = self.t_offsets()
         ts, gs = nt | 1, self.D3 | 1
-        rb = self.DW_ROWS
-        while rb > 1 and (self.DW_ROWS * ts + rb * gs) * self.itemsize > self.DW_LDS_BYTES:
+        rb = self.dw_rows
+        while rb > 1 and (self.dw_rows * ts + rb * gs) * self.itemsize > self.DW_LDS_BYTES:
             rb //= 2
         return ts, gs, rb
 
     DW_LDS_BYTES = 24 * 1024
     DW_UNROLL = 2         # rows of the dW loop whose LDS reads are in flight together
-    DW_ROWS = 32          # rows of a dW tile
+    DW_ROWS = 32          # rows of a dW tile (fewer when T of so many rows would not fit DW_T_BYTES)
+    DW_T_BYTES = 16 * 1024
 
     def backward_dw_body(self) -> str:
         E = Emitter()
         ts, gs, rb = self.dw_lds()
         toff, nt = self.t_offsets()
         regs = self.dw_positions()
-        R_ = self.DW_ROWS
+        R_ = self.dw_rows
         E("const int lane = threadIdx.x;")
         E(f"__shared__ T Tl[{R_ * ts}];")
         E(f"__shared__ T Gl[{rb * gs}];")
@@ -449,7 +467,7 @@ class UVWRowsGenerator(UVWGenerator):
         E = Emitter()
         E("const int l = threadIdx.x & 15, sub = threadIdx.x >> 4, pos = blockIdx.x * 16 + l;")
         E("__shared__ T sums[1024];")
-        E(f"const u64 tiles = (n + {self.DW_ROWS - 1}) / {self.DW_ROWS};")
+        E(f"const u64 tiles = (n + {self.dw_rows - 1}) / {self.dw_rows};")
         E(f"const u64 rows = tiles < {self.WAVES} ? tiles : {self.WAVES};")
         E("const T* __restrict__ part = (const T*)ws;")
         E("T s = (T)0;")
@@ -475,6 +493,6 @@ class UVWRowsGenerator(UVWGenerator):
         FIXED, ROW = 0, 1
         fwd = [dict(kernel="forward", num_threads=64, grid_kind=ROW, work_per_block=64)]
         bwd = [dict(kernel="backward", num_threads=64, grid_kind=ROW, work_per_block=64),
-               dict(kernel="backward_dw", num_threads=64, grid_kind=ROW, work_per_block=self.DW_ROWS, num_blocks=self.WAVES),
+               dict(kernel="backward_dw", num_threads=64, grid_kind=ROW, work_per_block=self.dw_rows, num_blocks=self.WAVES),
                dict(kernel="backward_reduce", num_threads=1024, grid_kind=FIXED, num_blocks=self.npos // 16)]
         return fwd, bwd, (lambda nnz=0, nodes=0: self.ws_elems * self.itemsize)

@@ -144,3 +144,39 @@ def test_random_second_operand_multiplicities(cuda, seed):
     dW = ow.oeq_to_e3nn(oprob, w.grad.cpu().numpy())
     for got, ref in zip((x.grad.cpu().numpy(), y.grad.cpu().numpy(), dW), otp.backward(oprob, X, Y, We, G)):
         assert rel_err(got, ref) <= tol
+
+
+@pytest.mark.parametrize("seed", range(6000, 6012))
+def test_random_uvw_with_few_shared_weights(cuda, seed):
+    """Fully connected problems with small, ragged multiplicities and shared weights: most draws are served by the
+    vector-ALU kernels with a row per lane (one to several register groups per row on either side, one to four
+    copies of the second operand, batches from one row to several tiles per wavefront), the rest by the MFMA kernels."""
+    import torch
+    import openequivariance_amd as oeq
+    rng = np.random.default_rng(seed)
+    dtype = np.float64 if rng.random() < 0.25 else np.float32
+    tol = FP32_TOL if dtype == np.float32 else FP64_TOL
+    n = int(rng.choice([1, 31, 64, 65, 200, 700]))
+    mul = lambda: int(rng.choice([1, 2, 3, 5, 6, 7, 10, 24]))
+    while True:
+        l1 = sorted(rng.choice(4, size=rng.integers(1, 4), replace=False))
+        irreps = ("+".join(f"{mul()}x{l}{_par(l)}" for l in l1),
+                  "+".join(f"{int(rng.choice([1, 1, 2, 4]))}x{l}{_par(l)}" for l in range(int(rng.integers(0, 3)) + 1)),
+                  "+".join(f"{mul()}x{l}{p}" for l in range(int(rng.integers(0, 4)) + 1) for p in "eo"
+                           if p == _par(l) or rng.random() < 0.3))
+        prob, oprob = common.fully_connected(irreps, shared=True, dtype=dtype)
+        if prob.instructions:
+            break
+    tp = oeq.TensorProduct(prob, torch_op=True)
+    print(f"seed={seed} {dtype.__name__} {irreps} paths={len(prob.instructions)} wn={prob.weight_numel} n={n} "
+          f"{type(tp.generator).__name__}", flush=True)
+    X, Y, We, G = common.tp_inputs(prob, n, seed, dtype, w_scale=0.3)
+    W = ow.e3nn_to_oeq(oprob, We)
+    x, y, w = (torch.tensor(a, device=cuda, requires_grad=True) for a in (X, Y, W))
+    z = tp(x, y, w)
+    z.backward(torch.tensor(G, device=cuda))
+    torch.cuda.synchronize()
+    assert rel_err(z.detach().cpu().numpy(), otp.forward(oprob, X, Y, We)) <= tol
+    dW = ow.oeq_to_e3nn(oprob, w.grad.cpu().numpy())
+    for got, ref in zip((x.grad.cpu().numpy(), y.grad.cpu().numpy(), dW), otp.backward(oprob, X, Y, We, G)):
+        assert rel_err(got, ref) <= tol
