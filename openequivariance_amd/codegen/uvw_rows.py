@@ -28,10 +28,13 @@ at compile-time offsets are hoisted and spilled by the compiler (a lane read per
 job in one instruction); a conditional store in the middle of the unrolled code makes the compiler
 move the arithmetic of everything stored later past it, with all its operands alive until then (512
 registers and scratch): every store is unconditional, lanes past the batch repeat the last row;
-writing Z as records or as whole-row runs through the LDS slot is a tie in fp32 (35 / 32 us) and
-65 / 36 us in fp64.
+Z written as a lane's own records (16 bytes of 64 different cache lines per instruction) takes 30 us for
+74 MB whatever the arithmetic beside it, as whole-row runs through the LDS slot 17 us for the whole
+kernel - provided the groups are cut so that all of them are whole numbers of vectors.
 """
 from __future__ import annotations
+
+import math
 
 import numpy as np
 
@@ -89,24 +92,47 @@ class UVWRowsGenerator(UVWGenerator):
 
     # ------------------------------------------------------------------ pieces
     def groups(self, blocks):
-        """A row cut into runs of whole channel records, across block boundaries, of at most CHUNK_WORDS words
-        each: a list of groups, a group a list of (block, first channel, end channel).  A group is contiguous
-        in memory."""
-        out, cur, words = [], [], 0
+        """A row cut into runs of whole channel records of at most CHUNK_WORDS words each: a list of groups, a
+        group a list of (block, first channel, end channel), contiguous in memory.  A block's records are
+        taken four (fp64: two) at a time as far as its multiplicity allows, so that the group is a whole number
+        of 16-byte vectors and can leave through the LDS slot as whole-row runs; the records that are left
+        over (fewer than four) form groups of their own, together with the left-overs of the next blocks."""
+        vw = 16 // self.itemsize
+        if sum(blk.dim for blk in blocks) <= self.CHUNK_WORDS:          # a short row is one group
+            return [[(blk, 0, blk.mul) for blk in blocks if blk.dim]]
+        out, cur, words, tails = [], [], 0, False
+
+        def close():
+            nonlocal cur, words, tails
+            if cur:
+                out.append(cur)
+            cur, words, tails = [], 0, False
+
+        def add(blk, lo, hi, tail):
+            nonlocal words, tails
+            cur.append((blk, lo, hi))
+            words += (hi - lo) * blk.D
+            tails = tails or tail
         for blk in blocks:
-            lo = 0
-            while blk.dim and lo < blk.mul:
-                room = (self.CHUNK_WORDS - words) // blk.D
+            if not blk.dim:
+                continue
+            step = vw // math.gcd(vw, blk.D)           # records per whole number of vectors
+            full, pos = blk.mul // step * step, 0
+            while pos < full:
+                if tails:
+                    close()
+                room = (self.CHUNK_WORDS - words) // (blk.D * step) * step
                 if room == 0 and cur:
-                    out.append(cur)
-                    cur, words = [], 0
+                    close()
                     continue
-                hi = min(blk.mul, lo + max(1, room))
-                cur.append((blk, lo, hi))
-                words += (hi - lo) * blk.D
-                lo = hi
-        if cur:
-            out.append(cur)
+                take = min(full - pos, max(room, step))
+                add(blk, pos, pos + take, False)
+                pos += take
+            if pos < blk.mul:
+                if cur and (not tails or words + (blk.mul - pos) * blk.D > self.CHUNK_WORDS):
+                    close()
+                add(blk, pos, blk.mul, True)
+        close()
         return out
 
     @staticmethod
