@@ -403,7 +403,7 @@ class UVWRowsGenerator(UVWGenerator):
         return ts, gs, rb
 
     DW_LDS_BYTES = 24 * 1024
-    DW_UNROLL = 2         # rows of the dW loop whose LDS reads are in flight together
+    DW_UNROLL = 0         # rows of the dW loop unrolled together (0: by type, see backward_dw_body)
     DW_ROWS = 32          # rows of a dW tile (fewer when T of so many rows would not fit DW_T_BYTES)
     DW_T_BYTES = 16 * 1024
 
@@ -422,8 +422,23 @@ class UVWRowsGenerator(UVWGenerator):
         E(f"const u64 tiles = (n + {R_ - 1}) / {R_};")
         E("for (u64 tile = blockIdx.x; tile < tiles; tile += gridDim.x) {")
         E.level += 1
-        # T of this lane's row (zero past the batch, which also voids whatever dZ holds there)
+        E(f"const u64 row0 = tile * {R_};")
         self.emit_tile(E, "tile", zero_y=True, rows=R_)
+        # dZ: rb rows at a time, contiguous in memory; the next batch travels to registers while this one is used
+        nit = _ceil(rb * self.D3, 64)
+        dest = "i_" if gs == self.D3 else f"i_ + i_ / {self.D3}"
+        E(f"T R[{nit}];")
+        E("int limit;                     // words of the requested batch that lie within the tensor")
+
+        def request(r0: str):
+            E(f"{{ const T* __restrict__ gp = G + (row0 + {r0}) * {self.D3};")
+            E(f"  const u64 left = n - (row0 + {r0});")
+            E(f"  limit = (int)(left < {rb} ? left : {rb}) * {self.D3};")
+            E("#pragma unroll")
+            E(f"  for (int i = 0; i < {nit}; ++i) R[i] = gp[min(64 * i + lane, limit - 1)];")
+            E("}")
+        request("0")
+        # T of this lane's row (zero past the batch, which also voids whatever dZ holds there)
         E(f"const T* __restrict__ Xr = X + row * {self.D1};")
         E("oeq_sync();")
         xgs = self.groups(self.in1)
@@ -445,21 +460,6 @@ class UVWRowsGenerator(UVWGenerator):
                         E("}")
             E.level -= 1
             E("}")
-        # dZ: rb rows at a time, contiguous in memory; the next batch travels to registers while this one is used
-        nit = _ceil(rb * self.D3, 64)
-        dest = "i_" if gs == self.D3 else f"i_ + i_ / {self.D3}"
-        E(f"const u64 row0 = tile * {R_};")
-        E(f"T R[{nit}];")
-        E("int limit;                     // words of the requested batch that lie within the tensor")
-
-        def request(r0: str):
-            E(f"{{ const T* __restrict__ gp = G + (row0 + {r0}) * {self.D3};")
-            E(f"  const u64 left = n - (row0 + {r0});")
-            E(f"  limit = (int)(left < {rb} ? left : {rb}) * {self.D3};")
-            E("#pragma unroll")
-            E(f"  for (int i = 0; i < {nit}; ++i) R[i] = gp[min(64 * i + lane, limit - 1)];")
-            E("}")
-        request("0")
         E(f"for (int r0 = 0; r0 < {R_} && row0 + r0 < n; r0 += {rb}) {{")
         E.level += 1
         E("oeq_sync();")
@@ -471,7 +471,9 @@ class UVWRowsGenerator(UVWGenerator):
         request(f"r0 + {rb}")
         E.level -= 1
         E("}")
-        E(f"#pragma unroll {self.DW_UNROLL}")
+        # fp32: the whole batch unrolled, so that a row is an immediate offset of the LDS reads (35 -> 28 us on the
+        # first tetris layer); fp64 has no registers for that (56 -> 82 us)
+        E(f"#pragma unroll {self.DW_UNROLL or (rb if self.T == 'float' else 2)}")
         E(f"for (int r = 0; r < {rb}; ++r) {{")
         E(f"    const T* __restrict__ tr = Tl + (r0 + r) * {ts};")
         E(f"    const T* __restrict__ gr_ = Gl + r * {gs};")
