@@ -298,3 +298,26 @@ def test_uvw_few_weights_one_row_per_lane(cuda, name, dtype, waves, monkeypatch)
     x2, y2, w2 = (t.detach().clone().requires_grad_(True) for t in (x, y, w))
     tp(x2, y2, w2).backward(torch.tensor(G, device=cuda))
     assert torch.equal(w2.grad, w.grad)
+
+
+@pytest.mark.parametrize("name", ["DiffDock-L=1", "tetris-poly-1", "dense"])
+def test_uvw_empty_batch(cuda, name):
+    """No rows: an empty output, empty dX and dY, and - for shared weights - a dW of zeros, from all three uvw
+    kernel families (per-row weights, few shared weights, MFMA)."""
+    import torch
+    import openequivariance_amd as oeq
+    shared = name != "DiffDock-L=1"
+    irreps = {"DiffDock-L=1": DIFFDOCK["DiffDock-L=1"], "tetris-poly-1": TETRIS_POLY["tetris-poly-1"],
+              "dense": ("16x0e+16x1o", "1x0e+1x1o", "16x0e+16x1o")}[name]
+    prob, _ = common.fully_connected(irreps, shared=shared)
+    tp = oeq.TensorProduct(prob, torch_op=True)
+    d1, d2, d3, wn = prob.irreps_in1.dim, prob.irreps_in2.dim, prob.irreps_out.dim, prob.weight_numel
+    x = torch.zeros(0, d1, device=cuda, requires_grad=True)
+    y = torch.zeros(0, d2, device=cuda, requires_grad=True)
+    w = (torch.randn(wn, device=cuda) if shared else torch.zeros(0, wn, device=cuda)).requires_grad_(True)
+    z = tp(x, y, w)
+    assert z.shape == (0, d3)
+    z.backward(torch.zeros(0, d3, device=cuda))
+    torch.cuda.synchronize()
+    assert x.grad.shape == (0, d1) and y.grad.shape == (0, d2)
+    assert w.grad.shape == w.shape and not w.grad.abs().any()
