@@ -121,7 +121,7 @@ class UVWRowsGenerator(UVWGenerator):
             while pos < full:
                 if tails:
                     close()
-                room = (self.CHUNK_WORDS - words) // (blk.D * step) * step
+                room = max(0, self.CHUNK_WORDS - words) // (blk.D * step) * step
                 if room == 0 and cur:
                     close()
                     continue
@@ -211,7 +211,8 @@ class UVWRowsGenerator(UVWGenerator):
     def slot_words(self) -> int:
         """LDS words of the slot that turns a wavefront's records (one row per lane) into whole-row runs."""
         vw = 16 // self.itemsize
-        return 64 * (self.CHUNK_WORDS + vw)
+        longest = max(self.span(g)[1] for blocks in (self.in1, self.out) for g in self.groups(blocks))
+        return 64 * (max(self.CHUNK_WORDS, longest) + vw)      # (four records of l >= 4 exceed CHUNK_WORDS)
 
     def emit_group_store(self, E: Emitter, name: str, ptr: str, group, rowdim: int) -> None:
         """The group's words of all 64 rows -> memory.  A lane's own record store touches 16 bytes of 64

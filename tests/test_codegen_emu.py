@@ -397,8 +397,10 @@ def test_uvw_per_row_weights(a, t_words, monkeypatch):
 @pytest.mark.parametrize("a,n", [(("1x0e+1x1o+1x2e+1x3o", "1x0e+1x1o+1x2e+1x3o", "64x0e+24x1e+24x1o+16x2e+16x2o"), 70),
                                  (("64x0e+24x1e+24x1o+16x2e+16x2o", "1x0e+1x1o+1x2e+1x3o", "1x0o+6x0e"), 130),
                                  (("3x0e+2x1o", "2x0e+1x1o", "5x0e+4x1o+1x2e"), 64),
-                                 (("8x0e+10x1o", "1x0e+1x1o", "9x0e+11x1o"), 97)],
-                         ids=["tetris_poly_1", "tetris_poly_2", "several_copies", "several_groups_on_both_sides"])
+                                 (("8x0e+10x1o", "1x0e+1x1o", "9x0e+11x1o"), 97),
+                                 (("2x0e+9x4e", "1x0e+1x2e", "8x4e+3x2e"), 70)],
+                         ids=["tetris_poly_1", "tetris_poly_2", "several_copies", "several_groups_on_both_sides",
+                              "four_records_longer_than_a_group"])
 def test_uvw_shared_weights_one_row_per_lane(a, n, monkeypatch):
     """The vector-ALU kernels for uvw problems with few weights: ragged last tile, several tiles per wavefront
     (the grid bound is lowered to 2 so that a wavefront accumulates dW over more than one tile)."""
