@@ -1,6 +1,6 @@
 """Ahead-of-time hipRTC compilation of the benchmark configurations' kernels.
 
-hipRTC cross-compiles for gfx950 without a GPU, so the code objects of the five benchmark
+hipRTC cross-compiles for gfx950 without a GPU, so the code objects of the benchmark
 problems can be produced where the package is built and picked up from the in-tree cache on the
 GPU machine.  Problems outside this list are compiled on first construction as usual.
 """
@@ -14,7 +14,7 @@ from . import runtime as rt
 from .conv import select_conv_generator
 from .problem import ChannelwiseTPP, FullyConnectedTPProblem, TPProblem
 from .tensor_product import select_generator
-from .workloads import DENSE, LARGE, MACE, MACE_ALL, NEQUIP
+from .workloads import DENSE, DIFFDOCK_L2, LARGE, MACE, MACE_ALL, NEQUIP, TETRIS_POLY
 
 
 def benchmark_generators():
@@ -31,6 +31,11 @@ def benchmark_generators():
     for dt in (np.float32, np.float64):
         p = FullyConnectedTPProblem(*DENSE, shared_weights=True, internal_weights=False, irrep_dtype=dt, weight_dtype=dt)
         gens.append((f"dense/uvw/{np.dtype(dt).name}", select_generator(p)))
+        p = FullyConnectedTPProblem(*DIFFDOCK_L2, shared_weights=False, internal_weights=False, irrep_dtype=dt, weight_dtype=dt)
+        gens.append((f"diffdock/uvw per-row weights/{np.dtype(dt).name}", select_generator(p)))
+        for which, irreps in TETRIS_POLY.items():
+            p = FullyConnectedTPProblem(*irreps, shared_weights=True, internal_weights=False, irrep_dtype=dt, weight_dtype=dt)
+            gens.append((f"tetris-poly-{which}/uvw few weights/{np.dtype(dt).name}", select_generator(p)))
     return gens
 
 
