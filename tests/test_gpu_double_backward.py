@@ -62,3 +62,21 @@ def test_conv_double_backward(cuda, deterministic):
     r, c = torch.tensor(rows), torch.tensor(cols)
     _check(lambda x, y, w: conv.forward(x, y, w, *idx), lambda x, y, w: ref.conv_forward(x, y, w, r, c),
            common.conv_inputs(prob, nodes, nnz, 63, sh_lmax=2), cuda)
+
+
+@pytest.mark.parametrize("kind", ["few_shared_weights", "mfma", "per_row_weights"])
+def test_uvw_double_backward(cuda, kind):
+    """The same second-order check through the three uvw kernel families (multiplicities of at most 32 and one
+    copy of the second operand: the external weight order is e3nn's there, so the oracle takes the same W)."""
+    import openequivariance_amd as oeq
+    from openequivariance_amd.codegen.uvw import UVWGenerator
+    from openequivariance_amd.codegen.uvw_batched import UVWBatchedGenerator
+    from openequivariance_amd.codegen.uvw_rows import UVWRowsGenerator
+    irreps, shared, gen = {"few_shared_weights": (("6x0e+5x1o", "1x0e+1x1o", "1x0o+6x0e+3x1o"), True, UVWRowsGenerator),
+                           "mfma": (("16x0e+16x1o", "1x0e+1x1o", "16x0e+16x1o"), True, UVWGenerator),
+                           "per_row_weights": (("16x0e+16x1o", "1x0e+1x1o", "16x0e+16x1o"), False, UVWBatchedGenerator)}[kind]
+    prob, oprob = common.fully_connected(irreps, shared=shared)
+    tp = oeq.TensorProduct(prob, torch_op=True)
+    assert type(tp.generator) is gen
+    ref = torch_cpu.TorchTP(oprob, dtype=__import__("torch").float64)
+    _check(lambda x, y, w: tp(x, y, w), ref.forward, common.tp_inputs(prob, 90, 63, w_scale=0.3), cuda)
