@@ -33,6 +33,7 @@ DENSE = ("64x0e+64x1o+64x2e", "1x0e+1x1o+1x2e", "64x0e+64x1o+64x2e")
 TETRIS_POLY = {"1": ("1x0e+1x1o+1x2e+1x3o", "1x0e+1x1o+1x2e+1x3o", "64x0e+24x1e+24x1o+16x2e+16x2o"),
                "2": ("64x0e+24x1e+24x1o+16x2e+16x2o", "1x0e+1x1o+1x2e+1x3o", "1x0o+6x0e")}
 DIFFDOCK_L2 = ("10x1o+10x1e+48x0e+48x0o", "1x0e+1x1o+1x2e", "10x1o+10x1e+48x0e+48x0o")
+DIFFDOCK_L1 = ("10x1o+10x1e+48x0e+48x0o", "1x0e+1x1o", "10x1o+10x1e+48x0e+48x0o")
 
 
 def _normal(rng, shape, dtype, scale=1.0, chunk=1 << 24):
@@ -350,14 +351,19 @@ def get(name: str) -> Workload:
         w.alg_flops = {"forward": dense * w.units, "backward": 2 * dense * w.units}
         w.alg_bytes = _tp_bytes(prob, w.units, 4 if dt == "f32" else 8)
         return w
-    if name in ("diffdock_uvw_f32", "diffdock_uvw_f64"):
+    if name in ("diffdock_uvw_f32", "diffdock_uvw_f64", "diffdock1_uvw_f32", "diffdock1_uvw_f64"):
         dt = "f32" if name.endswith("f32") else "f64"
-        w = Workload(name, "uvw TP with a weight vector per row (DiffDock-L=2 of the reference's uvw benchmark), "
-                     "10x1o+10x1e+48x0e+48x0o (x) SH(lmax 2) -> 10x1o+10x1e+48x0e+48x0o, 12 instructions, 7128 weights "
-                     f"per row, batch 50000, {dt}, forward+backward", "tp", DIFFDOCK_L2, 50000, "rows/s", "hbm", dt,
-                     12351, {"batch": 50000, "paths": 12}, sh_lmax=2, mode="uvw", w_scale=0.2, shared=False,
+        L = 1 if name.startswith("diffdock1") else 2
+        irreps = DIFFDOCK_L1 if L == 1 else DIFFDOCK_L2
+        w = Workload(name, f"uvw TP with a weight vector per row (DiffDock-L={L} of the reference's uvw benchmark), "
+                     f"{irreps[0]} (x) SH(lmax {L}) -> {irreps[2]}, batch 50000, {dt}, forward+backward", "tp", irreps,
+                     50000, "rows/s", "hbm", dt, 12351, {"batch": 50000}, sh_lmax=L, mode="uvw", w_scale=0.2, shared=False,
                      device_inputs=True)
-        w.alg_bytes = _tp_bytes(w.problem(), w.units, 4 if dt == "f32" else 8)
+        prob = w.problem()
+        w.config["paths"] = len(prob.instructions)
+        w.description = w.description.replace(", batch 50000", f", {len(prob.instructions)} instructions, "
+                                              f"{prob.weight_numel} weights per row, batch 50000")
+        w.alg_bytes = _tp_bytes(prob, w.units, 4 if dt == "f32" else 8)
         return w
     if name.startswith("tetris_poly") and name[11:] in ("1_uvw_f32", "1_uvw_f64", "2_uvw_f32", "2_uvw_f64"):
         which, dt = name[11], name[-3:]
@@ -373,5 +379,5 @@ def get(name: str) -> Workload:
 
 ALL = ("readme_uvu", "mace_uvu", "mace_uvu_all_parities", "nequip_conv_atomic", "nequip_conv_det", "nequip_conv_det_all_parities",
        "large_conv_det", "large_conv_atomic", "large_conv_det_all_parities", "mace_conv_det", "mace_conv_atomic",
-       "dense_uvw_f32", "dense_uvw_f64", "diffdock_uvw_f32", "diffdock_uvw_f64",
+       "dense_uvw_f32", "dense_uvw_f64", "diffdock_uvw_f32", "diffdock_uvw_f64", "diffdock1_uvw_f32", "diffdock1_uvw_f64",
        "tetris_poly1_uvw_f32", "tetris_poly1_uvw_f64", "tetris_poly2_uvw_f32", "tetris_poly2_uvw_f64")
