@@ -50,9 +50,10 @@ class UVUDirectGenerator(UVUGenerator):
         # caches alike: 0.63 -> 0.56 ms); on the forward the hint measured slower (stores: 0.46 -> 0.52 ms
         # with flushed caches), so it keeps plain accesses.  ``tunables.tp_nontemporal`` lists the accesses
         # that get the hint (fl, fs, bl, bs = forward / backward loads / stores).  Writing the backward's dX
-        # through the LDS slot as full-line vector stores measured a tie (0.626 against 0.632 ms) and costs
-        # 37 registers, so dX keeps its record stores; dealing a row to four wavefronts of one workgroup
-        # measured no gain either (forward 0.456 ms, backward 0.59 ms).
+        # through the LDS slot as full-line vector stores costs 37 registers on this problem and measured
+        # slower (0.588 against 0.562 ms), so its dX keeps the record stores (dx_through_slot has the rule);
+        # dealing a row to four wavefronts of one workgroup measured no gain either (forward 0.456 ms,
+        # backward 0.59 ms).
         self._nt_modes = set(tunables.current.tp_nontemporal.split(",")) if kind == "tp" else set()
         self.nt_load = self.nt_store = False
         # one row per wavefront: the row index is wave-uniform and an out-of-range wavefront exits
@@ -129,6 +130,19 @@ class UVUDirectGenerator(UVUGenerator):
                                    self.act(blk), op)
         else:
             self.emit_slot_out(E, blk, names, ptr, rowdim, row_of, op)
+
+    def dx_through_slot(self, blk: Block) -> bool:
+        """Batch product: dX of this block leaves through the LDS slot as full 16-byte-per-lane vectors instead of
+        a lane's own record.  Measured on MI355X, backward in ms, records / slot: the single-path problems of
+        the reference's roofline set with l1 = 3, 5, 5, 6, 7, 7 (records of 7 to 15 words) 0.483 / 0.445,
+        1.006 / 0.660, 0.928 / 0.794, 1.261 / 1.123, 1.558 / 1.295, 1.592 / 1.212; l1 = 1 and 2 0.186 / 0.185 and
+        0.357 / 0.330; against that the 17-path MACE problem (l1 <= 2) 0.562 / 0.588, its 24-path variant
+        0.797 / 0.855, the 13-path 256-channel problem 0.320 / 0.329, the 11-path NequIP problem 0.079 / 0.078: long
+        records and single paths take the slot, short records in many-path problems (where its registers are
+        missed) keep the record stores."""
+        if self.kind != "tp":
+            return False
+        return blk.D >= 7 or len(self.paths) == 1
 
     def uexpr(self, c) -> str:
         return f"({c * self.P} + ul)" if isinstance(c, int) else f"(c * {self.P} + ul)"
@@ -309,7 +323,7 @@ class UVUDirectGenerator(UVUGenerator):
         E = Emitter()
         atomic = (self.kind == "conv_atomic")
         self.nt_load, self.nt_store = "bl" in self._nt_modes, "bs" in self._nt_modes
-        self.emit_lane_direct(E, lds=atomic)
+        self.emit_lane_direct(E, lds=atomic or any(self.dx_through_slot(self.in1[i]) for i in self.used_in1))
         xrow, zrow, srow = self._rows(E, backward=True)
         E(f"T* __restrict__ Wgr = Wg + {srow} * {self.WN};")
         self.emit_y_load_direct(E)
@@ -351,7 +365,8 @@ class UVUDirectGenerator(UVUGenerator):
                     continue
                 if a.idx in self.used_in1:
                     self.emit_block_store(E, a, [f"dx{a.idx}_{m}" for m in range(a.D)], "Xg", self.D1, xrow,
-                                          self.xrow_of, "atomic" if atomic else "store", via_lds=atomic)
+                                          self.xrow_of, "atomic" if atomic else "store",
+                                          via_lds=atomic or self.dx_through_slot(a))
                 elif not atomic:
                     self.emit_record_store(E, ["(T)0"] * a.D, f"Xg + (u64){xrow} * {self.D1} + {a.off} + u * {a.D}",
                                            self.act(a))

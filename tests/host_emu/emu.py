@@ -65,6 +65,8 @@ static inline int oeq_shfl_xor_i32(int v, int mask) { g_xi[threadIdx.x] = v; oeq
 static inline u64 oeq_uniform_u64(u64 v) { return v; }
 struct VT { T v[16 / sizeof(T)]; T& operator[](int i) { return v[i]; } const T& operator[](int i) const { return v[i]; } };
 typedef VT VTU;
+#define __builtin_nontemporal_store(v, p) (*(p) = (v))
+#define __builtin_nontemporal_load(p) (*(p))
 #define OEQ_DMA(BYTES, POLICY, g, lds_base) memcpy((char*)(lds_base) + ((BYTES) == 12 ? 16 : (BYTES)) * (threadIdx.x & 63), (g), (BYTES))
 static inline void oeq_release_agent() {}
 static inline void oeq_acquire_agent() {}

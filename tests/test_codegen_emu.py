@@ -43,6 +43,19 @@ def test_direct_tp_record_stores_only():
     _tp(UVUDirectGenerator, common.NEQUIP, 3, 3, vector_stores=False)
 
 
+@pytest.mark.parametrize("irreps,n", [(("128x3e", "1x3e", "128x3e"), 5),              # two full chunks, one path
+                                      (("20x5e+70x0e", "1x5e+1x0e", "70x3e+70x0e"), 7),  # 11-word records, ragged chunks
+                                      (("8x7e", "1x4e", "8x7e"), 9)],                     # eight rows per wavefront
+                         ids=["one_path_l3", "long_records_among_short_ones", "l7_eight_rows_per_wave"])
+def test_direct_tp_dx_through_the_lds_slot(irreps, n):
+    """Backward of the batch product with dX blocks that leave through the LDS slot (long records, single paths):
+    every lane count per row, chunks that are not full, blocks that keep their record stores beside them."""
+    prob, _ = common.channelwise(irreps)
+    g = UVUDirectGenerator(prob, "tp")
+    assert any(g.dx_through_slot(g.in1[i]) for i in g.used_in1)
+    _tp(UVUDirectGenerator, irreps, n, 31)
+
+
 def test_generic_tp_shared_weights():
     ins = [(0, 0, 0, "uvu", True), (1, 1, 0, "uvu", True), (1, 0, 1, "uvu", True)]
     a = ("24x0e+24x1o", "1x0e+1x1o", "24x0e+24x1o")
