@@ -45,6 +45,7 @@ class UVUDirectGenerator(UVUGenerator):
         self.lds_elems = max(stage) if stage else 0
         self.ZB = 0
         self.unroll_bwd_chunks = 1
+        self._lazy = False            # set per kernel body by lazy_operands()
         # Batch product: every tensor is read or written exactly once.  The backward's loads and stores
         # carry the non-temporal hint (measured on the 128-channel MACE problem, warm and with flushed
         # caches alike: 0.63 -> 0.56 ms); on the forward the hint measured slower (stores: 0.46 -> 0.52 ms
@@ -131,6 +132,36 @@ class UVUDirectGenerator(UVUGenerator):
         else:
             self.emit_slot_out(E, blk, names, ptr, rowdim, row_of, op)
 
+    LAZY_OPERANDS = None      # None: by the rule of lazy_operands(); True / False force it
+
+    def lazy_operands(self, direction: str) -> bool:
+        """Batch product with many paths: request dZ and the weights one output block ahead of their use
+        instead of all at the top of the row, and form the products x_i y_j that several paths share per
+        output block instead of carrying each in a register (two in fp64) from its first use to its last.
+        The carried products are what pushes the forward of the 68-path NequIP problem to 401 registers in
+        fp32 and past 512 into scratch in fp64 (130 with this); it costs vector-ALU work where registers
+        were not short.  Measured on MI355X over the reference's uvu set (batch 50 000, ms, eager / lazy):
+
+            problem (channels, paths)     fp32 forward   fp32 backward  fp64 forward   fp64 backward
+            mace-large   (128, 17)        0.452 / 0.486  0.559 / 0.572  0.962 / 0.961  1.345 / 1.369
+            mace-medium  (128,  8)        0.169 / 0.186  0.229 / 0.216  0.351 / 0.365  0.731 / 0.486
+            nequip-lips     (32, 30)      0.176 / 0.203  0.270 / 0.232  0.365 / 0.381  0.659 / 0.518
+            nequip-aspirin  (64, 10)      0.089 / 0.096  0.116 / 0.120  0.177 / 0.187  0.276 / 0.254
+            nequip-toluene  (64, 30)      0.344 / 0.374  0.469 / 0.442  0.731 / 0.748  1.132 / 1.025
+            nequip-benzene  (64, 68)      1.006 / 1.060  1.408 / 1.195  5.432 / 2.080  6.051 / 2.905
+            nequip-water    (32, 10)      0.039 / 0.040  0.058 / 0.061  0.089 / 0.096  0.153 / 0.130
+
+        The rule below takes the lazy form where it wins by more than a few per cent: the forward in fp64
+        from 40 paths on, the backward in fp64 or from 30 paths on."""
+        if self.LAZY_OPERANDS is not None:
+            return bool(self.LAZY_OPERANDS)
+        if self.kind != "tp":
+            return False
+        fp64, n = self.T == "double", len(self.paths)
+        if direction == "forward":
+            return fp64 and n >= 40
+        return fp64 or n >= 30
+
     def dx_through_slot(self, blk: Block) -> bool:
         """Batch product: dX of this block leaves through the LDS slot as full 16-byte-per-lane vectors instead of
         a lane's own record.  Measured on MI355X, backward in ms, records / slot: the single-path problems of
@@ -151,17 +182,26 @@ class UVUDirectGenerator(UVUGenerator):
         """Channel index of this lane in chunk c, clamped into the block."""
         return self.uexpr(c) if self.full(blk) else f"min({self.uexpr(c)}, {blk.mul - 1})"
 
+    def rows_always_stored(self) -> bool:
+        """Batch product with several rows per wavefront: the lanes past the batch work on its last row once
+        more and store it again (the same values to the same addresses) instead of storing nothing.  A store
+        under ``if (row < n)`` splits the unrolled kernel into blocks, and the compiler then moves the
+        arithmetic of what is stored later (all of dX) past the earlier ones, with every operand alive until
+        then: the 30-path NequIP problem with 32 channels took 335 registers in fp32 and spilled in fp64
+        (backward 1.35 ms against 0.39 ms of the forward)."""
+        return self.kind == "tp"
+
     def act(self, blk: Block) -> str:
-        rv = "true" if self.uniform_rows else "rv"
+        rv = "true" if (self.uniform_rows or self.rows_always_stored()) else "rv"
         if self.full(blk):
             return rv
-        return f"(u < {blk.mul})" if self.uniform_rows else f"(rv && u < {blk.mul})"
+        return f"(u < {blk.mul})" if rv == "true" else f"(rv && u < {blk.mul})"
 
     def act_c(self, blk: Block, c) -> str:
-        rv = "true" if self.uniform_rows else "rv"
+        rv = "true" if (self.uniform_rows or self.rows_always_stored()) else "rv"
         if self.full(blk):
             return rv
-        return f"({self.uexpr(c)} < {blk.mul})" if self.uniform_rows else f"(rv && {self.uexpr(c)} < {blk.mul})"
+        return f"({self.uexpr(c)} < {blk.mul})" if rv == "true" else f"(rv && {self.uexpr(c)} < {blk.mul})"
 
     def emit_record_load(self, E: Emitter, names, ptr: str, act: str, zero: bool = False) -> None:
         """Unconditional loads (the caller passes an address that is valid for every lane: idle
@@ -187,7 +227,13 @@ class UVUDirectGenerator(UVUGenerator):
 
     def emit_y_load_direct(self, E: Emitter) -> None:
         for f in self.used_y:
-            E(f"const T y{f} = Yr[{f}];")
+            E(f"{'' if self._lazy else 'const '}T y{f} = Yr[{f}];")
+
+    def emit_forget_products(self, E: Emitter) -> None:
+        """Between two output blocks of a many-path problem: the products x_i y_j that several paths share
+        are formed again per block instead of being carried, each in a register (two in fp64), from the
+        first block that uses them to the last."""
+        E(" ".join(f"OEQ_OPAQUE(y{f});" for f in self.used_y))
 
     def emit_weights(self, E: Emitter, p: Path, wptr: str) -> None:
         for v in range(p.mv):
@@ -235,8 +281,8 @@ class UVUDirectGenerator(UVUGenerator):
                 rc = "row"
             else:
                 E(f"const u64 row = (u64)blockIdx.x * {self.R} + sub;")
-                E("const bool rv = row < n;")
-                E("const u64 rowc = rv ? row : n - 1;")    # idle lanes read the last row and store nothing
+                E("const bool rv = row < n; (void)rv;")
+                E("const u64 rowc = rv ? row : n - 1;")    # idle lanes work on the last row once more
                 rc = "rowc"
             E(f"const T* __restrict__ Yr = Y + {rc} * {self.D2};")
             E(f"const T* __restrict__ Wr = W + {rc} * {self.WN};")
@@ -244,8 +290,8 @@ class UVUDirectGenerator(UVUGenerator):
                 self.xrow_of = self.zrow_of = (lambda r: ("row", "true"))
             else:
                 base = f"(u64)blockIdx.x * {self.R}"
-                self.xrow_of = self.zrow_of = (lambda r: (f"({base} + {r})", f"({base} + {r} < n)"))
-            return rc, rc, "row"
+                self.xrow_of = self.zrow_of = (lambda r: (f"min({base} + {r}, n - 1)", "true"))
+            return rc, rc, rc
         # convolution: an edge is idle when it is out of range or names a node that does not exist;
         # idle lanes read edge/node 0 (callers never launch with zero nodes) and store nothing
         if self.uniform_rows:
@@ -289,10 +335,12 @@ class UVUDirectGenerator(UVUGenerator):
         self.nt_load, self.nt_store = "fl" in self._nt_modes, "fs" in self._nt_modes
         self.emit_lane_direct(E, lds=True)
         xrow, zrow, _ = self._rows(E)
+        lazy = self._lazy = self.lazy_operands("forward")
         self.emit_y_load_direct(E)
         for c in range(self.NCH):
             self.emit_x_preload(E, c, xrow)
-            self.emit_weight_preload(E, c)
+            if not lazy:
+                self.emit_weight_preload(E, c)
         for c in range(self.NCH):
             self._cur_c = self._loop_c = c
             E("{")
@@ -300,9 +348,20 @@ class UVUDirectGenerator(UVUGenerator):
             E(f"const int c = {c}; (void)c;")
             E(f"const int u = {c * self.P} + ul;")
             self.emit_x_alias(E, c)
+            outs = [o for o in self.out if o.dim and o.idx in self.used_out]
+            if lazy and outs:
+                self.emit_weight_preload(E, c, only={p.t for p in self.paths_into(outs[0].idx)})
             for o in self.out:
                 if o.dim == 0:
                     continue
+                if lazy and o.idx in self.used_out:
+                    # one output block's weights in flight ahead of the block being computed; the fence keeps
+                    # the compiler from gathering the loads of all blocks at the top again
+                    E("oeq_sched_fence();")
+                    self.emit_forget_products(E)
+                    nxt = outs[outs.index(o) + 1:]
+                    if nxt:
+                        self.emit_weight_preload(E, c, only={p.t for p in self.paths_into(nxt[0].idx)})
                 E("{")
                 E.level += 1
                 if o.idx in self.used_out:
@@ -326,6 +385,7 @@ class UVUDirectGenerator(UVUGenerator):
         self.emit_lane_direct(E, lds=atomic or any(self.dx_through_slot(self.in1[i]) for i in self.used_in1))
         xrow, zrow, srow = self._rows(E, backward=True)
         E(f"T* __restrict__ Wgr = Wg + {srow} * {self.WN};")
+        self._lazy = self.lazy_operands("backward")
         self.emit_y_load_direct(E)
         for f in self.used_y:
             E(f"T dy{f} = (T)0;")
@@ -334,19 +394,32 @@ class UVUDirectGenerator(UVUGenerator):
         def chunk(E, c):
             tag = c if isinstance(c, int) else "c"
             self._cur_c = tag
-            self.emit_x_preload(E, c, xrow)
-            self.emit_weight_preload(E, c)
-            for oi in self.used_out:
+            lazy = self._lazy
+
+            def fetch(oi):
                 o = self.out[oi]
                 self.emit_record_load(E, [f"G{oi}_{k}" for k in range(o.D)],
                                       f"G + (u64){zrow} * {self.D3} + {o.off} + {self.uclamp(o, c)} * {o.D}",
                                       self.act(o), zero=True)
+                if lazy:
+                    self.emit_weight_preload(E, c, only={p.t for p in self.paths_into(oi)})
+            self.emit_x_preload(E, c, xrow)
+            if not lazy:
+                self.emit_weight_preload(E, c)
+            for oi in (self.used_out[:1] if lazy else self.used_out):
+                fetch(oi)
             self.emit_x_alias(E, tag)
             for i in self.used_in1:
                 for m in range(self.in1[i].D):
                     E(f"T dx{i}_{m} = (T)0;")
-            for oi in self.used_out:
+            for n_, oi in enumerate(self.used_out):
                 o = self.out[oi]
+                if lazy:
+                    # dZ and weights of one output block in flight ahead of the block being worked on
+                    E("oeq_sched_fence();")
+                    self.emit_forget_products(E)
+                    if n_ + 1 < len(self.used_out):
+                        fetch(self.used_out[n_ + 1])
                 E("{")
                 E.level += 1
                 for k in range(o.D):
@@ -398,8 +471,8 @@ class UVUDirectGenerator(UVUGenerator):
             self.emit_dy_reduce(E)
             writer = "ul == 0"
         if self.kind == "tp":
-            E(f"if (rv && {writer}) {{")
-            E(f"    T* __restrict__ Ygr = Yg + row * {self.D2};")
+            E(f"if ({writer}) {{")
+            E(f"    T* __restrict__ Ygr = Yg + {'row' if self.uniform_rows else 'rowc'} * {self.D2};")
         else:
             E(f"if (e < nnz && {writer}) {{")
             E(f"    T* __restrict__ Ygr = Yg + e * {self.D2};")

@@ -87,6 +87,7 @@ static inline V2 oeq_ldnt2(const T* p) { assert((uintptr_t)p % (2 * sizeof(T)) =
 static inline void oeq_stnt2(T* p, V2 v) { assert((uintptr_t)p % (2 * sizeof(T)) == 0); p[0] = v[0]; p[1] = v[1]; }
 static inline void oeq_block_sync() { pthread_barrier_wait(&g_bar); }
 static inline void oeq_sched_fence() {}
+#define OEQ_OPAQUE(x) ((void)0)
 static inline void __syncthreads() { pthread_barrier_wait(&g_bar); }
 #define __HIP_MEMORY_SCOPE_AGENT 0
 #define __HIP_MEMORY_SCOPE_WORKGROUP 0

@@ -56,6 +56,17 @@ def test_direct_tp_dx_through_the_lds_slot(irreps, n):
     _tp(UVUDirectGenerator, irreps, n, 31)
 
 
+@pytest.mark.parametrize("irreps,n", [(common.NEQUIP, 5),
+                                      (("5x0e+3x1o+70x2e", "1x0e+1x1o+1x2e", "5x0e+3x1o+70x2e+7x3o"), 3),
+                                      (("64x0o+64x0e+64x1o+64x1e", "1x0e+1x1o", "64x0o+64x0e+64x1o+64x1e"), 2)],
+                         ids=["two_rows_per_wave", "ragged_two_chunks", "both_parities"])
+def test_direct_tp_operands_one_output_block_ahead(irreps, n, monkeypatch):
+    """The batch product with dZ and the weights requested one output block ahead and the shared x_i y_j
+    products formed per block (the form many-path problems take), forced here on small problems."""
+    monkeypatch.setattr(UVUDirectGenerator, "LAZY_OPERANDS", True)
+    _tp(UVUDirectGenerator, irreps, n, 41)
+
+
 def test_generic_tp_shared_weights():
     ins = [(0, 0, 0, "uvu", True), (1, 1, 0, "uvu", True), (1, 0, 1, "uvu", True)]
     a = ("24x0e+24x1o", "1x0e+1x1o", "24x0e+24x1o")
