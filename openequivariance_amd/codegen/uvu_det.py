@@ -105,7 +105,11 @@ class UVUDetGenerator(UVUDirectGenerator):
         # per-edge register footprint is small enough to keep several wavefronts per SIMD
         if prefetch_backward is None:
             prefetch_backward = tunables.current.det_prefetch
-        self.prefetch_backward = (words <= 80) if prefetch_backward is None else prefetch_backward
+        # (fp64: every word is two registers, and the second set does not fit what two wavefronts per SIMD leave
+        # each: with it the 32-channel NequIP backward spilled 636 bytes per lane and took 1.26 instead of 0.43 ms,
+        # the 128-channel MACE backward 19.4 instead of 6.3 ms)
+        self.prefetch_backward = ((words <= 80 and self.T == "float") if prefetch_backward is None
+                                  else prefetch_backward)
         # W / Y / dW / dY are touched once: the streaming hint keeps them from evicting the gathered rows
         # (256 channels, without the hint: forward 2.58 -> 2.73 ms, backward 7.68 -> 8.91 ms)
         self.nontemporal = True
