@@ -37,6 +37,10 @@ from .uvu_direct import UVUDirectGenerator
 class UVUDetGenerator(UVUDirectGenerator):
     _allow_det = True
     SPLIT_WORDS = 80
+    # words per group when the backward is split (fp64, 5000 nodes / 150 000 edges, 64 -> 24 words per group: 17 paths
+    # at 128 channels 3.12 -> 2.52 ms, 68 paths 9.38 -> 7.56 ms, 30 paths 2.11 -> 1.98 and 1.27 -> 1.33 ms)
+    SPLIT_TARGET = {"float": 64, "double": 24}
+    FWD_SPLIT_WORDS = {"float": 100, "double": 72}
     # int64 words of one on-the-fly grouping of the edges in the workspace: group pointers and fill cursors
     # (node_count + 1 each), the position list (nnz), the counters (node_count + 1) and the ticket of the
     # counting kernel
@@ -48,7 +52,7 @@ class UVUDetGenerator(UVUDirectGenerator):
 
     def __init__(self, problem: TPProblem, prefetch_backward=None, vector_stores: bool = True,
                  forward_perm: bool = False, backward_perm: bool = False, idx_ctype: str = "i64",
-                 allow_split: bool = True, lds=None, long_node=None):
+                 allow_split: bool = True, lds=None, long_node=None, fwd_split=None):
         super().__init__(problem, "conv_det", vector_stores=vector_stores)
         self.idx_ctype = idx_ctype
         # True: the forward walks the receiver-grouped edge order listed in the workspace (built on
@@ -89,7 +93,7 @@ class UVUDetGenerator(UVUDirectGenerator):
         split = tunables.current.det_split                      # 0: never; a number: threshold for A/B runs
         limit = split if split else self.SPLIT_WORDS
         if words > limit and split != 0 and allow_split:
-            H = min(len(self.used_out), -(-words // 64))
+            H = min(len(self.used_out), -(-words // self.SPLIT_TARGET[self.T]))
         self.out_groups = [[] for _ in range(H)]
         for oi in sorted(self.used_out, key=lambda i: -(self.out[i].D + len(self.paths_into(i)))):
             min(self.out_groups, key=words_of).append(oi)
@@ -142,6 +146,20 @@ class UVUDetGenerator(UVUDirectGenerator):
         self.lds_forward = (self.T == "float" and self.P >= self.D2 and lds is not False
                             and (self.NCH == 1 or (fwd_operands >= 26 and not forward_perm) or lds is True)
                             and 16 * (fwd_words + self.lds_elems) * 4 <= 160 * 1024)
+        # Forward: the sums of every output block of a node stay in registers across its edge list.  Beyond
+        # FWD_SPLIT_WORDS words per lane the loop spilled them (5000 nodes, 150 000 edges, fp32 / fp64: 30 paths and 102
+        # words 0.68 / 3.33 ms, 68 paths and 312 words 19.6 / 44.6 ms), so the output blocks are dealt into groups, one
+        # forward launch per group: each launch reads X, Y and its own weights and writes its blocks of Z (the same
+        # problems then 0.35 / 0.75 and 1.14 / 2.71 ms; 71 words in one launch: 0.38 / 0.95 ms, in two 0.41 / 0.99).
+        z_regs = lambda outs: sum(self.out[i].D for i in outs)
+        HF = 1
+        fsplit = self.FWD_SPLIT_WORDS[self.T] if fwd_split is None else fwd_split
+        if fsplit and z_regs(self.used_out) > fsplit:
+            HF = min(len(self.used_out), -(-z_regs(self.used_out) // fsplit))
+        self.fwd_groups = [[] for _ in range(HF)]
+        for oi in sorted(self.used_out, key=lambda i: -self.out[i].D):
+            min(self.fwd_groups, key=z_regs).append(oi)
+        self.fwd_groups = [sorted(g_) for g_ in self.fwd_groups if g_] or [[]]
         self.uniform_rows = False          # validity is per lane (edge lists differ between sub-rows)
         self.chunk_in_grid = True
         # the regrouped backward arithmetic (see UVUGenerator.regroup_pairs) where registers are to spare: measured
@@ -161,10 +179,11 @@ class UVUDetGenerator(UVUDirectGenerator):
         self.piece_base = f"((({self.flags_off} + 4ull * ((nnz + 255) / 256)) + 255ull) & ~255ull)"
 
     @contextlib.contextmanager
-    def _group(self, h: int):
-        """Restricts the generator to the paths into the output blocks of group h (backward launches)."""
+    def _group(self, h: int, groups=None):
+        """Restricts the generator to the paths into the output blocks of group h (of the backward launches, or
+        of ``groups``)."""
         saved = (self.paths, self.used_out, self.used_in1, self.used_y)
-        outs = self.out_groups[h]
+        outs = (self.out_groups if groups is None else groups)[h]
         self.paths = [p for p in saved[0] if p.o.idx in outs]
         self.used_out = list(outs)
         self.used_in1 = sorted({p.a.idx for p in self.paths})
@@ -177,6 +196,18 @@ class UVUDetGenerator(UVUDirectGenerator):
     def backward_kernels(self):
         """(kernel name, group) of the backward launches, in launch order."""
         return [("backward" if h == 0 else f"backward_g{h}", h) for h in range(self.H)]
+
+    def forward_kernels(self):
+        """(kernel name, group) of the forward launches, in launch order."""
+        return [("forward" if h == 0 else f"forward_g{h}", h) for h in range(len(self.fwd_groups))]
+
+    def forward_kernel_sources(self):
+        """The forward's compute kernels as the templates emit them: name and body."""
+        return [dict(name=name, body=self.conv_det_forward_body(h)) for name, h in self.forward_kernels()]
+
+    def forward_steps(self, step: dict):
+        """One launch like ``step`` per group of output blocks."""
+        return [dict(step, kernel=name) for name, _ in self.forward_kernels()]
 
     def backward_kernel_sources(self):
         """The backward's compute kernels as the templates emit them: name, workgroup size, attributes, body."""
@@ -301,10 +332,11 @@ class UVUDetGenerator(UVUDirectGenerator):
         self.noderow_of = (lambda r: ("node", "nv"))
 
     def emit_node_output(self, E: Emitter, blocks, used, regs_of, ptr: str, rowdim: int, via_lds: bool,
-                         zero_unused: bool, add_existing: bool) -> None:
+                         zero_unused: bool, add_existing: bool, elsewhere=()) -> None:
         """The sums a wavefront holds for its node (registers ``regs_of(block)`` of the blocks in ``used``) ->
         row ``node`` of ``ptr``; blocks nothing contributes to are zero-filled (``zero_unused``); with
-        ``add_existing`` the row already holds the sums of an earlier launch and is added to.  A piece
+        ``add_existing`` the row already holds the sums of an earlier launch and is added to; blocks in
+        ``elsewhere`` are written by another launch and left alone.  A piece
         stores its sums in its partial row instead; the piece of a node that finishes last adds all pieces
         in list order and writes the node's row."""
         for blk in blocks:
@@ -330,7 +362,7 @@ class UVUDetGenerator(UVUDirectGenerator):
                         E(f"if ({self.store_act(blk)}) {{ const T* __restrict__ q_ = {dst}; "
                           + " ".join(f"{n} += q_[{m}];" for m, n in enumerate(regs_of(blk))) + " }")
                     self.emit_record_store(E, regs_of(blk), dst, self.store_act(blk))
-                elif zero:
+                elif zero and blk.idx not in elsewhere:
                     self.emit_record_store(E, ["(T)0"] * blk.D, dst, self.store_act(blk))
                 E.level -= 1
                 E("}")
@@ -486,6 +518,7 @@ class UVUDetGenerator(UVUDirectGenerator):
         for s in fwd:
             if s["kernel"] == "forward":
                 s.update(work_per_block=1, grid_kind=3, num_blocks=self.LONG)
+        fwd = [t for s in fwd for t in (self.forward_steps(s) if s["kernel"] == "forward" else [s])]
         bwd = [s for s in bwd if s["kernel"] == "prep_backward"] + self.backward_steps()
 
         def ws(nnz=0, nodes=0):
@@ -503,7 +536,11 @@ class UVUDetGenerator(UVUDirectGenerator):
         return 8, 8, 0
 
     # ================================================================= forward
-    def conv_det_forward_body(self) -> str:
+    def conv_det_forward_body(self, h: int = 0) -> str:
+        with self._group(h, self.fwd_groups):
+            return self._forward_body(h)
+
+    def _forward_body(self, h: int) -> str:
         E = Emitter()
         self.emit_lane_direct(E, lds=True)
         if self.forward_perm:
@@ -576,7 +613,8 @@ class UVUDetGenerator(UVUDirectGenerator):
             self.emit_pingpong_loop(E, names, load_idx, load, compute)
         E("const bool rv = nv;")
         self.emit_node_output(E, self.out, self.used_out, lambda o: [f"z{o.idx}_{k}" for k in range(o.D)], "Z", self.D3,
-                              via_lds=True, zero_unused=True, add_existing=False)
+                              via_lds=True, zero_unused=(h == 0), add_existing=False,
+                              elsewhere={oi for g_ in self.fwd_groups for oi in g_} - set(self.used_out))
         return E.text()
 
     def uclamp(self, blk, c) -> str:

@@ -96,8 +96,8 @@ class UVUSortedGenerator:
                          prep=True, counter_clear=True),
                     dict(kernel="group_count" + sfx, num_threads=S, grid_kind=ROW, work_per_block=S, prep=True),
                     dict(kernel="group_fill" + sfx, num_threads=256, grid_kind=ROW, work_per_block=256, prep=True)]
-        fwd = grouping("") + [dict(kernel="forward", num_threads=64, grid_kind=3, work_per_block=1, num_blocks=f.LONG,
-                                   grid_y=f.NCH)]
+        fwd = grouping("") + f.forward_steps(dict(kernel="forward", num_threads=64, grid_kind=3, work_per_block=1,
+                                                  num_blocks=f.LONG, grid_y=f.NCH))
         G = f.group_bytes
         if not self.grouped_backward:
             _, bwd, _ = self.bwd.plan()

@@ -328,6 +328,10 @@ def run_conv(gen, steps: Sequence[Dict], X, Y, W, rows, cols, G=None, tperm=None
             if gen.recv_backward:
                 extra += CONV_EXTRA_GROUPED_BWD.replace("_backward", "_recv")
             det = gen.bwd
+    fdet = gen if gen.kind == "conv_det" else getattr(gen, "fwd", None)
+    if fdet is not None:
+        for k in fdet.forward_kernels()[1:]:
+            extra += f'        else if (k == "{k[0]}") FWD_CALL({k[0]});\n'
     if det is not None:
         if det.ordered_backward:
             extra += CONV_EXTRA_ORDER

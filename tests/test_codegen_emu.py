@@ -167,6 +167,53 @@ def test_conv_long_node_of_more_pieces_than_one_group():
     assert rel_err(out["Z"], otp.conv_forward(oprob, X, Y, W, rows, cols)) < TOL
 
 
+@pytest.mark.parametrize("case", ["det_registers", "det_lds", "det_two_chunks", "unsorted", "det_hubs", "unsorted_hubs",
+                                  "untouched_output_block"])
+def test_conv_forward_one_launch_per_group_of_output_blocks(case, monkeypatch):
+    """The forward of problems with more output words than a wavefront keeps in registers runs once per group of
+    output blocks: forced here on small problems (a group per 4 words), on a junk-filled Z, with hubs
+    walked in pieces, with an output block that no path writes, over a position list built on the fly."""
+    from openequivariance_amd.codegen.uvu_recv import UVURecvGenerator
+    monkeypatch.setattr(UVUDetGenerator, "FWD_SPLIT_WORDS", {"float": 4, "double": 4})
+    irreps = {"det_two_chunks": ("5x0e+3x1o+70x2e", "1x0e+1x1o+1x2e", "5x0e+3x1o+70x2e+7x3o"),
+              }.get(case, common.NEQUIP)
+    prob, oprob = common.channelwise(irreps)
+    if case == "untouched_output_block":
+        a = ("16x0e+16x1o", "1x0e+1x1o", "16x0e+16x1o+16x2e+16x1e")
+        ins = [(0, 0, 0, "uvu", True), (1, 1, 0, "uvu", True), (0, 1, 1, "uvu", True), (1, 0, 1, "uvu", True),
+               (1, 1, 3, "uvu", True)]
+        prob = oeq.TPProblem(*a, ins, shared_weights=False, internal_weights=False)
+        oprob = spec.Problem(*a, ins, shared_weights=False)
+    det = case.startswith("det") or case == "untouched_output_block"
+    if case in ("det_registers", "det_lds"):
+        g = UVUDetGenerator(prob, lds=case == "det_lds")
+        assert g.lds_forward == (case == "det_lds")
+    elif det:
+        g = UVUDetGenerator(prob)
+    else:
+        g = UVUSortedGenerator(prob, grouped_backward=False)
+    f = g.fwd if hasattr(g, "fwd") else g
+    assert len(f.fwd_groups) >= 2 and sorted(o for grp in f.fwd_groups for o in grp) == f.used_out
+    if case.endswith("hubs"):
+        nodes, nnz = 12, 400
+        rows, cols = common.hub_graph(nodes - 1, nnz, 21, hub_in=3, hub_out=5, in_edges=150, out_edges=130)
+    else:
+        nodes, nnz = 7, 45
+        rows, cols = common.random_graph(nodes - 1, nnz, 5)               # the last node has no edges
+    tperm = np.arange(nnz)
+    if det:
+        rows, cols, tperm, _ = otp.coord_graph(rows, cols)
+    X, Y, W, G = common.conv_inputs(prob, nodes, nnz, 6)
+    fwd, bwd, ws = g.plan()
+    assert [s["kernel"] for s in fwd if s["kernel"].startswith("forward")] == [k for k, _ in f.forward_kernels()]
+    out = emu.run_conv(g, fwd, X, Y, W, rows, cols, tperm=tperm, ws_bytes=ws(nnz, nodes))
+    assert rel_err(out["Z"], otp.conv_forward(oprob, X, Y, W, rows, cols)) < TOL
+    assert not out["Z"][nodes - 1].any()
+    if case == "untouched_output_block":
+        blk = [b for b in f.out if b.idx not in f.used_out]
+        assert blk and not out["Z"][:, blk[0].off:blk[0].off + blk[0].dim].any()
+
+
 @pytest.mark.parametrize("staged", [True, False])
 def test_conv_det_long_edge_lists(staged):
     """Edge lists of about 13 edges per node (6-7 iterations of two sub-lists) reach the steady state of

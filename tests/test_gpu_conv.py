@@ -199,6 +199,26 @@ def test_conv_fp64(cuda):
     _run(prob, oprob, 64, 900, 36, False, dtype=np.float64, sh_lmax=2)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64], ids=["fp32", "fp64"])
+@pytest.mark.parametrize("deterministic", [False, True])
+@pytest.mark.parametrize("which", ["nequip-lips", "nequip-revmd17-benzene"])
+def test_conv_forward_in_groups_of_output_blocks(cuda, which, deterministic, dtype):
+    """The reference's NequIP convolution problems with 30 and 68 paths (outputs of either parity up to l = 2 and
+    3: 102 and 312 output words per channel): the forward runs one launch per group of output blocks, the backward
+    (sender order in fp64) likewise; a hub node makes one edge list long enough to be walked in pieces."""
+    from openequivariance_amd.benchmark import benchmark_configs as bc
+    irreps = [c[:3] for c in bc.nequip_conv if c[3] == which][0]
+    prob, oprob = common.channelwise(irreps, dtype=dtype)
+    nodes, nnz = 40, 900
+    rows, cols = common.hub_graph(nodes - 1, nnz, 61, hub_in=3, hub_out=5, in_edges=300, out_edges=200)
+    tperm = None
+    if deterministic:
+        rows, cols, tperm, _ = otp.coord_graph(rows, cols)
+    conv, _ = _run(prob, oprob, nodes, nnz, 62, deterministic, dtype=dtype, graph=(rows, cols, tperm))
+    f = getattr(conv.generator, "fwd", conv.generator)
+    assert len(f.fwd_groups) >= 2 and f.piece_tiles(nnz, nodes) > 0
+
+
 @pytest.mark.parametrize("deterministic", [False, True])
 def test_conv_fp64_ragged_chunks(cuda, deterministic):
     """fp64 with multiplicities above one wavefront (two chunks, the second partly filled) and below it."""
