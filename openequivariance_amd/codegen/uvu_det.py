@@ -41,6 +41,7 @@ class UVUDetGenerator(UVUDirectGenerator):
     # at 128 channels 3.12 -> 2.52 ms, 68 paths 9.38 -> 7.56 ms, 30 paths 2.11 -> 1.98 and 1.27 -> 1.33 ms)
     SPLIT_TARGET = {"float": 64, "double": 24}
     FWD_SPLIT_WORDS = {"float": 100, "double": 72}
+    FWD_COHERENT = True
     # int64 words of one on-the-fly grouping of the edges in the workspace: group pointers and fill cursors
     # (node_count + 1 each), the position list (nnz), the counters (node_count + 1) and the ticket of the
     # counting kernel
@@ -156,10 +157,7 @@ class UVUDetGenerator(UVUDirectGenerator):
         fsplit = self.FWD_SPLIT_WORDS[self.T] if fwd_split is None else fwd_split
         if fsplit and z_regs(self.used_out) > fsplit:
             HF = min(len(self.used_out), -(-z_regs(self.used_out) // fsplit))
-        self.fwd_groups = [[] for _ in range(HF)]
-        for oi in sorted(self.used_out, key=lambda i: -self.out[i].D):
-            min(self.fwd_groups, key=z_regs).append(oi)
-        self.fwd_groups = [sorted(g_) for g_ in self.fwd_groups if g_] or [[]]
+        self.fwd_groups = self.coherent_groups(HF, z_regs) if self.FWD_COHERENT else self.dealt_groups(HF, z_regs)
         self.uniform_rows = False          # validity is per lane (edge lists differ between sub-rows)
         self.chunk_in_grid = True
         # the regrouped backward arithmetic (see UVUGenerator.regroup_pairs) where registers are to spare: measured
@@ -177,6 +175,29 @@ class UVUDetGenerator(UVUDirectGenerator):
         self.LONG = max(0, int(tunables.current.long_node)) if long_node is None else int(long_node)
         # byte offset (C expression) of the piece area in the workspace: counters, then partial rows
         self.piece_base = f"((({self.flags_off} + 4ull * ((nnz + 255) / 256)) + 255ull) & ~255ull)"
+
+    def dealt_groups(self, n: int, words_of):
+        """The output blocks in n groups of about equal ``words_of``, largest block first."""
+        groups = [[] for _ in range(n)]
+        for oi in sorted(self.used_out, key=lambda i: -words_of([i])):
+            min(groups, key=words_of).append(oi)
+        return [sorted(g_) for g_ in groups if g_] or [[]]
+
+    def coherent_groups(self, n: int, words_of):
+        """The output blocks in n groups of about equal ``words_of``, cut from the list ordered by the in1 block
+        their paths read: a launch gathers only the X blocks its paths use, so groups that share them gather
+        less."""
+        first_in = lambda oi: min((p.a.idx for p in self.paths_into(oi)), default=0)
+        order = sorted(self.used_out, key=lambda oi: (first_in(oi), oi))
+        total = words_of(order)
+        groups, acc = [[]], 0
+        for oi in order:
+            w = words_of([oi])
+            if groups[-1] and len(groups) < n and acc + w / 2 > total * len(groups) / n:
+                groups.append([])
+            groups[-1].append(oi)
+            acc += w
+        return [sorted(g_) for g_ in groups if g_] or [[]]
 
     @contextlib.contextmanager
     def _group(self, h: int, groups=None):

@@ -254,14 +254,17 @@ def build(source: str, main: str) -> pathlib.Path:
     exe = CACHE / f"emu_{key}"
     if exe.exists():
         return exe
-    src = CACHE / f"emu_{key}.cpp"
+    # (per-process names: test workers running side by side may build the same source at the same time)
+    src = CACHE / f"emu_{key}.{os.getpid()}.cpp"
+    tmp = f"{exe}.{os.getpid()}.tmp"
     src.write_text(text)
     cmd = ["g++", "-std=c++17", "-O1", "-g", "-fsanitize=address", "-static-libasan", "-fno-omit-frame-pointer",
-           "-Wno-unknown-pragmas", "-ffp-contract=off", str(src), "-o", str(exe) + ".tmp", "-lpthread"]
+           "-Wno-unknown-pragmas", "-ffp-contract=off", str(src), "-o", tmp, "-lpthread"]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError("host build of generated kernel failed:\n" + res.stderr[-6000:])
-    os.replace(str(exe) + ".tmp", exe)
+    os.replace(tmp, exe)
+    os.replace(src, CACHE / f"emu_{key}.cpp")
     return exe
 
 
