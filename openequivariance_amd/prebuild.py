@@ -28,6 +28,9 @@ def benchmark_generators():
     for label, irreps in (("nequip", NEQUIP), ("large", LARGE), ("mace", MACE)):
         for det in (False, True):
             gens.append((f"{label}/conv_{'det' if det else 'atomic'}", select_conv_generator(ChannelwiseTPP(*irreps), det)))
+    for det in (False, True):
+        p = ChannelwiseTPP(*MACE, irrep_dtype=np.float64, weight_dtype=np.float64)
+        gens.append((f"mace/conv_{'det' if det else 'atomic'}/float64", select_conv_generator(p, det)))
     for dt in (np.float32, np.float64):
         p = FullyConnectedTPProblem(*DENSE, shared_weights=True, internal_weights=False, irrep_dtype=dt, weight_dtype=dt)
         gens.append((f"dense/uvw/{np.dtype(dt).name}", select_generator(p)))

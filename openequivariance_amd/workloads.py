@@ -322,12 +322,14 @@ def get(name: str) -> Workload:
                         "conv", LARGE, 800000, "edges/s", "hbm", "f32", 12349,
                         {"nodes": 20000, "paths": 13, "deterministic": det}, nodes=20000, deterministic=det, sh_lmax=3,
                         device_inputs=True)
-    if name in ("mace_conv_det", "mace_conv_atomic"):
-        det = name.endswith("det")
+    if name in ("mace_conv_det", "mace_conv_atomic", "mace_conv_det_f64", "mace_conv_atomic_f64"):
+        # (the reference's convolution benchmark runs this problem in fp32 and in fp64, test/benchmark.py:179-188)
+        dt = "f64" if name.endswith("_f64") else "f32"
+        det = "_det" in name
         return Workload(name, "MACE-style fused uvu conv (the problem of the tensor-product benchmark as a convolution), "
-                        "128x0e+128x1o+128x2e (x) SH(lmax 3) -> l3<=3, 17 paths, 10000 nodes, 300000 edges, fp32, "
+                        f"128x0e+128x1o+128x2e (x) SH(lmax 3) -> l3<=3, 17 paths, 10000 nodes, 300000 edges, fp{dt[1:]}, "
                         "forward+backward, " + ("deterministic (receiver-sorted)" if det else "unsorted"),
-                        "conv", MACE, 300000, "edges/s", "hbm", "f32", 12350,
+                        "conv", MACE, 300000, "edges/s", "hbm", dt, 12350,
                         {"nodes": 10000, "paths": 17, "deterministic": det}, nodes=10000, deterministic=det, sh_lmax=3)
     if name == "nequip_conv_det_all_parities":
         return Workload(name, "fused uvu conv, 32x0e+32x1o+32x2e (x) SH(lmax 2) -> every triangle-allowed l3<=2 of either "
@@ -379,5 +381,5 @@ def get(name: str) -> Workload:
 
 ALL = ("readme_uvu", "mace_uvu", "mace_uvu_all_parities", "nequip_conv_atomic", "nequip_conv_det", "nequip_conv_det_all_parities",
        "large_conv_det", "large_conv_atomic", "large_conv_det_all_parities", "mace_conv_det", "mace_conv_atomic",
-       "dense_uvw_f32", "dense_uvw_f64", "diffdock_uvw_f32", "diffdock_uvw_f64", "diffdock1_uvw_f32", "diffdock1_uvw_f64",
+       "mace_conv_det_f64", "mace_conv_atomic_f64", "dense_uvw_f32", "dense_uvw_f64", "diffdock_uvw_f32", "diffdock_uvw_f64", "diffdock1_uvw_f32", "diffdock1_uvw_f64",
        "tetris_poly1_uvw_f32", "tetris_poly1_uvw_f64", "tetris_poly2_uvw_f32", "tetris_poly2_uvw_f64")
