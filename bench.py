@@ -731,7 +731,7 @@ def measure(name, steps, warmup, cold=True, cpu=True, cpu_sample=0, ceiling=True
     return wl, rec
 
 
-# every BASELINE configuration besides the headline one (config 2 = mace_uvu), the MACE problem as a convolution, and
+# every benchmark configuration besides the headline one (config 2 = mace_uvu), the MACE problem as a convolution, and
 # one problem of each of the other two uvw kernel families (per-row weights, few shared weights)
 OTHER_WORKLOADS = ("readme_uvu", "nequip_conv_det", "nequip_conv_atomic", "dense_uvw_f32", "dense_uvw_f64",
                    "large_conv_det", "large_conv_atomic", "mace_conv_det", "diffdock_uvw_f32", "tetris_poly1_uvw_f32")
@@ -770,7 +770,7 @@ def main():
            "roofline": rec["roofline"], "torch_op": rec["torch_op"], "cpu_baseline": rec["cpu_baseline"],
            "device": torch.cuda.get_device_name(0)}
     if not args.workload and not args.headline_only:
-        # the other BASELINE configurations, same protocol (same steps and warm-up, HIP events around every
+        # the other benchmark configurations, same protocol (same steps and warm-up, HIP events around every
         # launch), with a shorter CPU leg each
         others = {}
         for name in OTHER_WORKLOADS:
