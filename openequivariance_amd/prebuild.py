@@ -14,6 +14,7 @@ from . import runtime as rt
 from .conv import select_conv_generator
 from .problem import ChannelwiseTPP, FullyConnectedTPProblem, TPProblem
 from .tensor_product import select_generator
+from .workloads import get as get_workload
 from .workloads import DENSE, DIFFDOCK_L2, LARGE, MACE, MACE_ALL, NEQUIP, TETRIS_POLY
 
 
@@ -31,6 +32,7 @@ def benchmark_generators():
     for det in (False, True):
         p = ChannelwiseTPP(*MACE, irrep_dtype=np.float64, weight_dtype=np.float64)
         gens.append((f"mace/conv_{'det' if det else 'atomic'}/float64", select_conv_generator(p, det)))
+    gens.append(("benzene/conv_det", select_conv_generator(get_workload("benzene_conv_det").problem(), True)))
     for dt in (np.float32, np.float64):
         p = FullyConnectedTPProblem(*DENSE, shared_weights=True, internal_weights=False, irrep_dtype=dt, weight_dtype=dt)
         gens.append((f"dense/uvw/{np.dtype(dt).name}", select_generator(p)))

@@ -331,6 +331,17 @@ def get(name: str) -> Workload:
                         "forward+backward, " + ("deterministic (receiver-sorted)" if det else "unsorted"),
                         "conv", MACE, 300000, "edges/s", "hbm", dt, 12350,
                         {"nodes": 10000, "paths": 17, "deterministic": det}, nodes=10000, deterministic=det, sh_lmax=3)
+    if name in ("benzene_conv_det", "benzene_conv_det_f64"):
+        # the largest problem of the reference's list (test/benchmark.py:44-55, nequip-revmd17-benzene): 68 paths, 312
+        # output words per channel, forward and backward in several launches over groups of output blocks
+        from .benchmark.benchmark_configs import nequip_conv
+        irreps = tuple(s_.replace(" ", "") for s_ in [c for c in nequip_conv if c[3] == "nequip-revmd17-benzene"][0][:3])
+        dt = "f64" if name.endswith("_f64") else "f32"
+        return Workload(name, "NequIP-style fused uvu conv with irreps of either parity up to l = 3 (nequip-revmd17-benzene of "
+                        f"the reference's problem list), 64 channels, 68 paths, 5000 nodes, 150000 edges, fp{dt[1:]}, "
+                        "forward+backward, deterministic (receiver-sorted)",
+                        "conv", irreps, 150000, "edges/s", "hbm", dt, 12353,
+                        {"nodes": 5000, "paths": 68, "deterministic": True}, nodes=5000, deterministic=True, sh_lmax=3)
     if name == "nequip_conv_det_all_parities":
         return Workload(name, "fused uvu conv, 32x0e+32x1o+32x2e (x) SH(lmax 2) -> every triangle-allowed l3<=2 of either "
                         "parity, 15 paths, 5000 nodes, 150000 edges, fp32, forward+backward, deterministic (receiver-sorted)",
@@ -381,5 +392,5 @@ def get(name: str) -> Workload:
 
 ALL = ("readme_uvu", "mace_uvu", "mace_uvu_all_parities", "nequip_conv_atomic", "nequip_conv_det", "nequip_conv_det_all_parities",
        "large_conv_det", "large_conv_atomic", "large_conv_det_all_parities", "mace_conv_det", "mace_conv_atomic",
-       "mace_conv_det_f64", "mace_conv_atomic_f64", "dense_uvw_f32", "dense_uvw_f64", "diffdock_uvw_f32", "diffdock_uvw_f64", "diffdock1_uvw_f32", "diffdock1_uvw_f64",
+       "mace_conv_det_f64", "mace_conv_atomic_f64", "benzene_conv_det", "benzene_conv_det_f64", "dense_uvw_f32", "dense_uvw_f64", "diffdock_uvw_f32", "diffdock_uvw_f64", "diffdock1_uvw_f32", "diffdock1_uvw_f64",
        "tetris_poly1_uvw_f32", "tetris_poly1_uvw_f64", "tetris_poly2_uvw_f32", "tetris_poly2_uvw_f64")
