@@ -178,3 +178,40 @@ def test_backward_split_over_output_block_groups():
     with mace._group(1):
         assert {p.o.idx for p in mace.paths} == set(mace.out_groups[1])
     assert len(mace.paths) == 17                         # restored after the group context
+
+
+def test_forward_split_over_output_block_groups():
+    """The convolution forward keeps a node's output words in registers: beyond 100 (fp32) / 72 (fp64) words per
+    channel it runs as one launch per group of output blocks.  The groups partition the output blocks, stay near
+    the limit, and are cut along the in1 blocks; none of the benchmark configurations is split; fp64 splits the
+    backward into groups of about 24 words."""
+    from openequivariance_amd.benchmark import benchmark_configs as bc
+    from openequivariance_amd.codegen.uvu_det import UVUDetGenerator
+    from openequivariance_amd.codegen.uvu_sorted import UVUSortedGenerator
+    from openequivariance_amd.problem import ChannelwiseTPP
+    want = {"mace-large": (1, 1), "mace-medium": (1, 1), "nequip-lips": (2, 2), "nequip-revmd17-aspirin": (1, 1),
+            "nequip-revmd17-toluene": (2, 2), "nequip-revmd17-benzene": (4, 5), "nequip-water": (1, 1)}
+    for cfg in bc.mace_conv + bc.nequip_conv:
+        for k, dt in enumerate((np.float32, np.float64)):
+            g = UVUDetGenerator(ChannelwiseTPP(*cfg[:3], irrep_dtype=dt, weight_dtype=dt))
+            words = lambda grp: sum(g.out[i].D for i in grp)
+            assert len(g.fwd_groups) == want[cfg[3]][k], (cfg[3], dt)
+            assert sorted(sum(g.fwd_groups, [])) == g.used_out and all(g.fwd_groups)
+            assert max(map(words, g.fwd_groups)) <= 1.1 * g.FWD_SPLIT_WORDS[g.T] or len(g.fwd_groups) == 1
+            fwd, _, _ = g.plan()
+            names = [s["kernel"] for s in fwd if s["kernel"].startswith("forward")]
+            assert names == ["forward"] + [f"forward_g{h}" for h in range(1, len(g.fwd_groups))]
+            steps = [s for s in fwd if s["kernel"].startswith("forward")]
+            assert all({k_: v for k_, v in s.items() if k_ != "kernel"} == {k_: v for k_, v in steps[0].items() if k_ != "kernel"}
+                       for s in steps)
+    for irreps in (workloads.NEQUIP, workloads.LARGE, workloads.MACE, workloads.NEQUIP_ALL, workloads.LARGE_ALL):
+        assert len(UVUDetGenerator(ChannelwiseTPP(*irreps)).fwd_groups) == 1
+    benz = ChannelwiseTPP(*[c for c in bc.nequip_conv if c[3] == "nequip-revmd17-benzene"][0][:3])
+    g = UVUDetGenerator(benz)
+    gathered = lambda groups: sum(sum(g.in1[a].D for a in {p.a.idx for p in g.paths if p.o.idx in grp}) for grp in groups)
+    assert gathered(g.fwd_groups) < 0.5 * gathered(g.dealt_groups(4, lambda grp: sum(g.out[i].D for i in grp)))
+    s = UVUSortedGenerator(benz)
+    assert [st["kernel"] for st in s.plan()[0]][-4:] == ["forward", "forward_g1", "forward_g2", "forward_g3"]
+    assert all(f"void {n}(" in s.render() for n in ("forward", "forward_g1", "forward_g2", "forward_g3"))
+    mace64 = UVUDetGenerator(ChannelwiseTPP(*workloads.MACE, irrep_dtype=np.float64, weight_dtype=np.float64))
+    assert mace64.H == 5 and not mace64.prefetch_backward
