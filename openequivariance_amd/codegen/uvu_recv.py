@@ -42,9 +42,10 @@ class UVURecvGenerator(UVUDetGenerator):
     MIN_TILE_ITERS = 8       # edge-loop iterations of the smallest tile
     MAX_TILES = 16384        # tiles per chunk of the largest launches (the tile then grows with the edge count)
     DX_UNROLL = 4            # spill rows in flight per lane group in pass 2
+    RECV_SPLIT_WORDS = 100   # dZ words per lane above which pass 1 runs in several launches (0: never)
 
     def __init__(self, problem: TPProblem, vector_stores: bool = True, idx_ctype: str = "i64", prefetch=None, staged=None,
-                 backward_perm: bool = False):
+                 backward_perm: bool = False, recv_split=None):
         # pass 1 is one launch: the per-edge dX rows cannot be split over launches of output-block groups.
         # ``backward_perm``: the edge list is in no order; pass 1 walks the receiver-grouped position list and pass
         # 2 the sender-grouped one, both built in the workspace by the grouping kernels (pass 1 staged only).
@@ -79,6 +80,19 @@ class UVURecvGenerator(UVUDetGenerator):
         self.regroup_pairs = bool(self.REGROUP_STAGED and self.staged_edges)
         if self.staged_edges:
             self.waves_hint = 0
+        # Pass 1 in several launches when the dZ row of a receiver is too long to hold beside an edge's operands
+        # (312 words per lane with 68 paths: 512 registers and scratch): the output blocks are grouped so that no
+        # in1 block is read by paths of two groups, hence every launch writes words of the per-edge dX rows that
+        # no other launch writes, and its own rows of dW; dY goes through one partial row per (chunk, launch).
+        self.spill_word, w = {}, 0
+        for i in self.used_in1:
+            for m in range(self.in1[i].D):
+                self.spill_word[(i, m)] = w
+                w += 1
+        self.recv_groups = self._disjoint_groups(self.RECV_SPLIT_WORDS if recv_split is None else recv_split) \
+            if self.staged_edges else [list(self.used_out)]
+        self.HR = len(self.recv_groups)
+        self.dy_slots = self.NCH * self.HR
         if not backward_perm:
             self.dypart_off = "(2 * (node_count + 1) + node_count) * sizeof(i64)"
         self.spill_off = (f"((({self.dypart_off} + {self.dy_slots if self.dy_slots > 1 else 0}ull * nnz * {self.D2} * sizeof(T)) "
@@ -93,9 +107,9 @@ class UVURecvGenerator(UVUDetGenerator):
 
     # ------------------------------------------------------------------ plan
     def backward_steps(self):
-        steps = [dict(kernel="backward", num_threads=64, grid_kind=1, work_per_block=self.MIN_TILE_ITERS * self.R,
-                      num_blocks=self.MAX_TILES, grid_y=self.NCH),
-                 dict(kernel="backward_dx", num_threads=64, grid_kind=3, work_per_block=1, num_blocks=self.LONG, grid_y=self.NCH)]
+        steps = [dict(kernel=name, num_threads=64, grid_kind=1, work_per_block=self.MIN_TILE_ITERS * self.R,
+                      num_blocks=self.MAX_TILES, grid_y=self.NCH) for name, _ in self.backward_kernels()] \
+            + [dict(kernel="backward_dx", num_threads=64, grid_kind=3, work_per_block=1, num_blocks=self.LONG, grid_y=self.NCH)]
         if self.dy_slots > 1:
             steps.append(dict(kernel="backward_dy_reduce", num_threads=256, grid_kind=1,
                               work_per_block=self.dy_rows_per_block))
@@ -116,19 +130,46 @@ class UVURecvGenerator(UVUDetGenerator):
             + self.dy_partial_bytes(nnz)
         return ((((head + 255) & ~255) + self.spill_bytes(nnz) + self.flag_bytes(nnz)) + 255) & ~255
 
+    def _disjoint_groups(self, limit: int):
+        """Groups of output blocks of at most ``limit`` words per channel (where the problem allows) such that no in1
+        block is read by paths of two groups: the connected sets of (output block, in1 block) are packed in the
+        order of their in1 blocks."""
+        held = lambda outs: sum(self.out[i].D for i in outs)
+        if not limit or held(self.used_out) <= limit:
+            return [list(self.used_out)]
+        sets = []                                        # (in1 blocks, output blocks) connected through paths
+        for oi in self.used_out:
+            ins, outs = {p.a.idx for p in self.paths_into(oi)}, {oi}
+            for t in [t for t in sets if t[0] & ins]:
+                sets.remove(t)
+                ins |= t[0]
+                outs |= t[1]
+            sets.append((ins, outs))
+        groups = []
+        for ins, outs in sorted(sets, key=lambda t: min(t[0])):
+            if groups and held(groups[-1]) + held(outs) <= limit:
+                groups[-1] += sorted(outs)
+            else:
+                groups.append(sorted(outs))
+        return [sorted(g_) for g_ in groups]
+
+    def backward_kernels(self):
+        return [("backward" if h == 0 else f"backward_g{h}", h) for h in range(self.HR)]
+
     def backward_kernel_sources(self):
         w = self.waves_hint
         attr = f" __attribute__((amdgpu_waves_per_eu({w}, {w})))" if w else ""
-        return [dict(name="backward", threads=64, attr=attr, body=self._edges_body()),
-                dict(name="backward_dx", threads=64, attr="", body=self._dx_body())]
+        return [dict(name=name, threads=64, attr=attr, body=self._edges_body(h)) for name, h in self.backward_kernels()] \
+            + [dict(name="backward_dx", threads=64, attr="", body=self._dx_body())]
 
     # ---------------------------------------------------------------- pass 1
-    def _edges_body(self) -> str:
+    def _edges_body(self, h: int = 0) -> str:
         E = Emitter()
         R, P, NCH = self.R, self.P, self.NCH
         self.emit_lane_direct(E, lds=False)
         if self.staged_edges:
-            return self._edges_body_staged(E)
+            with self._group(h, self.recv_groups):
+                return self._edges_body_staged(E, h)
         E("// (tile, chunk) of this workgroup: ids are dealt to the 8 XCDs round robin, each XCD gets a contiguous run of items")
         E(f"const u64 tiles = gridDim.x, items = tiles * {NCH};")
         E("const u64 bid = blockIdx.x + (u64)blockIdx.y * gridDim.x;")
@@ -254,7 +295,7 @@ class UVURecvGenerator(UVUDetGenerator):
                                            "bool I0rv = false, I1rv = false, I0ev = false, I1ev = false;")
         return E.text()
 
-    def _edges_body_staged(self, E: Emitter) -> str:
+    def _edges_body_staged(self, E: Emitter, grp: int = 0) -> str:
         """Pass 1 through the LDS stage of the forward (same operands: X records of the sender, path weights, Y):
         the edge loop of emit_staged_loop over the tile's consecutive edges, dZ of the receiver held in registers
         and reloaded when the receiver changes, the edge's dW / dY / dX rows kept in registers and stored at the top
@@ -298,13 +339,15 @@ class UVURecvGenerator(UVUDetGenerator):
             E.level += 1
             E("const i64 r_ = rows[e];")
             E("if (r_ >= 0 && r_ < (i64)node_count) continue;")
-            E(f"if (c == 0) for (int q = 0; q < {self.WN}; ++q) Wg[e * {self.WN} + q] = (T)0;")
+            if grp == 0:
+                E(f"if (c == 0) for (int q = 0; q < {self.WN}; ++q) Wg[e * {self.WN} + q] = (T)0;")
             if self.dy_slots > 1:
-                E(f"{{ T* __restrict__ p_ = (T*)((char*)ws + DYPART_OFF) + ((u64)c * nnz + e) * {self.D2}; "
+                E(f"{{ T* __restrict__ p_ = (T*)((char*)ws + DYPART_OFF) + ((u64)(c * {self.HR} + {grp}) * nnz + e) * {self.D2}; "
                   f"for (int q = 0; q < {self.D2}; ++q) p_[q] = (T)0; }}")
             else:
                 E(f"if (c == 0) for (int q = 0; q < {self.D2}; ++q) Yg[e * {self.D2} + q] = (T)0;")
-            E(f"{{ T* __restrict__ p_ = spill + ((e * {NCH} + c) * {self.NW}) * {P}; for (int q = 0; q < {self.NW * P}; ++q) p_[q] = (T)0; }}")
+            if grp == 0:        # (the whole row: the later launches do not visit these edges either)
+                E(f"{{ T* __restrict__ p_ = spill + ((e * {NCH} + c) * {self.NW}) * {P}; for (int q = 0; q < {self.NW * P}; ++q) p_[q] = (T)0; }}")
             E.level -= 1
             E("}")
             E.level -= 1
@@ -376,7 +419,7 @@ class UVURecvGenerator(UVUDetGenerator):
             writer = "ul == 0" if P < 64 else "lane == 63"
             E(f"if (pev && {writer}) {{")
             if self.dy_slots > 1:
-                E(f"    T* __restrict__ Ygr = (T*)((char*)ws + DYPART_OFF) + ((u64)c * nnz + e) * {self.D2};")
+                E(f"    T* __restrict__ Ygr = (T*)((char*)ws + DYPART_OFF) + ((u64)(c * {self.HR} + {grp}) * nnz + e) * {self.D2};")
             else:
                 E(f"    T* __restrict__ Ygr = Yg + e * {self.D2};")
             for f in range(self.D2):
@@ -384,11 +427,9 @@ class UVURecvGenerator(UVUDetGenerator):
             E("}")
             E("if (pev) {")
             E(f"    T* __restrict__ sp = spill + ((e * {NCH} + c) * {self.NW}) * {P} + ul;")
-            w = 0
             for i in self.used_in1:
                 for m in range(self.in1[i].D):
-                    E(f"    oeq_stnt(sp + {w * P}, pv ? pdx{i}_{m} : (T)0);")
-                    w += 1
+                    E(f"    oeq_stnt(sp + {self.spill_word[(i, m)] * P}, pv ? pdx{i}_{m} : (T)0);")
             E("}")
             E.level -= 1
             E("}")

@@ -214,6 +214,40 @@ def test_conv_forward_one_launch_per_group_of_output_blocks(case, monkeypatch):
         assert blk and not out["Z"][:, blk[0].off:blk[0].off + blk[0].dim].any()
 
 
+@pytest.mark.parametrize("case", ["det", "det_two_chunks", "det_four_lane_groups", "unsorted", "unsorted_invalid_edges"])
+def test_conv_receiver_order_pass_one_per_group_of_output_blocks(case, monkeypatch):
+    """Pass 1 of the receiver-order backward in several launches (forced here: a launch per 4 dZ words): the groups
+    share no in1 block, so each launch writes its own words of the per-edge dX rows and its own rows of dW; dY is
+    summed from one partial row per (chunk, launch)."""
+    from openequivariance_amd.codegen.uvu_recv import UVURecvGenerator
+    monkeypatch.setattr(UVURecvGenerator, "RECV_SPLIT_WORDS", 4)
+    irreps = {"det_two_chunks": ("5x0e+3x1o+70x2e", "1x0e+1x1o+1x2e", "5x0e+3x1o+70x2e+7x3o"),
+              "det_four_lane_groups": ("16x0e+16x1o", "1x0e+1x1o", "16x0e+16x0o+16x1e+16x1o")}.get(case, common.NEQUIP)
+    prob, oprob = common.channelwise(irreps)
+    det = case.startswith("det")
+    g = UVURecvGenerator(prob) if det else UVUSortedGenerator(prob, grouped_backward=True, recv_backward=True)
+    b = g if det else g.bwd
+    assert b.staged_edges and b.HR >= 2 and sorted(sum(b.recv_groups, [])) == b.used_out
+    ins = [{p.a.idx for p in b.paths if p.o.idx in grp} for grp in b.recv_groups]
+    assert all(not (x & y) for k, x in enumerate(ins) for y in ins[k + 1:])
+    nodes, nnz = 9, 70
+    rows, cols = common.random_graph(nodes - 1, nnz, 15, self_loops=True)
+    valid = np.ones(nnz, dtype=bool)
+    if case == "unsorted_invalid_edges":
+        rows, cols, valid = common.with_invalid_edges(rows, cols, nodes, 16)
+    tperm = np.arange(nnz)
+    if det:
+        rows, cols, tperm, _ = otp.coord_graph(rows, cols)
+    X, Y, W, G = common.conv_inputs(prob, nodes, nnz, 17)
+    _, bwd, ws = g.plan()
+    assert [s["kernel"] for s in bwd if s["kernel"].startswith("backward")][:b.HR + 1] == \
+        ["backward"] + [f"backward_g{h}" for h in range(1, b.HR)] + ["backward_dx"]
+    out = emu.run_conv(g, bwd, X, Y, W, rows, cols, G=G, tperm=tperm, ws_bytes=ws(nnz, nodes))
+    ref = common.conv_reference_on_valid_edges(otp, oprob, X, Y, W, G, rows, cols, valid)[1:]
+    for got, want in zip((out["Xg"], out["Yg"], out["Wg"]), ref):
+        assert rel_err(got, want) < TOL
+
+
 @pytest.mark.parametrize("staged", [True, False])
 def test_conv_det_long_edge_lists(staged):
     """Edge lists of about 13 edges per node (6-7 iterations of two sub-lists) reach the steady state of

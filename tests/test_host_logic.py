@@ -215,3 +215,34 @@ def test_forward_split_over_output_block_groups():
     assert all(f"void {n}(" in s.render() for n in ("forward", "forward_g1", "forward_g2", "forward_g3"))
     mace64 = UVUDetGenerator(ChannelwiseTPP(*workloads.MACE, irrep_dtype=np.float64, weight_dtype=np.float64))
     assert mace64.H == 5 and not mace64.prefetch_backward
+
+
+def test_receiver_order_pass_one_groups_share_no_in1_block():
+    """Above 100 dZ words per lane pass 1 of the receiver-order backward runs per group of output blocks; the
+    groups partition the output blocks and no in1 block feeds two of them, so the launches write disjoint words of
+    the per-edge dX rows.  The benchmark configurations stay one launch."""
+    from openequivariance_amd.benchmark import benchmark_configs as bc
+    from openequivariance_amd.codegen.uvu_recv import UVURecvGenerator
+    from openequivariance_amd.problem import ChannelwiseTPP, TPProblem
+    want = {"mace-large": 1, "mace-medium": 1, "nequip-lips": 2, "nequip-revmd17-aspirin": 1, "nequip-revmd17-toluene": 2,
+            "nequip-revmd17-benzene": 4, "nequip-water": 1}
+    for cfg in bc.mace_conv + bc.nequip_conv:
+        g = UVURecvGenerator(ChannelwiseTPP(*cfg[:3]))
+        assert g.HR == want[cfg[3]] and g.dy_slots == g.NCH * g.HR, cfg[3]
+        assert sorted(sum(g.recv_groups, [])) == g.used_out
+        ins = [{p.a.idx for p in g.paths if p.o.idx in grp} for grp in g.recv_groups]
+        assert all(not (x & y) for k, x in enumerate(ins) for y in ins[k + 1:])
+        words = sorted(g.spill_word.values())
+        assert words == list(range(g.NW))
+        names = [s["kernel"] for s in g.plan()[1]]
+        assert names[names.index("backward"):][:g.HR + 1] == [k for k, _ in g.backward_kernels()] + ["backward_dx"]
+        assert ("backward_dy_reduce" in names) == (g.dy_slots > 1)
+    for irreps in (workloads.MACE, workloads.NEQUIP_ALL, workloads.LARGE_ALL):
+        assert UVURecvGenerator(ChannelwiseTPP(*irreps)).HR == 1
+    # every output block reads the one in1 block: nothing to split along
+    ins = [(0, k, k, "uvu", True) for k in range(4)]
+    one = UVURecvGenerator(TPProblem("64x3e", "1x0e+1x2e+1x4e+1x6e", "64x3e+64x3e+64x3e+64x3e", ins, shared_weights=False,
+                                     internal_weights=False), recv_split=8)
+    assert one.HR == 1
+    assert UVURecvGenerator(ChannelwiseTPP(*workloads.NEQUIP), recv_split=4).HR == 3
+    assert UVURecvGenerator(ChannelwiseTPP(*workloads.NEQUIP, irrep_dtype=np.float64, weight_dtype=np.float64), recv_split=4).HR == 1
