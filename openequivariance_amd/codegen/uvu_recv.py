@@ -43,6 +43,11 @@ class UVURecvGenerator(UVUDetGenerator):
     MAX_TILES = 16384        # tiles per chunk of the largest launches (the tile then grows with the edge count)
     DX_UNROLL = 4            # spill rows in flight per lane group in pass 2
     RECV_SPLIT_WORDS = 100   # dZ words per lane above which pass 1 runs in several launches (0: never)
+    # the same for pass 1 with register loads.  fp64 (no stage): unsplit, the dZ row, an edge's operands and its results
+    # need more than 512 registers (17 paths at 128 channels, 5000 nodes / 150 000 edges: 3.90 ms against 2.51 ms in
+    # sender order); a launch per in1 block - 16 / 25 / 30 words held, 127 - 336 registers - takes 2.49 ms, and 30 paths
+    # at 32 / 64 channels 1.00 / 1.73 ms against 1.32 / 1.98 ms
+    RECV_SPLIT_WORDS_REGISTER_LOADS = {"float": 0, "double": 32}
 
     def __init__(self, problem: TPProblem, vector_stores: bool = True, idx_ctype: str = "i64", prefetch=None, staged=None,
                  backward_perm: bool = False, recv_split=None):
@@ -89,9 +94,15 @@ class UVURecvGenerator(UVUDetGenerator):
             for m in range(self.in1[i].D):
                 self.spill_word[(i, m)] = w
                 w += 1
-        self.recv_groups = self._disjoint_groups(self.RECV_SPLIT_WORDS if recv_split is None else recv_split) \
-            if self.staged_edges else [list(self.used_out)]
+        limit = (self.RECV_SPLIT_WORDS if self.staged_edges else self.RECV_SPLIT_WORDS_REGISTER_LOADS[self.T]) \
+            if recv_split is None else recv_split
+        self.recv_groups = self._disjoint_groups(limit)
         self.HR = len(self.recv_groups)
+        # pass 1 with register loads is worth choosing (fp64 only, caller's edge order only): every launch holds few
+        # enough dZ words to leave room for an edge's operands and results
+        self.register_loads_fit = (self.T == "double" and not backward_perm and not self.staged_edges and
+                                   max(sum(self.out[i].D for i in g_) for g_ in self.recv_groups)
+                                   <= self.RECV_SPLIT_WORDS_REGISTER_LOADS["double"])
         self.dy_slots = self.NCH * self.HR
         if not backward_perm:
             self.dypart_off = "(2 * (node_count + 1) + node_count) * sizeof(i64)"
@@ -153,13 +164,19 @@ class UVURecvGenerator(UVUDetGenerator):
                 groups.append(sorted(outs))
         return [sorted(g_) for g_ in groups]
 
+    def group_waves_hint(self) -> int:
+        """``waves_hint`` for a launch of pass 1 (launches over groups are left to their register count)."""
+        return self.waves_hint if self.HR == 1 else 0
+
     def backward_kernels(self):
         return [("backward" if h == 0 else f"backward_g{h}", h) for h in range(self.HR)]
 
     def backward_kernel_sources(self):
-        w = self.waves_hint
-        attr = f" __attribute__((amdgpu_waves_per_eu({w}, {w})))" if w else ""
-        return [dict(name=name, threads=64, attr=attr, body=self._edges_body(h)) for name, h in self.backward_kernels()] \
+        def attr(h):
+            with self._group(h, self.recv_groups):
+                w = self.group_waves_hint()
+            return f" __attribute__((amdgpu_waves_per_eu({w}, {w})))" if w else ""
+        return [dict(name=name, threads=64, attr=attr(h), body=self._edges_body(h)) for name, h in self.backward_kernels()] \
             + [dict(name="backward_dx", threads=64, attr="", body=self._dx_body())]
 
     # ---------------------------------------------------------------- pass 1
@@ -167,9 +184,11 @@ class UVURecvGenerator(UVUDetGenerator):
         E = Emitter()
         R, P, NCH = self.R, self.P, self.NCH
         self.emit_lane_direct(E, lds=False)
-        if self.staged_edges:
-            with self._group(h, self.recv_groups):
-                return self._edges_body_staged(E, h)
+        with self._group(h, self.recv_groups):
+            return self._edges_body_staged(E, h) if self.staged_edges else self._edges_body_registers(E, h)
+
+    def _edges_body_registers(self, E: Emitter, grp: int = 0) -> str:
+        R, P, NCH = self.R, self.P, self.NCH
         E("// (tile, chunk) of this workgroup: ids are dealt to the 8 XCDs round robin, each XCD gets a contiguous run of items")
         E(f"const u64 tiles = gridDim.x, items = tiles * {NCH};")
         E("const u64 bid = blockIdx.x + (u64)blockIdx.y * gridDim.x;")
@@ -274,7 +293,7 @@ class UVURecvGenerator(UVUDetGenerator):
             writer = "ul == 0" if P < 64 else "lane == 63"
             E(f"if (cur_ev && {writer}) {{")
             if self.dy_slots > 1:
-                E(f"    T* __restrict__ Ygr = (T*)((char*)ws + DYPART_OFF) + ((u64)c * nnz + e) * {self.D2};")
+                E(f"    T* __restrict__ Ygr = (T*)((char*)ws + DYPART_OFF) + ((u64)(c * {self.HR} + {grp}) * nnz + e) * {self.D2};")
             else:
                 E(f"    T* __restrict__ Ygr = Yg + e * {self.D2};")
             for f in range(self.D2):
@@ -284,11 +303,9 @@ class UVURecvGenerator(UVUDetGenerator):
             # edge that names no node: the dZ held belongs to another edge then)
             E("if (cur_ev) {")
             E(f"    T* __restrict__ sp = spill + ((e * {NCH} + c) * {self.NW}) * {P} + ul;")
-            w = 0
             for i in self.used_in1:
                 for m in range(self.in1[i].D):
-                    E(f"    oeq_stnt(sp + {w * P}, rv ? dx{i}_{m} : (T)0);")
-                    w += 1
+                    E(f"    oeq_stnt(sp + {self.spill_word[(i, m)] * P}, rv ? dx{i}_{m} : (T)0);")
             E("}")
         self.emit_pingpong_loop(E, names, load_idx, load, compute, prefetch_first=self.prefetch_edges, pre=pre,
                                 index_decl="u64 I0e = 0, I1e = 0, I0n = 0, I1n = 0; i64 I0r = -1, I1r = -1; "

@@ -112,11 +112,13 @@ def select_conv_generator(config: TPProblem, deterministic: bool, vector_stores:
             # (32 channels, outputs of either parity) 0.223 / 0.208 ms, 7.1 (256 channels, either parity) 10.94 /
             # 9.43 ms, 7.9 (the 128-channel MACE problem) 2.14 / 1.71 ms.  Without the stage (fp64, or fewer
             # channels than Y components) pass 1 runs one edge at a time: 16.3 against 10.96 ms at 7.1; those
-            # problems keep the sender order.
+            # problems keep the sender order, except in fp64 where pass 1 can run as one launch per group of
+            # output blocks with few dZ words held (the MACE problem in fp64, 10 000 nodes / 300 000 edges: 5.04
+            # / 4.77 ms; 30 paths at 32 channels 1.32 / 1.00 ms).
             order = "send"
             if config.irreps_out.dim >= RECV_ORDER_MIN_RATIO * config.irreps_in1.dim:
                 g = UVURecvGenerator(config, vector_stores=vector_stores, idx_ctype=idx_ctype)
-                if g.staged_edges:
+                if g.staged_edges or g.register_loads_fit:
                     return g
         if order == "recv":
             return UVURecvGenerator(config, vector_stores=vector_stores, idx_ctype=idx_ctype)

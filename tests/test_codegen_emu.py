@@ -214,31 +214,36 @@ def test_conv_forward_one_launch_per_group_of_output_blocks(case, monkeypatch):
         assert blk and not out["Z"][:, blk[0].off:blk[0].off + blk[0].dim].any()
 
 
-@pytest.mark.parametrize("case", ["det", "det_two_chunks", "det_four_lane_groups", "unsorted", "unsorted_invalid_edges"])
+@pytest.mark.parametrize("case", ["det", "det_two_chunks", "det_four_lane_groups", "unsorted", "unsorted_invalid_edges",
+                                  "det_fp64_register_loads", "det_fp64_two_chunks_invalid_edges"])
 def test_conv_receiver_order_pass_one_per_group_of_output_blocks(case, monkeypatch):
     """Pass 1 of the receiver-order backward in several launches (forced here: a launch per 4 dZ words): the groups
     share no in1 block, so each launch writes its own words of the per-edge dX rows and its own rows of dW; dY is
     summed from one partial row per (chunk, launch)."""
     from openequivariance_amd.codegen.uvu_recv import UVURecvGenerator
     monkeypatch.setattr(UVURecvGenerator, "RECV_SPLIT_WORDS", 4)
+    monkeypatch.setattr(UVURecvGenerator, "RECV_SPLIT_WORDS_REGISTER_LOADS", {"float": 4, "double": 4})
     irreps = {"det_two_chunks": ("5x0e+3x1o+70x2e", "1x0e+1x1o+1x2e", "5x0e+3x1o+70x2e+7x3o"),
+              "det_fp64_two_chunks_invalid_edges": ("5x0e+3x1o+70x2e", "1x0e+1x1o+1x2e", "5x0e+3x1o+70x2e+7x3o"),
               "det_four_lane_groups": ("16x0e+16x1o", "1x0e+1x1o", "16x0e+16x0o+16x1e+16x1o")}.get(case, common.NEQUIP)
-    prob, oprob = common.channelwise(irreps)
+    fp64 = "fp64" in case
+    prob, oprob = common.channelwise(irreps, dtype=np.float64 if fp64 else np.float32)
     det = case.startswith("det")
     g = UVURecvGenerator(prob) if det else UVUSortedGenerator(prob, grouped_backward=True, recv_backward=True)
     b = g if det else g.bwd
-    assert b.staged_edges and b.HR >= 2 and sorted(sum(b.recv_groups, [])) == b.used_out
+    assert b.staged_edges == (not fp64) and b.HR >= 2 and sorted(sum(b.recv_groups, [])) == b.used_out
     ins = [{p.a.idx for p in b.paths if p.o.idx in grp} for grp in b.recv_groups]
     assert all(not (x & y) for k, x in enumerate(ins) for y in ins[k + 1:])
     nodes, nnz = 9, 70
     rows, cols = common.random_graph(nodes - 1, nnz, 15, self_loops=True)
     valid = np.ones(nnz, dtype=bool)
-    if case == "unsorted_invalid_edges":
+    if case.endswith("invalid_edges"):
         rows, cols, valid = common.with_invalid_edges(rows, cols, nodes, 16)
     tperm = np.arange(nnz)
     if det:
         rows, cols, tperm, _ = otp.coord_graph(rows, cols)
-    X, Y, W, G = common.conv_inputs(prob, nodes, nnz, 17)
+    valid = (rows >= 0) & (rows < nodes) & (cols >= 0) & (cols < nodes)
+    X, Y, W, G = common.conv_inputs(prob, nodes, nnz, 17, dtype=np.float64 if fp64 else np.float32)
     _, bwd, ws = g.plan()
     assert [s["kernel"] for s in bwd if s["kernel"].startswith("backward")][:b.HR + 1] == \
         ["backward"] + [f"backward_g{h}" for h in range(1, b.HR)] + ["backward_dx"]

@@ -87,7 +87,8 @@ def test_deterministic_backward_order_is_chosen_by_shape(cuda):
     """Static rule: the two-pass receiver-order backward when a dZ row is at least 5.5 times as long as an X row
     and pass 1 can stage its operands through LDS (fp32, at least as many channels per row group as Y
     components): the MACE problem (7.9) and configs 3 and 5 with outputs of either parity (5.7, 7.1) take it,
-    configs 3 and 5 themselves (3.9, 4.8) and fp64 problems keep the sender order."""
+    configs 3 and 5 themselves (3.9, 4.8) keep the sender order.  fp64 has no stage: the receiver order is taken where
+    pass 1 can run as one launch per in1 block with at most 32 dZ words held (the MACE problem), not otherwise."""
     from openequivariance_amd import workloads
     from openequivariance_amd.codegen.uvu_recv import UVURecvGenerator
     from openequivariance_amd.conv import select_conv_generator
@@ -96,9 +97,14 @@ def test_deterministic_backward_order_is_chosen_by_shape(cuda):
         assert isinstance(g, UVURecvGenerator) and g.staged_edges and g.regroup_pairs
     for irreps in (common.NEQUIP, common.LARGE):
         assert not isinstance(select_conv_generator(common.channelwise(irreps)[0], True), UVURecvGenerator)
-    assert not isinstance(select_conv_generator(common.channelwise(common.MACE, dtype=np.float64)[0], True), UVURecvGenerator)
+    g = select_conv_generator(common.channelwise(common.MACE, dtype=np.float64)[0], True)
+    assert isinstance(g, UVURecvGenerator) and not g.staged_edges and g.HR == 3
+    for irreps in (common.NEQUIP, workloads.MACE_ALL):
+        assert not isinstance(select_conv_generator(common.channelwise(irreps, dtype=np.float64)[0], True), UVURecvGenerator)
     prob, oprob = common.channelwise(common.MACE)
     _run(prob, oprob, 60, 900, 40, True, sh_lmax=3)
+    prob, oprob = common.channelwise(common.MACE, dtype=np.float64)
+    _run(prob, oprob, 60, 900, 41, True, dtype=np.float64, sh_lmax=3)
 
 
 def test_unsorted_mace_conv_backward_in_receiver_order(cuda, monkeypatch):
@@ -205,7 +211,8 @@ def test_conv_fp64(cuda):
 def test_conv_forward_in_groups_of_output_blocks(cuda, which, deterministic, dtype):
     """The reference's NequIP convolution problems with 30 and 68 paths (outputs of either parity up to l = 2 and
     3: 102 and 312 output words per channel): the forward runs one launch per group of output blocks, the backward
-    (sender order in fp64) likewise; a hub node makes one edge list long enough to be walked in pieces."""
+    likewise (fp32: receiver order, pass 1 per group of blocks sharing no in1 block; fp64: the same with register loads
+    for the 30-path problem, sender order for the 68-path one); a hub node makes one edge list long enough to be walked in pieces."""
     from openequivariance_amd.benchmark import benchmark_configs as bc
     irreps = [c[:3] for c in bc.nequip_conv if c[3] == which][0]
     prob, oprob = common.channelwise(irreps, dtype=dtype)

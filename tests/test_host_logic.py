@@ -245,4 +245,14 @@ def test_receiver_order_pass_one_groups_share_no_in1_block():
                                      internal_weights=False), recv_split=8)
     assert one.HR == 1
     assert UVURecvGenerator(ChannelwiseTPP(*workloads.NEQUIP), recv_split=4).HR == 3
-    assert UVURecvGenerator(ChannelwiseTPP(*workloads.NEQUIP, irrep_dtype=np.float64, weight_dtype=np.float64), recv_split=4).HR == 1
+    # fp64 has no LDS stage: pass 1 with register loads, a launch per in1 block, chosen where every launch holds at
+    # most 32 dZ words
+    from openequivariance_amd.conv import select_conv_generator
+    f64 = lambda irreps: ChannelwiseTPP(*irreps, irrep_dtype=np.float64, weight_dtype=np.float64)
+    mace64 = select_conv_generator(f64(workloads.MACE), True)
+    assert isinstance(mace64, UVURecvGenerator) and not mace64.staged_edges and mace64.register_loads_fit
+    assert [sum(mace64.out[i].D for i in grp) for grp in mace64.recv_groups] == [16, 24, 31]
+    for irreps in (workloads.NEQUIP, workloads.LARGE, workloads.MACE_ALL):
+        assert not isinstance(select_conv_generator(f64(irreps), True), UVURecvGenerator)
+    assert not UVURecvGenerator(f64(workloads.MACE_ALL)).register_loads_fit
+    assert not UVURecvGenerator(f64(workloads.MACE), backward_perm=True).register_loads_fit
