@@ -324,7 +324,8 @@ static int conv_forward(oeq_conv* c, const void* L1, const void* L2, const void*
     if (c->fwd.empty()) return fail("this operator was built without a forward plan");
     if (nnz > 0 && node_count == 0) return fail("convolution called with %llu edges but no nodes", (unsigned long long)nnz);
     if (nnz > 0 && (!rows || !cols)) return fail("forward: rows / cols are NULL");
-    if ((nnz > 0 || node_count > 0) && check_pointers(c->fwd, workspace, tperm, "forward")) return 1;
+    // (an empty edge list has no transpose permutation to read: a NULL pointer is what an empty tensor gives)
+    if ((nnz > 0 || node_count > 0) && check_pointers(c->fwd, workspace, nnz > 0 ? tperm : (const void*)1, "forward")) return 1;
     if (call_flags & ~(uint32_t)(OEQ_CALL_PREPARED | OEQ_CALL_COUNTERS_ZERO)) return fail("forward: unknown call flags 0x%x", call_flags);
     void* args[] = {&L1, &L2, &W, &L3, &rows, &cols, &nnz, &node_count, &workspace, &tperm};
     for (auto& s : c->fwd) {
@@ -341,7 +342,8 @@ static int conv_backward(oeq_conv* c, const void* L1, void* L1g, const void* L2,
     if (c->bwd.empty()) return fail("this operator was built without a backward plan");
     if (nnz > 0 && node_count == 0) return fail("convolution called with %llu edges but no nodes", (unsigned long long)nnz);
     if (nnz > 0 && (!rows || !cols)) return fail("backward: rows / cols are NULL");
-    if ((nnz > 0 || node_count > 0) && check_pointers(c->bwd, workspace, tperm, "backward")) return 1;
+    // (an empty edge list has no transpose permutation to read: a NULL pointer is what an empty tensor gives)
+    if ((nnz > 0 || node_count > 0) && check_pointers(c->bwd, workspace, nnz > 0 ? tperm : (const void*)1, "backward")) return 1;
     if (call_flags & ~(uint32_t)(OEQ_CALL_PREPARED | OEQ_CALL_COUNTERS_ZERO)) return fail("backward: unknown call flags 0x%x", call_flags);
     void* args[] = {&L1, &L1g, &L2, &L2g, &W, &Wg, &L3g, &rows, &cols, &nnz, &node_count, &workspace, &tperm};
     for (auto& s : c->bwd) {

@@ -52,7 +52,7 @@ def forward(prob: Problem, X, Y, W):
             out = np.einsum("zuv,ijk,zui,zvj->zuk", w, C, x, y, optimize=True)
         else:
             out = np.einsum("zuvw,ijk,zui,zvj->zwk", w, C, x, y, optimize=True)
-        Z[:, o3:o3 + mo * (2 * l3 + 1)] += p["coeff"] * out.reshape(B, -1)
+        Z[:, o3:o3 + mo * (2 * l3 + 1)] += p["coeff"] * out.reshape(B, mo * (2 * l3 + 1))
     return Z
 
 
@@ -78,13 +78,13 @@ def backward(prob: Problem, X, Y, W, G):
             dx = np.einsum("zuvw,ijk,zvj,zwk->zui", w, C, y, g, optimize=True)
             dy = np.einsum("zuvw,ijk,zui,zwk->zvj", w, C, x, g, optimize=True)
             dw = np.einsum("ijk,zui,zvj,zwk->zuvw", C, x, y, g, optimize=True)
-        dX[:, o1:o1 + m1 * (2 * l1 + 1)] += dx.reshape(B, -1)
-        dY[:, o2:o2 + m2 * (2 * l2 + 1)] += dy.reshape(B, -1)
+        dX[:, o1:o1 + m1 * (2 * l1 + 1)] += dx.reshape(B, m1 * (2 * l1 + 1))
+        dY[:, o2:o2 + m2 * (2 * l2 + 1)] += dy.reshape(B, m2 * (2 * l2 + 1))
         sl = slice(p["woff"], p["woff"] + prod(p["shape"]))
         if shared:
             dW[sl] += dw.sum(axis=0).reshape(-1)
         else:
-            dW[:, sl] += dw.reshape(B, -1)
+            dW[:, sl] += dw.reshape(B, sl.stop - sl.start)
     return dX, dY, dW
 
 

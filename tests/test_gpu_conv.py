@@ -294,6 +294,12 @@ def test_no_edges(cuda):
             args.append(e)
         z = conv.forward(*args)
         assert z.shape == (7, 1120) and float(z.abs().max()) == 0.0
+        # the backward of an empty edge list: dX = 0, empty dY and dW (an empty transpose permutation is a NULL pointer)
+        x, y, w = (a.clone().requires_grad_(True) for a in args[:3])
+        conv.forward(x, y, w, *args[3:]).backward(torch.randn(7, 1120, device=cuda))
+        torch.cuda.synchronize()
+        assert x.grad.shape == (7, 288) and float(x.grad.abs().max()) == 0.0
+        assert y.grad.shape == (0, 9) and w.grad.shape == (0, 352)
 
 
 def test_deterministic_bit_reproducible(cuda):
