@@ -71,7 +71,8 @@ enum { OEQ_GRID_FIXED = 0, OEQ_GRID_PER_ROW = 1, OEQ_GRID_PER_NODE = 2, OEQ_GRID
 #define OEQ_PIECE_MIN_EDGES 32u
 /* What a step dereferences and what it is for.  A call whose plan holds a step with
  * OEQ_STEP_NEEDS_WORKSPACE (OEQ_STEP_NEEDS_TPERM) is rejected, before anything is launched, when the
- * workspace (transpose permutation) pointer is NULL.  OEQ_STEP_GRAPH_PREP marks the steps that only
+ * workspace (transpose permutation) pointer is NULL; a call with nnz == 0 has no transpose permutation
+ * to read and may pass NULL for it.  OEQ_STEP_GRAPH_PREP marks the steps that only
  * derive graph structure (CSR pointers, position lists, node order) from rows / cols /
  * transpose_perm into the workspace: a call with OEQ_CALL_PREPARED skips them.  OEQ_STEP_COUNTER_CLEAR
  * marks a step that only zeroes counters in the workspace which the operator's later steps leave
