@@ -731,10 +731,11 @@ def measure(name, steps, warmup, cold=True, cpu=True, cpu_sample=0, ceiling=True
     return wl, rec
 
 
-# every benchmark configuration besides the headline one (config 2 = mace_uvu), the MACE problem as a convolution, and
-# one problem of each of the other two uvw kernel families (per-row weights, few shared weights)
+# every benchmark configuration besides the headline one (config 2 = mace_uvu), the MACE problem as a convolution in both
+# precisions, and one problem of each of the other two uvw kernel families (per-row weights, few shared weights)
 OTHER_WORKLOADS = ("readme_uvu", "nequip_conv_det", "nequip_conv_atomic", "dense_uvw_f32", "dense_uvw_f64",
-                   "large_conv_det", "large_conv_atomic", "mace_conv_det", "mace_conv_det_f64", "diffdock_uvw_f32", "tetris_poly1_uvw_f32")
+                   "large_conv_det", "large_conv_atomic", "mace_conv_det", "mace_conv_det_f64", "diffdock_uvw_f32",
+                   "tetris_poly1_uvw_f32")
 
 
 def main():
