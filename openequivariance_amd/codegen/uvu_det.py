@@ -40,7 +40,7 @@ class UVUDetGenerator(UVUDirectGenerator):
     # words per group when the backward is split (fp64, 5000 nodes / 150 000 edges, 64 -> 24 words per group: 17 paths
     # at 128 channels 3.12 -> 2.52 ms, 68 paths 9.38 -> 7.56 ms, 30 paths 2.11 -> 1.98 and 1.27 -> 1.33 ms)
     SPLIT_TARGET = {"float": 64, "double": 24}
-    FWD_SPLIT_WORDS = {"float": 100, "double": 72}
+    FWD_SPLIT_WORDS = {"float": 100, "double": 32}
     FWD_COHERENT = True
     # int64 words of one on-the-fly grouping of the edges in the workspace: group pointers and fill cursors
     # (node_count + 1 each), the position list (nnz), the counters (node_count + 1) and the ticket of the
@@ -152,6 +152,10 @@ class UVUDetGenerator(UVUDirectGenerator):
         # words 0.68 / 3.33 ms, 68 paths and 312 words 19.6 / 44.6 ms), so the output blocks are dealt into groups, one
         # forward launch per group: each launch reads X, Y and its own weights and writes its blocks of Z (the same
         # problems then 0.35 / 0.75 and 1.14 / 2.71 ms; 71 words in one launch: 0.38 / 0.95 ms, in two 0.41 / 0.99).
+        # With the groups cut along the in1 blocks (coherent_groups) a launch gathers only its own X blocks and finer
+        # groups pay in fp64, where one launch needs 366 registers: 71 words in groups of at most 32, 0.94 -> 0.88 ms; 102
+        # words 0.51 -> 0.42 ms; 312 words 2.29 -> 2.02 ms; 256 channels with outputs of either parity 1.84 -> 1.45 ms
+        # (fp32, groups of 64 instead of 100: 71 words 0.375 -> 0.388 ms, 312 words 1.04 -> 0.95 ms).
         z_regs = lambda outs: sum(self.out[i].D for i in outs)
         HF = 1
         fsplit = self.FWD_SPLIT_WORDS[self.T] if fwd_split is None else fwd_split
