@@ -33,12 +33,25 @@ def _channelwise(rng, muls):
 # them, unsorted - with 16 to 64 lanes per row and one or two chunks, and draws that stage a multi-chunk forward)
 @pytest.mark.parametrize("seed", list(range(3000, 3024)) + [4002, 4011, 4014, 4029, 4088, 4095, 4114, 4145, 4149, 4188])
 def test_random_convolution(cuda, seed):
+    _random_convolution(cuda, seed, np.float32)
+
+
+# (fp64 has kernels of its own choice: no LDS stage, the receiver order with register loads in one launch per in1
+# block, forward groups of 32 output words)
+# (5001 - 5045: draws that take the receiver order; the others keep the sender order)
+@pytest.mark.parametrize("seed", [5000, 5001, 5003, 5004, 5011, 5017, 5030, 5039, 5040, 5045])
+def test_random_convolution_fp64(cuda, seed):
+    _random_convolution(cuda, seed, np.float64)
+
+
+def _random_convolution(cuda, seed, dtype):
     import torch
     import openequivariance_amd as oeq
     rng = np.random.default_rng(seed)
+    tol = FP32_TOL if dtype == np.float32 else FP64_TOL
     while True:                                   # drawn again until at least one path is allowed
         irreps = _channelwise(rng, [1, 3, 8, 16, 20, 32, 48, 64, 100, 128])
-        prob, oprob = common.channelwise(irreps)
+        prob, oprob = common.channelwise(irreps, dtype=dtype)
         if prob.instructions:
             break
     nodes, nnz = int(rng.integers(1, 80)), int(rng.integers(0, 2000))
@@ -47,17 +60,18 @@ def test_random_convolution(cuda, seed):
         tperm = None
         if deterministic:
             rows, cols, tperm, _ = otp.coord_graph(rows, cols)
-        X, Y, W, G = common.conv_inputs(prob, nodes, nnz, seed)
-        print(f"seed={seed} {irreps} paths={len(prob.instructions)} nodes={nodes} nnz={nnz} det={deterministic}", flush=True)
+        X, Y, W, G = common.conv_inputs(prob, nodes, nnz, seed, dtype)
         conv = oeq.TensorProductConv(prob, torch_op=True, deterministic=deterministic)
+        print(f"seed={seed} {np.dtype(dtype).name} {irreps} paths={len(prob.instructions)} nodes={nodes} nnz={nnz} "
+              f"det={deterministic} {type(conv.generator).__name__}", flush=True)
         x, y, w = (torch.tensor(a, device=cuda, requires_grad=True) for a in (X, Y, W))
         idx = [torch.tensor(a, device=cuda) for a in ((rows, cols, tperm) if deterministic else (rows, cols))]
         z = conv.forward(x, y, w, *idx)
         z.backward(torch.tensor(G, device=cuda))
         torch.cuda.synchronize()
-        assert rel_err(z.detach().cpu().numpy(), otp.conv_forward(oprob, X, Y, W, rows, cols)) <= FP32_TOL
+        assert rel_err(z.detach().cpu().numpy(), otp.conv_forward(oprob, X, Y, W, rows, cols)) <= tol
         for got, ref in zip((x.grad, y.grad, w.grad), otp.conv_backward(oprob, X, Y, W, G, rows, cols)):
-            assert rel_err(got.cpu().numpy(), ref) <= FP32_TOL
+            assert rel_err(got.cpu().numpy(), ref) <= tol
 
 
 @pytest.mark.parametrize("seed", range(4000, 4030))
