@@ -53,7 +53,7 @@ class UVURecvGenerator(UVUDetGenerator):
                  backward_perm: bool = False, recv_split=None):
         # pass 1 is one launch: the per-edge dX rows cannot be split over launches of output-block groups.
         # ``backward_perm``: the edge list is in no order; pass 1 walks the receiver-grouped position list and pass
-        # 2 the sender-grouped one, both built in the workspace by the grouping kernels (pass 1 staged only).
+        # 2 the sender-grouped one, both built in the workspace by the grouping kernels.
         super().__init__(problem, vector_stores=vector_stores, idx_ctype=idx_ctype, allow_split=False,
                          backward_perm=backward_perm)
         assert self.H == 1
@@ -98,9 +98,9 @@ class UVURecvGenerator(UVUDetGenerator):
             if recv_split is None else recv_split
         self.recv_groups = self._disjoint_groups(limit)
         self.HR = len(self.recv_groups)
-        # pass 1 with register loads is worth choosing (fp64 only, caller's edge order only): every launch holds few
+        # pass 1 with register loads is worth choosing (fp64 only): every launch holds few
         # enough dZ words to leave room for an edge's operands and results
-        self.register_loads_fit = (self.T == "double" and not backward_perm and not self.staged_edges and
+        self.register_loads_fit = (self.T == "double" and not self.staged_edges and
                                    max(sum(self.out[i].D for i in g_) for g_ in self.recv_groups)
                                    <= self.RECV_SPLIT_WORDS_REGISTER_LOADS["double"])
         self.dy_slots = self.NCH * self.HR
@@ -189,24 +189,13 @@ class UVURecvGenerator(UVUDetGenerator):
 
     def _edges_body_registers(self, E: Emitter, grp: int = 0) -> str:
         R, P, NCH = self.R, self.P, self.NCH
-        E("// (tile, chunk) of this workgroup: ids are dealt to the 8 XCDs round robin, each XCD gets a contiguous run of items")
-        E(f"const u64 tiles = gridDim.x, items = tiles * {NCH};")
-        E("const u64 bid = blockIdx.x + (u64)blockIdx.y * gridDim.x;")
-        E("const u64 xcd = bid & 7, turn = bid >> 3;")
-        E("const u64 item = xcd * (items >> 3) + min(xcd, items & 7) + turn;")
-        E(f"const int c = (int)(item % {NCH}); (void)c;")
-        E(f"const u64 tile = item / {NCH};")
-        E(f"const int u = c * {P} + ul;")
-        E(f"const u64 per = ((nnz + tiles - 1) / tiles + {R - 1}) / {R} * {R};       // edges per tile")
-        E("const u64 beg = min(tile * per, nnz);")
-        E("const int len = (int)(min(beg + per, nnz) - beg);")
-        E(f"const int maxlen = (len + {R - 1}) / {R};")
-        E(f"T* __restrict__ spill = (T*)((char*)ws + {self.spill_off});")
-        self._cur_c = "e"
+        self._emit_tile_header(E, grp)
         E("bool rv = false;")
         for oi in self.used_out:
             E("T " + ", ".join(f"G{oi}_{k} = (T)0" for k in range(self.out[oi].D)) + ";")
         E("i64 cur_rcv = -1;")
+        if self.backward_perm:
+            E("const i64* __restrict__ rlist = (const i64*)ws + 2 * (node_count + 1);     // edge ids grouped by receiver")
         names = []
         for i in self.used_in1:
             names += [f"x{i}_{m}" for m in range(self.in1[i].D)]
@@ -216,8 +205,15 @@ class UVURecvGenerator(UVUDetGenerator):
         def load_idx(E, it, q):
             E("{")
             E.level += 1
-            E(f"const bool ev = {self.edge_pos(it)} < len;")
-            E(f"const u64 e = ev ? beg + (u64){self.edge_pos(it)} : nnz - 1;      // idle lane groups re-read the last edge, masked below")
+            if self.backward_perm:
+                # the tile's positions of the receiver-grouped list name the edges
+                E(f"const bool lv = {self.edge_pos(it)} < len;")
+                E(f"const i64 e0 = rlist[lv ? beg + (u64){self.edge_pos(it)} : beg];")
+                E("const bool ev = lv && e0 >= 0 && e0 < (i64)nnz;")
+                E("const u64 e = ev ? (u64)e0 : nnz - 1;")
+            else:
+                E(f"const bool ev = {self.edge_pos(it)} < len;")
+                E(f"const u64 e = ev ? beg + (u64){self.edge_pos(it)} : nnz - 1;      // idle lane groups re-read the last edge, masked below")
             E("const i64 snd = cols[e], rcv = rows[e];")
             E("const bool ok = ev && snd >= 0 && snd < (i64)node_count && rcv >= 0 && rcv < (i64)node_count;")
             E(f"I{q}e = e; I{q}ev = ev; I{q}rv = ok; I{q}n = ok ? (u64)snd : 0; I{q}r = ok ? rcv : -1;")
@@ -312,13 +308,10 @@ class UVURecvGenerator(UVUDetGenerator):
                                            "bool I0rv = false, I1rv = false, I0ev = false, I1ev = false;")
         return E.text()
 
-    def _edges_body_staged(self, E: Emitter, grp: int = 0) -> str:
-        """Pass 1 through the LDS stage of the forward (same operands: X records of the sender, path weights, Y):
-        the edge loop of emit_staged_loop over the tile's consecutive edges, dZ of the receiver held in registers
-        and reloaded when the receiver changes, the edge's dW / dY / dX rows kept in registers and stored at the top
-        of the next iteration."""
+    def _emit_tile_header(self, E: Emitter, grp: int) -> None:
+        """(tile, chunk) of the workgroup, the tile's range of list positions, and - over a position list built on
+        the fly - the zero rows of the edges that are in no group."""
         R, P, NCH = self.R, self.P, self.NCH
-        nt = 2 if self.nontemporal else 0
         E("// (tile, chunk) of this workgroup: ids are dealt to the 8 XCDs round robin, each XCD gets a contiguous run of items")
         E(f"const u64 tiles = gridDim.x, items = tiles * {NCH};")
         E("const u64 bid = blockIdx.x + (u64)blockIdx.y * gridDim.x;")
@@ -371,6 +364,15 @@ class UVURecvGenerator(UVUDetGenerator):
             E("}")
             E.level -= 1
             E("}")
+
+    def _edges_body_staged(self, E: Emitter, grp: int = 0) -> str:
+        """Pass 1 through the LDS stage of the forward (same operands: X records of the sender, path weights, Y):
+        the edge loop of emit_staged_loop over the tile's consecutive edges, dZ of the receiver held in registers
+        and reloaded when the receiver changes, the edge's dW / dY / dX rows kept in registers and stored at the top
+        of the next iteration."""
+        R, P, NCH = self.R, self.P, self.NCH
+        nt = 2 if self.nontemporal else 0
+        self._emit_tile_header(E, grp)
         E("bool rv = false;")
         for oi in self.used_out:
             E("T " + ", ".join(f"G{oi}_{k} = (T)0" for k in range(self.out[oi].D)) + ";")

@@ -61,8 +61,11 @@ class UVUSortedGenerator:
             if recv_backward is not False and (recv_backward or self.fwd.D3 >= self.RECV_ORDER_MIN_RATIO * self.fwd.D1):
                 # long dZ rows: the two-pass backward in receiver order (pass 1 over the receiver grouping, which the
                 # backward then builds as well; pass 2 over the sender grouping), where pass 1 can stage its operands
+                # (fp32).  In fp64 pass 1 with register loads, one launch per in1 block, runs over the position list as
+                # well, but the second counting sort costs what it gains: the MACE problem, 10 000 nodes / 300 000 edges,
+                # backward 5.16 ms in sender order, 5.32 ms in receiver order; it is taken on request only
                 recv = UVURecvGenerator(problem, vector_stores=vector_stores, idx_ctype=idx_ctype, backward_perm=True)
-                if recv.staged_edges:
+                if recv_backward is True or recv.staged_edges:
                     self.bwd, self.recv_backward = recv, True
         else:
             self.bwd = UVUDirectGenerator(problem, "conv_atomic", vector_stores=vector_stores)

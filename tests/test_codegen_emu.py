@@ -215,7 +215,8 @@ def test_conv_forward_one_launch_per_group_of_output_blocks(case, monkeypatch):
 
 
 @pytest.mark.parametrize("case", ["det", "det_two_chunks", "det_four_lane_groups", "unsorted", "unsorted_invalid_edges",
-                                  "det_fp64_register_loads", "det_fp64_two_chunks_invalid_edges"])
+                                  "det_fp64_register_loads", "det_fp64_two_chunks_invalid_edges", "unsorted_fp64",
+                                  "unsorted_fp64_invalid_edges"])
 def test_conv_receiver_order_pass_one_per_group_of_output_blocks(case, monkeypatch):
     """Pass 1 of the receiver-order backward in several launches (forced here: a launch per 4 dZ words): the groups
     share no in1 block, so each launch writes its own words of the per-edge dX rows and its own rows of dW; dY is

@@ -120,6 +120,28 @@ def test_unsorted_mace_conv_backward_in_receiver_order(cuda, monkeypatch):
     assert not conv.generator.recv_backward
 
 
+def test_unsorted_fp64_conv_backward_in_receiver_order_on_request(cuda, monkeypatch):
+    """fp64 over an unsorted edge list keeps the sender order by default; the receiver order with register loads (one
+    launch of pass 1 per in1 block, over the receiver-grouped position list) runs when the generator is asked for it."""
+    import openequivariance_amd.conv as conv_mod
+    from openequivariance_amd import tunables
+    from openequivariance_amd.codegen.uvu_sorted import UVUSortedGenerator
+    monkeypatch.setattr(tunables.current, "autotune", False)
+    prob, oprob = common.channelwise(common.MACE, dtype=np.float64)
+    conv, _ = _run(prob, oprob, 60, 900, 44, False, dtype=np.float64, sh_lmax=3)
+    assert not conv.generator.recv_backward
+
+    def pick(config, deterministic, vector_stores=True, idx_dtype=np.int64):
+        assert not deterministic
+        return UVUSortedGenerator(config, vector_stores=vector_stores, grouped_backward=True, recv_backward=True,
+                                  idx_ctype="i64" if np.dtype(idx_dtype) == np.dtype(np.int64) else "int")
+    monkeypatch.setattr(conv_mod, "select_conv_generator", pick)
+    rows, cols = common.hub_graph(59, 900, 45, hub_in=3, hub_out=5, in_edges=300, out_edges=200)
+    conv, _ = _run(prob, oprob, 60, 900, 45, False, dtype=np.float64, sh_lmax=3, graph=(rows, cols, None))
+    b = conv.generator.bwd
+    assert conv.generator.recv_backward and not b.staged_edges and b.HR == 3
+
+
 @pytest.mark.parametrize("deterministic", [False, True])
 def test_mace_conv_backward_split_over_output_blocks(cuda, deterministic, monkeypatch):
     """The MACE problem as a convolution in sender order: 104 registers of operands per edge, so the backward

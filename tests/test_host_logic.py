@@ -255,4 +255,9 @@ def test_receiver_order_pass_one_groups_share_no_in1_block():
     for irreps in (workloads.NEQUIP, workloads.LARGE, workloads.MACE_ALL):
         assert not isinstance(select_conv_generator(f64(irreps), True), UVURecvGenerator)
     assert not UVURecvGenerator(f64(workloads.MACE_ALL)).register_loads_fit
-    assert not UVURecvGenerator(f64(workloads.MACE), backward_perm=True).register_loads_fit
+    # the operator over unsorted edge lists can run it as well (pass 1 then walks the receiver-grouped position list),
+    # on request only: the second counting sort costs what the order gains
+    from openequivariance_amd.codegen.uvu_sorted import UVUSortedGenerator
+    assert not UVUSortedGenerator(f64(workloads.MACE)).recv_backward
+    s64 = UVUSortedGenerator(f64(workloads.MACE), grouped_backward=True, recv_backward=True)
+    assert s64.recv_backward and s64.bwd.register_loads_fit and s64.bwd.HR == 3 and not s64.bwd.staged_edges
