@@ -42,7 +42,11 @@ class UVURecvGenerator(UVUDetGenerator):
     MIN_TILE_ITERS = 8       # edge-loop iterations of the smallest tile
     MAX_TILES = 16384        # tiles per chunk of the largest launches (the tile then grows with the edge count)
     DX_UNROLL = 4            # spill rows in flight per lane group in pass 2
-    RECV_SPLIT_WORDS = 100   # dZ words per lane above which pass 1 runs in several launches (0: never)
+    # dZ words per lane above which pass 1 runs in several launches (0: never); with one row group per wavefront
+    # RECV_SPLIT_WORDS_ONE_GROUP (30 paths, 102 words, 5000 nodes / 150 000 edges: at 32 channels - two row groups - 0.488
+    # ms in one launch, 0.421 ms in two; at 64 channels 0.781 and 0.804 ms)
+    RECV_SPLIT_WORDS = 100
+    RECV_SPLIT_WORDS_ONE_GROUP = 128
     # the same for pass 1 with register loads.  fp64 (no stage): unsplit, the dZ row, an edge's operands and its results
     # need more than 512 registers (17 paths at 128 channels, 5000 nodes / 150 000 edges: 3.90 ms against 2.51 ms in
     # sender order); a launch per in1 block - 16 / 25 / 30 words held, 127 - 336 registers - takes 2.49 ms, and 30 paths
@@ -94,7 +98,8 @@ class UVURecvGenerator(UVUDetGenerator):
             for m in range(self.in1[i].D):
                 self.spill_word[(i, m)] = w
                 w += 1
-        limit = (self.RECV_SPLIT_WORDS if self.staged_edges else self.RECV_SPLIT_WORDS_REGISTER_LOADS[self.T]) \
+        limit = ((self.RECV_SPLIT_WORDS if self.R > 1 else self.RECV_SPLIT_WORDS_ONE_GROUP) if self.staged_edges
+                 else self.RECV_SPLIT_WORDS_REGISTER_LOADS[self.T]) \
             if recv_split is None else recv_split
         self.recv_groups = self._disjoint_groups(limit)
         self.HR = len(self.recv_groups)

@@ -223,6 +223,7 @@ def test_conv_receiver_order_pass_one_per_group_of_output_blocks(case, monkeypat
     summed from one partial row per (chunk, launch)."""
     from openequivariance_amd.codegen.uvu_recv import UVURecvGenerator
     monkeypatch.setattr(UVURecvGenerator, "RECV_SPLIT_WORDS", 4)
+    monkeypatch.setattr(UVURecvGenerator, "RECV_SPLIT_WORDS_ONE_GROUP", 4)
     monkeypatch.setattr(UVURecvGenerator, "RECV_SPLIT_WORDS_REGISTER_LOADS", {"float": 4, "double": 4})
     irreps = {"det_two_chunks": ("5x0e+3x1o+70x2e", "1x0e+1x1o+1x2e", "5x0e+3x1o+70x2e+7x3o"),
               "det_fp64_two_chunks_invalid_edges": ("5x0e+3x1o+70x2e", "1x0e+1x1o+1x2e", "5x0e+3x1o+70x2e+7x3o"),

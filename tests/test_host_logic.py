@@ -218,14 +218,15 @@ def test_forward_split_over_output_block_groups():
 
 
 def test_receiver_order_pass_one_groups_share_no_in1_block():
-    """Above 100 dZ words per lane pass 1 of the receiver-order backward runs per group of output blocks; the
+    """Above 100 dZ words per lane (128 with 64 channels per wavefront) pass 1 of the receiver-order backward runs per
+    group of output blocks; the
     groups partition the output blocks and no in1 block feeds two of them, so the launches write disjoint words of
     the per-edge dX rows.  The benchmark configurations stay one launch."""
     from openequivariance_amd.benchmark import benchmark_configs as bc
     from openequivariance_amd.codegen.uvu_recv import UVURecvGenerator
     from openequivariance_amd.problem import ChannelwiseTPP, TPProblem
-    want = {"mace-large": 1, "mace-medium": 1, "nequip-lips": 2, "nequip-revmd17-aspirin": 1, "nequip-revmd17-toluene": 2,
-            "nequip-revmd17-benzene": 4, "nequip-water": 1}
+    want = {"mace-large": 1, "mace-medium": 1, "nequip-lips": 2, "nequip-revmd17-aspirin": 1, "nequip-revmd17-toluene": 1,
+            "nequip-revmd17-benzene": 3, "nequip-water": 1}
     for cfg in bc.mace_conv + bc.nequip_conv:
         g = UVURecvGenerator(ChannelwiseTPP(*cfg[:3]))
         assert g.HR == want[cfg[3]] and g.dy_slots == g.NCH * g.HR, cfg[3]
